@@ -1,0 +1,182 @@
+"""Benchmark of the fixed-fan-in sparse layer on one MI355X.
+
+One step = forward + backward (input gradient and weight gradient) of the layer over one batch of
+synthetic input that is already resident in HBM, through the same C-ABI entry points the op
+bindings use.  Prints ONE JSON line (metric: samples/s of forward+backward at 670,091 labels,
+fan-in 32), with the roofline figures of the slowest kernel and a CPU baseline timed on this box.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2] [--layout nb|bn]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0        # MI355X published HBM3E peak
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="c2", help="workload: c1..c4 (c2 is the headline)")
+    ap.add_argument("--layout", default="nb", choices=["nb", "bn"],
+                    help="features as [N,B] (the production 'Tp' op) or [B,N]")
+    ap.add_argument("--seed", type=int, default=42)
+    ap.add_argument("--cpu-labels", type=int, default=0, help="labels in the CPU-baseline sample (0 = auto)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    return ap.parse_args()
+
+
+def time_kernel(fn, stream, iters):
+    """Average duration (ms) of `fn`, HIP events recorded on the stream the kernels run on."""
+    import torch
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    fn()
+    stream.synchronize()
+    start.record(stream)
+    for _ in range(iters):
+        fn()
+    stop.record(stream)
+    stop.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def cpu_baseline(cfg, layout_tp, labels, seed):
+    """Times the CPU oracle (restatement of the reference's CPU kernels) on a bounded sample."""
+    import oracle
+    from ecml23_sparse_amd import synth
+
+    threads = oracle.default_threads()
+    t = synth.make_inputs(cfg, seed=seed, device="cpu", transposed=layout_tp, num_units=labels)
+    x, lookup, w, g = (t[k].numpy() for k in ("features", "lookup", "weights", "out_grad"))
+    oracle.forward(x[:, :], lookup[:1024], w[:1024], transposed=layout_tp, threads=threads)   # warm-up
+    best = None
+    for _ in range(2):
+        t0 = time.perf_counter()
+        oracle.forward(x, lookup, w, transposed=layout_tp, threads=threads)
+        oracle.weight_grad(x, lookup, w, g, transposed=layout_tp, threads=threads)
+        oracle.input_grad(x, lookup, w, g, transposed=layout_tp, threads=threads)
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    full_time = best * cfg.num_units / labels        # every pass is linear in the label count
+    return {
+        "value": cfg.batch / full_time,
+        "unit": "samples/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"{labels} of {cfg.num_units} labels (same B, N, K, laws); fwd+gW+gx in {best:.3f} s, "
+                  f"scaled linearly to the full label count",
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus above 1 is not supported "
+              "(the layer would shard by label, see DESIGN.md)", file=sys.stderr)
+        sys.exit(2)
+
+    import importlib
+
+    import torch
+
+    pkg = importlib.import_module("ecml23-sparse_amd")
+    from ecml23_sparse_amd import synth
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
+        sys.exit(3)
+    torch.cuda.set_device(0)
+    cfg = synth.CONFIGS[args.config]
+    tp = args.layout == "nb"
+    t = synth.make_inputs(cfg, seed=args.seed, device="cuda", transposed=tp)
+    x, lookup, w, g = t["features"], t["lookup"], t["weights"], t["out_grad"]
+    B, N, L, K = cfg.batch, cfg.num_features, cfg.num_units, cfg.fan_in
+    out = torch.empty((B, L), device="cuda")
+    gx = torch.empty_like(x)
+    gw = torch.empty_like(w)
+    lib = pkg._lib.lib()
+    check = pkg._lib.check
+    stream = torch.cuda.current_stream()
+    sh = stream.cuda_stream
+    ptr = lambda a: a.data_ptr()  # noqa: E731
+
+    def step():
+        check(lib.ffi_forward_f32(ptr(x), ptr(lookup), ptr(w), ptr(out), B, N, L, K, int(tp), sh))
+        check(lib.ffi_backward_f32(ptr(x), ptr(lookup), ptr(w), ptr(g), ptr(gx), ptr(gw), B, N, L, K, int(tp), sh))
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+
+    # per-kernel durations with events on the launch stream (explicit plan: the kernel alone)
+    import ctypes
+    plan = ctypes.c_void_p()
+    check(lib.ffi_plan_create(ptr(lookup), L, K, N, B, sh, ctypes.byref(plan)))
+    iters = max(3, min(args.steps, 20))
+    kernels = {
+        "forward": lambda: check(lib.ffi_forward_f32(ptr(x), ptr(lookup), ptr(w), ptr(out), B, N, L, K, int(tp), sh)),
+        "weight_grad": lambda: check(lib.ffi_weight_grad_f32(ptr(x), ptr(lookup), ptr(g), ptr(gw), B, N, L, K, int(tp), sh)),
+        "input_grad": lambda: check(lib.ffi_input_grad_planned_f32(plan, ptr(w), ptr(g), ptr(gx), B, int(tp), sh)),
+    }
+    kernel_ms = {name: time_kernel(fn, stream, iters) for name, fn in kernels.items()}
+    check(lib.ffi_plan_destroy(plan))
+    alg = synth.algorithmic_bytes(cfg)
+    dominant = max(kernel_ms, key=kernel_ms.get)
+    achieved = alg[dominant] / (kernel_ms[dominant] * 1e-3) / 1e9
+    roofline = {
+        "bound": "hbm",
+        "kernel": dominant,
+        "achieved": round(achieved, 2),
+        "peak": HBM_PEAK_GBPS,
+        "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBPS, 4),
+        "traffic": None,
+        "algorithmic_bytes": alg[dominant],
+        "kernel_ms": {k: round(v, 4) for k, v in kernel_ms.items()},
+        "all_kernels_gbps": {k: round(alg[k] / (v * 1e-3) / 1e9, 1) for k, v in kernel_ms.items()},
+        "three_pass_gbps": round(alg["total"] / (sum(kernel_ms.values()) * 1e-3) / 1e9, 1),
+    }
+
+    result = {
+        "metric": "ffi_fwd_bwd_samples_per_s",
+        "value": round(B / (ms_per_step * 1e-3), 1),
+        "unit": "samples/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": f"{cfg.name}: FFI layer fwd+input-grad+weight-grad, batch {B}, {N} inputs, "
+                               f"{L} labels, fan-in {K}, features [{'N,B' if tp else 'B,N'}]",
+                   "label_samples_per_s": round(B * L / (ms_per_step * 1e-3), 1)},
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        labels = args.cpu_labels or max(4096, min(L, int(2.0e9 / (B * K))))
+        result["cpu_baseline"] = cpu_baseline(cfg, tp, min(labels, L), args.seed)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,259 @@
+// extern "C" entry points of libffi_hip.so: argument checks, plan cache, dispatch.
+// No arithmetic lives here.
+#include "ffi_internal.h"
+
+#include <climits>
+#include <mutex>
+#include <new>
+#include <vector>
+
+namespace ffi {
+
+static thread_local int g_last_hip_error = 0;
+
+int hip_fail(hipError_t e) {
+    g_last_hip_error = (int)e;
+    (void)hipGetLastError();  // clear the sticky "last error" so later calls are not blamed
+    return FFI_ERR_HIP;
+}
+
+namespace {
+
+std::mutex g_cache_mutex;
+std::vector<ffi_plan*> g_cache;   // plans owned by the library, one per (device, lookup, shape)
+constexpr size_t kMaxCachedPlans = 8;
+
+// The reference narrows every size to int32 and fail-fasts otherwise (forward.cu:24-28).
+int check_dims(int64_t B, int64_t N, int64_t L, int64_t K, int transposed, Dims* d) {
+    if (B <= 0 || N <= 0 || L <= 0 || K <= 0) return FFI_ERR_BAD_SHAPE;
+    if (B >= INT32_MAX || N >= INT32_MAX || L >= INT32_MAX || K >= INT32_MAX) return FFI_ERR_TOO_LARGE;
+    if (L * K >= INT32_MAX) return FFI_ERR_TOO_LARGE;   // flat connection positions are int32
+    d->B = (int)B; d->N = (int)N; d->L = (int)L; d->K = (int)K; d->tp = transposed != 0;
+    return FFI_OK;
+}
+
+int plan_alloc(int L, int K, int N, ffi_plan** out) {
+    ffi_plan* p = new (std::nothrow) ffi_plan();
+    if (!p) return FFI_ERR_OUT_OF_MEMORY;
+    if (hipGetDevice(&p->device) != hipSuccess) { delete p; return FFI_ERR_NO_DEVICE; }
+    p->L = L; p->K = K; p->N = N;
+    const size_t total = (size_t)L * K;
+    bool ok = hipMalloc(&p->perm, total * sizeof(int32_t)) == hipSuccess &&
+              hipMalloc(&p->col_ptr, ((size_t)N + 1) * sizeof(int32_t)) == hipSuccess &&
+              hipMalloc(&p->d_scratch, 8 * sizeof(unsigned long long)) == hipSuccess &&
+              hipHostMalloc(&p->h_scratch, 8 * sizeof(unsigned long long)) == hipSuccess;
+    if (!ok) {
+        (void)hipGetLastError();
+        plan_free(p);
+        delete p;
+        return FFI_ERR_OUT_OF_MEMORY;
+    }
+    p->bytes = total * sizeof(int32_t) + ((size_t)N + 1) * sizeof(int32_t) + 64;
+    *out = p;
+    return FFI_OK;
+}
+
+// Finds or builds the cached plan for `lookup`; re-checks the content fingerprint on every call.
+// Caller holds g_cache_mutex.
+int cached_plan(const int32_t* lookup, const Dims& d, hipStream_t s, ffi_plan** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) return FFI_ERR_NO_DEVICE;
+    ffi_plan* hit = nullptr;
+    for (size_t i = 0; i < g_cache.size(); ++i) {
+        ffi_plan* p = g_cache[i];
+        if (p->device == dev && p->lookup == lookup && p->L == d.L && p->K == d.K && p->N == d.N) {
+            hit = p;
+            g_cache.erase(g_cache.begin() + i);   // move to the back (most recently used)
+            g_cache.push_back(p);
+            break;
+        }
+    }
+    if (hit) {
+        unsigned long long fp = 0, bad = 0;
+        FFI_TRY(plan_fingerprint(hit, lookup, s, &fp, &bad));
+        if (bad) return FFI_ERR_BAD_LOOKUP;
+        if (fp != hit->fingerprint) FFI_TRY(plan_build(hit, lookup, s));
+        *out = hit;
+        return FFI_OK;
+    }
+    if (g_cache.size() >= kMaxCachedPlans) {
+        // evict the least recently used plan of this device; its stream work must have drained
+        for (size_t i = 0; i < g_cache.size(); ++i) {
+            if (g_cache[i]->device == dev) {
+                (void)hipDeviceSynchronize();
+                plan_free(g_cache[i]);
+                delete g_cache[i];
+                g_cache.erase(g_cache.begin() + i);
+                break;
+            }
+        }
+    }
+    ffi_plan* p = nullptr;
+    FFI_TRY(plan_alloc(d.L, d.K, d.N, &p));
+    int st = plan_build(p, lookup, s);
+    if (st != FFI_OK) { plan_free(p); delete p; return st; }
+    g_cache.push_back(p);
+    *out = p;
+    return FFI_OK;
+}
+
+}  // namespace
+}  // namespace ffi
+
+using namespace ffi;
+
+extern "C" {
+
+int ffi_abi_version(void) { return 1; }
+const char* ffi_target_arch(void) { return "gfx950"; }
+int ffi_last_hip_error(void) { return g_last_hip_error; }
+
+const char* ffi_status_string(int status) {
+    switch (status) {
+        case FFI_OK: return "ok";
+        case FFI_ERR_NULL_POINTER: return "null pointer argument";
+        case FFI_ERR_BAD_SHAPE: return "a dimension is <= 0 or shapes disagree";
+        case FFI_ERR_TOO_LARGE: return "a size exceeds the 32-bit contract";
+        case FFI_ERR_HIP: return "HIP runtime call failed";
+        case FFI_ERR_OUT_OF_MEMORY: return "out of memory";
+        case FFI_ERR_BAD_LOOKUP: return "lookup holds a column id outside [0, num_features)";
+        case FFI_ERR_NO_DEVICE: return "no usable HIP device";
+        case FFI_ERR_BAD_ARGUMENT: return "bad argument";
+        default: return "unknown status";
+    }
+}
+
+int ffi_forward_f32(const float* features, const int32_t* lookup, const float* weights, float* result,
+                    int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in,
+                    int transposed, ffi_stream_t stream) {
+    if (!features || !lookup || !weights || !result) return FFI_ERR_NULL_POINTER;
+    Dims d;
+    FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
+    return launch_forward(features, lookup, weights, result, d, (hipStream_t)stream);
+}
+
+int ffi_weight_grad_f32(const float* features, const int32_t* lookup, const float* out_grad,
+                        float* weight_grad, int64_t batch, int64_t num_features, int64_t num_units,
+                        int64_t fan_in, int transposed, ffi_stream_t stream) {
+    if (!features || !lookup || !out_grad || !weight_grad) return FFI_ERR_NULL_POINTER;
+    Dims d;
+    FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
+    return launch_weight_grad(features, lookup, out_grad, weight_grad, d, (hipStream_t)stream);
+}
+
+int ffi_input_grad_f32(const int32_t* lookup, const float* weights, const float* out_grad,
+                       float* feature_grad, int64_t batch, int64_t num_features, int64_t num_units,
+                       int64_t fan_in, int transposed, ffi_stream_t stream) {
+    if (!lookup || !weights || !out_grad || !feature_grad) return FFI_ERR_NULL_POINTER;
+    Dims d;
+    FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    ffi_plan* p = nullptr;
+    FFI_TRY(cached_plan(lookup, d, (hipStream_t)stream, &p));
+    return launch_input_grad(p, weights, out_grad, feature_grad, d.B, d.tp, (hipStream_t)stream);
+}
+
+int ffi_backward_f32(const float* features, const int32_t* lookup, const float* weights,
+                     const float* out_grad, float* feature_grad, float* weight_grad, int64_t batch,
+                     int64_t num_features, int64_t num_units, int64_t fan_in, int transposed,
+                     ffi_stream_t stream) {
+    if (!features || !lookup || !weights || !out_grad) return FFI_ERR_NULL_POINTER;
+    if (!feature_grad && !weight_grad) return FFI_ERR_NULL_POINTER;
+    // weight gradient first, then input gradient, as backward.cpp:95-107 orders them
+    if (weight_grad)
+        FFI_TRY(ffi_weight_grad_f32(features, lookup, out_grad, weight_grad, batch, num_features, num_units, fan_in,
+                                    transposed, stream));
+    if (feature_grad)
+        FFI_TRY(ffi_input_grad_f32(lookup, weights, out_grad, feature_grad, batch, num_features, num_units, fan_in,
+                                   transposed, stream));
+    return FFI_OK;
+}
+
+int ffi_plan_create(const int32_t* lookup, int64_t num_units, int64_t fan_in, int64_t num_features,
+                    int64_t batch_hint, ffi_stream_t stream, ffi_plan** plan) {
+    if (!lookup || !plan) return FFI_ERR_NULL_POINTER;
+    *plan = nullptr;
+    Dims d;
+    FFI_TRY(check_dims(batch_hint > 0 ? batch_hint : 1, num_features, num_units, fan_in, 0, &d));
+    ffi_plan* p = nullptr;
+    FFI_TRY(plan_alloc(d.L, d.K, d.N, &p));
+    int st = plan_build(p, lookup, (hipStream_t)stream);
+    if (st != FFI_OK) { plan_free(p); delete p; return st; }
+    *plan = p;
+    return FFI_OK;
+}
+
+int ffi_plan_refresh(ffi_plan* plan, const int32_t* lookup, ffi_stream_t stream) {
+    if (!plan || !lookup) return FFI_ERR_NULL_POINTER;
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) return FFI_ERR_NO_DEVICE;
+    if (dev != plan->device) return FFI_ERR_BAD_ARGUMENT;
+    return plan_build(plan, lookup, (hipStream_t)stream);
+}
+
+int ffi_plan_destroy(ffi_plan* plan) {
+    if (!plan) return FFI_OK;
+    plan_free(plan);
+    delete plan;
+    return FFI_OK;
+}
+
+int ffi_input_grad_planned_f32(const ffi_plan* plan, const float* weights, const float* out_grad,
+                               float* feature_grad, int64_t batch, int transposed, ffi_stream_t stream) {
+    if (!plan || !weights || !out_grad || !feature_grad) return FFI_ERR_NULL_POINTER;
+    if (batch <= 0) return FFI_ERR_BAD_SHAPE;
+    if (batch >= INT32_MAX) return FFI_ERR_TOO_LARGE;
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) return FFI_ERR_NO_DEVICE;
+    if (dev != plan->device) return FFI_ERR_BAD_ARGUMENT;
+    return launch_input_grad(plan, weights, out_grad, feature_grad, (int)batch, transposed != 0, (hipStream_t)stream);
+}
+
+int ffi_cache_clear(void) {
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) return FFI_ERR_NO_DEVICE;
+    (void)hipDeviceSynchronize();
+    for (size_t i = 0; i < g_cache.size();) {
+        if (g_cache[i]->device == dev) {
+            plan_free(g_cache[i]);
+            delete g_cache[i];
+            g_cache.erase(g_cache.begin() + i);
+        } else {
+            ++i;
+        }
+    }
+    return FFI_OK;
+}
+
+size_t ffi_cache_bytes(void) {
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    size_t total = 0;
+    for (ffi_plan* p : g_cache)
+        if (p->device == dev) total += p->bytes;
+    return total;
+}
+
+int ffi_check_lookup(const int32_t* lookup, int64_t num_units, int64_t fan_in, int64_t num_features,
+                     ffi_stream_t stream) {
+    if (!lookup) return FFI_ERR_NULL_POINTER;
+    Dims d;
+    FFI_TRY(check_dims(1, num_features, num_units, fan_in, 0, &d));
+    ffi_plan tmp;
+    tmp.L = d.L; tmp.K = d.K; tmp.N = d.N;
+    if (hipMalloc(&tmp.d_scratch, 8 * sizeof(unsigned long long)) != hipSuccess ||
+        hipHostMalloc(&tmp.h_scratch, 8 * sizeof(unsigned long long)) != hipSuccess) {
+        (void)hipGetLastError();
+        plan_free(&tmp);
+        return FFI_ERR_OUT_OF_MEMORY;
+    }
+    unsigned long long fp = 0, bad = 0;
+    int st = plan_fingerprint(&tmp, lookup, (hipStream_t)stream, &fp, &bad);
+    plan_free(&tmp);
+    if (st != FFI_OK) return st;
+    return bad ? FFI_ERR_BAD_LOOKUP : FFI_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,124 @@
+"""Fixed-fan-in sparse matmul ops on torch device tensors, backed by the HIP C ABI.
+
+Mirrors the reference's Python op surface (sparse/ops/fixed_fan_in_ops.py:15-40): the same four
+functions with the same argument order ``(features, lookup, weights[, out_grad])`` and layouts,
+and the same gradient wiring ``[feature_grad, None, weight_grad]``.  Shape rules follow the op
+shape functions (tfsparse/cc/ops/fixed_fan_in_ops.cpp:14-53).  torch is used for device memory
+and streams only; all arithmetic runs in libffi_hip.so.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+_INDEX_DTYPES = (torch.int32, torch.uint32)
+
+
+def _stream_handle(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _check_inputs(features, lookup, weights, transposed, out_grad=None):
+    # rank / shape agreement, as the reference's shape functions demand at graph time
+    for name, t in (("features", features), ("lookup", lookup), ("weights", weights)):
+        if t.dim() != 2:
+            raise ValueError(f"{name} must have rank 2, got shape {tuple(t.shape)}")
+    if tuple(lookup.shape) != tuple(weights.shape):
+        raise ValueError(f"lookup {tuple(lookup.shape)} and weights {tuple(weights.shape)} must have equal shapes")
+    if features.dtype != torch.float32 or weights.dtype != torch.float32:
+        raise TypeError("only float32 features/weights are registered (as in the reference)")
+    if lookup.dtype not in _INDEX_DTYPES:
+        raise TypeError("lookup must be int32 or uint32 (as in the reference)")
+    if not features.is_cuda:
+        raise RuntimeError("the HIP path needs device tensors; there is no CPU fallback in this package")
+    if lookup.device != features.device or weights.device != features.device:
+        raise RuntimeError("features, lookup and weights must live on the same device")
+    batch = features.shape[1] if transposed else features.shape[0]
+    num_features = features.shape[0] if transposed else features.shape[1]
+    num_units, fan_in = lookup.shape
+    if out_grad is not None:
+        if out_grad.dim() != 2 or tuple(out_grad.shape) != (batch, num_units):
+            raise ValueError(f"out_grad must have shape {(batch, num_units)}, got {tuple(out_grad.shape)}")
+        if out_grad.dtype != torch.float32 or out_grad.device != features.device:
+            raise TypeError("out_grad must be float32 on the features' device")
+    return batch, num_features, num_units, fan_in
+
+
+def _forward(features, lookup, weights, transposed):
+    batch, num_features, num_units, fan_in = _check_inputs(features, lookup, weights, transposed)
+    features = features.contiguous()
+    lookup = lookup.contiguous()
+    weights = weights.contiguous()
+    with torch.cuda.device(features.device):
+        result = torch.empty((batch, num_units), dtype=torch.float32, device=features.device)
+        _lib.check(_lib.lib().ffi_forward_f32(
+            features.data_ptr(), lookup.data_ptr(), weights.data_ptr(), result.data_ptr(),
+            batch, num_features, num_units, fan_in, int(transposed), _stream_handle(features.device)))
+    return result
+
+
+def _backward(features, lookup, weights, out_grad, transposed):
+    batch, num_features, num_units, fan_in = _check_inputs(features, lookup, weights, transposed, out_grad)
+    features = features.contiguous()
+    lookup = lookup.contiguous()
+    weights = weights.contiguous()
+    out_grad = out_grad.contiguous()
+    with torch.cuda.device(features.device):
+        feature_grad = torch.empty_like(features)
+        weight_grad = torch.empty_like(weights)
+        _lib.check(_lib.lib().ffi_backward_f32(
+            features.data_ptr(), lookup.data_ptr(), weights.data_ptr(), out_grad.data_ptr(),
+            feature_grad.data_ptr(), weight_grad.data_ptr(),
+            batch, num_features, num_units, fan_in, int(transposed), _stream_handle(features.device)))
+    return feature_grad, weight_grad
+
+
+def fan_in_sparse_matmul_grad(features, lookup, weights, out_grad):
+    """Op FanInSparseMatmulGrad: returns ``(feature_grad [B,N], weight_grad [L,K])``."""
+    return _backward(features, lookup, weights, out_grad, False)
+
+
+def fan_in_sparse_matmul_grad_tp(features, lookup, weights, out_grad):
+    """Op FanInSparseMatmulGradTp: features and feature_grad are ``[N,B]``."""
+    return _backward(features, lookup, weights, out_grad, True)
+
+
+class FanInSparseMatmul(torch.autograd.Function):
+    """Forward op with the gradient the reference registers for it (fixed_fan_in_ops.py:31-34)."""
+
+    @staticmethod
+    def forward(ctx, features, lookup, weights):
+        ctx.save_for_backward(features, lookup, weights)
+        return _forward(features, lookup, weights, False)
+
+    @staticmethod
+    def backward(ctx, grad):
+        features, lookup, weights = ctx.saved_tensors
+        feature_grad, weight_grad = fan_in_sparse_matmul_grad(features, lookup, weights, grad)
+        return feature_grad, None, weight_grad
+
+
+class FanInSparseMatmulTp(torch.autograd.Function):
+    """Transposed-features op and its gradient (fixed_fan_in_ops.py:37-40)."""
+
+    @staticmethod
+    def forward(ctx, features, lookup, weights):
+        ctx.save_for_backward(features, lookup, weights)
+        return _forward(features, lookup, weights, True)
+
+    @staticmethod
+    def backward(ctx, grad):
+        features, lookup, weights = ctx.saved_tensors
+        feature_grad, weight_grad = fan_in_sparse_matmul_grad_tp(features, lookup, weights, grad)
+        return feature_grad, None, weight_grad
+
+
+def fan_in_sparse_matmul(features, lookup, weights):
+    """Op FanInSparseMatmul: ``result[b,j] = sum_k weights[j,k] * features[b, lookup[j,k]]``."""
+    return FanInSparseMatmul.apply(features, lookup, weights)
+
+
+def fan_in_sparse_matmul_tp(features, lookup, weights):
+    """Op FanInSparseMatmulTp: as above with features given as ``[N,B]``; result is ``[B,L]``."""
+    return FanInSparseMatmulTp.apply(features, lookup, weights)

@@ -1,0 +1,124 @@
+/*
+ * C ABI of the MI355X (gfx950) fixed-fan-in sparse layer kernels.
+ *
+ * This is the boundary a host framework binds to.  It replaces the GPU half of the reference's
+ * kernel functors
+ *     FixedFanInSparseMatmulKernel<GPUDevice,...>::operator()      tfsparse/cc/kernels/common.h:20-26
+ *     FixedFanInSparseMatmulGradKernel<GPUDevice,...>::operator()  tfsparse/cc/kernels/common.h:28-37
+ * as they are called from the TensorFlow op kernels in tfsparse/cc/kernels/register.cpp:18-39,48-72.
+ *
+ * Conventions
+ *   - all pointers are DEVICE pointers to dense, contiguous, row-major buffers owned by the caller;
+ *   - features is [batch, num_features], or [num_features, batch] when `transposed` != 0
+ *     (the reference's "Tp" ops); lookup, weights, weight_grad are [num_units, fan_in];
+ *     result / out_grad are [batch, num_units]; feature_grad has the shape of features;
+ *   - lookup holds column ids in [0, num_features); int32 and uint32 share the entry points
+ *     (same bits for valid ids), duplicates inside a row are legal and accumulate;
+ *   - outputs are fully overwritten; work is enqueued on `stream` (a hipStream_t passed as void*,
+ *     NULL = the default stream) and, with two documented exceptions, never synchronises the host;
+ *   - every function returns FFI_OK (0) or a negative ffi_status instead of aborting, where the
+ *     reference fail-fasts through gsl_Expects (forward.cu:19-28, backward.cu:27-40):
+ *     null pointers, any dimension <= 0 or > INT32_MAX, num_units*fan_in > INT32_MAX.
+ *   - the library is thread-safe; calls that share a plan or the internal plan cache serialise.
+ */
+#ifndef FFI_HIP_H
+#define FFI_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* ffi_stream_t;           /* hipStream_t */
+typedef struct ffi_plan ffi_plan;     /* column-ordered view of one lookup matrix (opaque) */
+
+enum ffi_status {
+    FFI_OK = 0,
+    FFI_ERR_NULL_POINTER = -1,
+    FFI_ERR_BAD_SHAPE = -2,       /* a dimension is <= 0, or shapes disagree */
+    FFI_ERR_TOO_LARGE = -3,       /* a size does not fit the 32-bit contract of the reference */
+    FFI_ERR_HIP = -4,             /* a HIP runtime call failed; see ffi_last_hip_error() */
+    FFI_ERR_OUT_OF_MEMORY = -5,
+    FFI_ERR_BAD_LOOKUP = -6,      /* a column id is outside [0, num_features) */
+    FFI_ERR_NO_DEVICE = -7,
+    FFI_ERR_BAD_ARGUMENT = -8
+};
+
+/* Library identification: ABI version (bumped on incompatible changes) and the code-object target. */
+int ffi_abi_version(void);
+const char* ffi_target_arch(void);
+const char* ffi_status_string(int status);
+/* hipError_t of the last failing runtime call on the calling thread (0 if none). */
+int ffi_last_hip_error(void);
+
+/*
+ * Forward:  result[b,j] = sum_k weights[j,k] * features[b, lookup[j,k]].
+ * Replaces FixedFanInSparseMatmulKernel<GPUDevice,float,Int,*,Transposed>::operator()
+ * (tfsparse/cc/kernels/forward.cu:36-74; CPU semantics tfsparse/cc/kernels/forward.cpp:9-44),
+ * i.e. the compute of ops FanInSparseMatmul / FanInSparseMatmulTp
+ * (tfsparse/cc/ops/fixed_fan_in_ops.cpp:55-71).
+ */
+int ffi_forward_f32(const float* features, const int32_t* lookup, const float* weights, float* result,
+                    int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in,
+                    int transposed, ffi_stream_t stream);
+
+/*
+ * Backward, both gradients from one call, as the reference's grad op does:
+ *   feature_grad[b,n] = sum over (j,k) with lookup[j,k]==n of weights[j,k] * out_grad[b,j]
+ *   weight_grad[j,k]  = sum_b features[b, lookup[j,k]] * out_grad[b,j]
+ * Replaces FixedFanInSparseMatmulGradKernel<GPUDevice,float,Int,*,Transposed>::operator()
+ * (tfsparse/cc/kernels/backward.cu:49-133; CPU semantics tfsparse/cc/kernels/backward.cpp:8-73),
+ * i.e. ops FanInSparseMatmulGrad / FanInSparseMatmulGradTp (fixed_fan_in_ops.cpp:73-93).
+ * Either output pointer may be NULL to skip that gradient.  The input gradient uses no float
+ * atomics: results are bit-identical from run to run.  It needs a column-ordered view of `lookup`
+ * which is built on the device on first use and cached inside the library, keyed on the lookup
+ * pointer and shape and guarded by a content fingerprint that is re-checked on every call, so
+ * in-place edits of lookup (rewiring, sparse/custom_layer.py:32-43) are picked up.
+ */
+int ffi_backward_f32(const float* features, const int32_t* lookup, const float* weights,
+                     const float* out_grad, float* feature_grad, float* weight_grad,
+                     int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in,
+                     int transposed, ffi_stream_t stream);
+
+/* The two halves of ffi_backward_f32 on their own (backward.cpp:8-36 and :39-73). */
+int ffi_weight_grad_f32(const float* features, const int32_t* lookup, const float* out_grad,
+                        float* weight_grad,
+                        int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in,
+                        int transposed, ffi_stream_t stream);
+int ffi_input_grad_f32(const int32_t* lookup, const float* weights, const float* out_grad,
+                       float* feature_grad,
+                       int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in,
+                       int transposed, ffi_stream_t stream);
+
+/*
+ * Explicit plans, for callers that know when lookup changes (e.g. once per rewire interval,
+ * sparse/optimizer.py:68-74) and want to skip the per-call fingerprint.  No counterpart in the
+ * reference, whose input gradient scatters with atomicAdd (backward.cu.h:119,139,161,182).
+ * ffi_plan_create synchronises `stream` once.  A plan is tied to the device it was made on.
+ */
+int ffi_plan_create(const int32_t* lookup, int64_t num_units, int64_t fan_in, int64_t num_features,
+                    int64_t batch_hint, ffi_stream_t stream, ffi_plan** plan);
+int ffi_plan_refresh(ffi_plan* plan, const int32_t* lookup, ffi_stream_t stream);
+int ffi_plan_destroy(ffi_plan* plan);
+int ffi_input_grad_planned_f32(const ffi_plan* plan, const float* weights, const float* out_grad,
+                               float* feature_grad, int64_t batch, int transposed, ffi_stream_t stream);
+
+/* Drops every cached plan and workspace of the calling thread's current device. */
+int ffi_cache_clear(void);
+/* Device bytes currently held by the library (plans + workspaces) on the current device. */
+size_t ffi_cache_bytes(void);
+
+/*
+ * Host-side audit of a lookup matrix (the reference checks index ranges only in audit builds,
+ * tfsparse/cc/kernels/kernel_data.cu.h:26-43,211).  Synchronises `stream`.
+ * Returns FFI_OK, or FFI_ERR_BAD_LOOKUP if any id is >= num_features (as unsigned).
+ */
+int ffi_check_lookup(const int32_t* lookup, int64_t num_units, int64_t fan_in, int64_t num_features,
+                     ffi_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FFI_HIP_H */

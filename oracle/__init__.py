@@ -1,0 +1,206 @@
+"""CPU oracle for the fixed-fan-in sparse layer: TEST INFRASTRUCTURE, never the product path.
+
+Thin ctypes binding over ``libffi_oracle.so`` (built from ``ffi_oracle.c`` by ``oracle/Makefile``)
+plus a dense numpy restatement of the reference's own ground truth
+(tfsparse/cc/kernels/reference.cpp:15-82) for small shapes.
+
+Only the test-suite, ``__graft_entry__.smoke()`` and the CPU-baseline leg of ``bench.py`` import
+this package.  All functions take and return numpy arrays.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libffi_oracle.so")
+_lib = None
+
+_f32p = ctypes.POINTER(ctypes.c_float)
+_f64p = ctypes.POINTER(ctypes.c_double)
+_i32p = ctypes.POINTER(ctypes.c_int32)
+_i64 = ctypes.c_int64
+
+
+def build(force: bool = False) -> str:
+    """Compile the C restatement with the Makefile next to it; returns the library path."""
+    if force and os.path.exists(_LIB_PATH):
+        os.remove(_LIB_PATH)
+    subprocess.run(["make", "-s", "-C", _HERE], check=True)
+    return _LIB_PATH
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = ctypes.CDLL(_LIB_PATH)
+        common = [_i64, _i64, _i64, _i64, ctypes.c_int, ctypes.c_int]
+        _lib.ffi_oracle_forward_f32.argtypes = [_f32p, _i32p, _f32p, _f32p] + common
+        _lib.ffi_oracle_forward_f64.argtypes = [_f32p, _i32p, _f32p, _f64p] + common
+        for name, outp in (("ffi_oracle_weight_grad_f32", _f32p), ("ffi_oracle_input_grad_f32", _f32p),
+                           ("ffi_oracle_weight_grad_f64", _f64p), ("ffi_oracle_input_grad_f64", _f64p)):
+            getattr(_lib, name).argtypes = [_f32p, _i32p, _f32p, _f32p, outp] + common
+        _lib.ffi_oracle_backward_f32.argtypes = [_f32p, _i32p, _f32p, _f32p, _f32p, _f32p] + common
+        for name in ("ffi_oracle_forward_f32", "ffi_oracle_forward_f64", "ffi_oracle_weight_grad_f32",
+                     "ffi_oracle_input_grad_f32", "ffi_oracle_weight_grad_f64", "ffi_oracle_input_grad_f64",
+                     "ffi_oracle_backward_f32"):
+            getattr(_lib, name).restype = ctypes.c_int
+        _lib.ffi_oracle_round_bf16_array.argtypes = [_f32p, _f32p, _i64]
+        _lib.ffi_oracle_round_bf16_array.restype = None
+        _lib.ffi_oracle_topk_f32.argtypes = [_f32p, _i64, _i64, ctypes.c_int, _f32p, _i32p]
+        _lib.ffi_oracle_topk_f32.restype = None
+    return _lib
+
+
+def default_threads() -> int:
+    """All hardware threads, as the reference's CPU harness does (testing/cpu.cpp:36-37)."""
+    return max(1, os.cpu_count() or 1)
+
+
+def _f32(a):
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    return a, a.ctypes.data_as(_f32p)
+
+
+def _idx(a):
+    a = np.asarray(a)
+    if a.dtype == np.uint32:
+        a = a.view(np.int32)          # same bits; the C side widens through uint32_t
+    a = np.ascontiguousarray(a, dtype=np.int32)
+    return a, a.ctypes.data_as(_i32p)
+
+
+def _dims(features, lookup, transposed):
+    if features.ndim != 2 or lookup.ndim != 2:
+        raise ValueError("features and lookup must be matrices")
+    if transposed:
+        N, B = features.shape
+    else:
+        B, N = features.shape
+    L, K = lookup.shape
+    return B, N, L, K
+
+
+def _check(rc, what):
+    if rc != 0:
+        raise RuntimeError(f"oracle {what} failed with status {rc}")
+
+
+def forward(features, lookup, weights, transposed=False, threads=None, f64=False):
+    """out[b,j] = sum_k weights[j,k] * features[b, lookup[j,k]]  (forward.cpp:9-44)."""
+    features, fp = _f32(features)
+    lookup, lp = _idx(lookup)
+    weights, wp = _f32(weights)
+    B, N, L, K = _dims(features, lookup, transposed)
+    assert weights.shape == (L, K)
+    threads = threads or default_threads()
+    if f64:
+        out = np.empty((B, L), dtype=np.float64)
+        _check(lib().ffi_oracle_forward_f64(fp, lp, wp, out.ctypes.data_as(_f64p), B, N, L, K, int(transposed), threads), "forward_f64")
+    else:
+        out = np.empty((B, L), dtype=np.float32)
+        _check(lib().ffi_oracle_forward_f32(fp, lp, wp, out.ctypes.data_as(_f32p), B, N, L, K, int(transposed), threads), "forward_f32")
+    return out
+
+
+def weight_grad(features, lookup, weights, out_grad, transposed=False, threads=None, f64=False):
+    """gw[j,k] = sum_b features[b, lookup[j,k]] * out_grad[b,j]  (backward.cpp:8-36)."""
+    features, fp = _f32(features)
+    lookup, lp = _idx(lookup)
+    weights, wp = _f32(weights)
+    out_grad, gp = _f32(out_grad)
+    B, N, L, K = _dims(features, lookup, transposed)
+    assert out_grad.shape == (B, L)
+    threads = threads or default_threads()
+    if f64:
+        gw = np.empty((L, K), dtype=np.float64)
+        _check(lib().ffi_oracle_weight_grad_f64(fp, lp, wp, gp, gw.ctypes.data_as(_f64p), B, N, L, K, int(transposed), threads), "weight_grad_f64")
+    else:
+        gw = np.empty((L, K), dtype=np.float32)
+        _check(lib().ffi_oracle_weight_grad_f32(fp, lp, wp, gp, gw.ctypes.data_as(_f32p), B, N, L, K, int(transposed), threads), "weight_grad_f32")
+    return gw
+
+
+def input_grad(features, lookup, weights, out_grad, transposed=False, threads=None, f64=False):
+    """gx[b, lookup[j,k]] += weights[j,k] * out_grad[b,j]  (backward.cpp:39-73)."""
+    features, fp = _f32(features)
+    lookup, lp = _idx(lookup)
+    weights, wp = _f32(weights)
+    out_grad, gp = _f32(out_grad)
+    B, N, L, K = _dims(features, lookup, transposed)
+    assert out_grad.shape == (B, L)
+    threads = threads or default_threads()
+    # pre-filled with garbage, like the reference's tests do, so an unwritten element shows
+    if f64:
+        gx = np.full(features.shape, np.nan, dtype=np.float64)
+        _check(lib().ffi_oracle_input_grad_f64(fp, lp, wp, gp, gx.ctypes.data_as(_f64p), B, N, L, K, int(transposed), threads), "input_grad_f64")
+    else:
+        gx = np.full(features.shape, np.nan, dtype=np.float32)
+        _check(lib().ffi_oracle_input_grad_f32(fp, lp, wp, gp, gx.ctypes.data_as(_f32p), B, N, L, K, int(transposed), threads), "input_grad_f32")
+    return gx
+
+
+def backward(features, lookup, weights, out_grad, transposed=False, threads=None):
+    """(feature_grad, weight_grad) in the order the grad op returns them (register.cpp:59-60)."""
+    gw = weight_grad(features, lookup, weights, out_grad, transposed, threads)
+    gx = input_grad(features, lookup, weights, out_grad, transposed, threads)
+    return gx, gw
+
+
+def round_bf16(a):
+    """fp32 -> bf16 -> fp32 with round-to-nearest-even."""
+    a, ap = _f32(a)
+    out = np.empty_like(a)
+    lib().ffi_oracle_round_bf16_array(ap, out.ctypes.data_as(_f32p), a.size)
+    return out
+
+
+def topk(scores, k):
+    """Per-row top-k: values descending, ties resolved towards the lower index."""
+    scores, sp = _f32(scores)
+    B, L = scores.shape
+    values = np.empty((B, k), dtype=np.float32)
+    indices = np.empty((B, k), dtype=np.int32)
+    lib().ffi_oracle_topk_f32(sp, B, L, int(k), values.ctypes.data_as(_f32p), indices.ctypes.data_as(_i32p))
+    return values, indices
+
+
+# ---- dense ground truth of the reference's own tests (reference.cpp:15-82), numpy float64 -------
+
+def dense_operator(lookup, weights, num_features):
+    """D[n, j] = sum of weights[j,k] over the k with lookup[j,k] == n  (reference.cpp:15-27)."""
+    lookup = np.asarray(lookup).astype(np.int64)
+    L, K = lookup.shape
+    D = np.zeros((num_features, L), dtype=np.float64)
+    np.add.at(D, (lookup.reshape(-1), np.repeat(np.arange(L), K)), np.asarray(weights, dtype=np.float64).reshape(-1))
+    return D
+
+
+def dense_forward(features, lookup, weights, transposed=False):
+    """out = X . D  (reference.cpp:30-45)."""
+    X = np.asarray(features, dtype=np.float64)
+    if transposed:
+        X = X.T
+    return X @ dense_operator(lookup, weights, X.shape[1])
+
+
+def dense_backward(features, lookup, weights, out_grad, transposed=False):
+    """gx = G . D^T, gw[j,k] = (X^T G)[lookup[j,k], j]  (reference.cpp:48-82)."""
+    X = np.asarray(features, dtype=np.float64)
+    if transposed:
+        X = X.T
+    G = np.asarray(out_grad, dtype=np.float64)
+    D = dense_operator(lookup, weights, X.shape[1])
+    gx = G @ D.T
+    if transposed:
+        gx = gx.T
+    dense_gw = X.T @ G
+    lookup = np.asarray(lookup).astype(np.int64)
+    L, K = lookup.shape
+    gw = dense_gw[lookup, np.arange(L)[:, None]]
+    return gx, gw

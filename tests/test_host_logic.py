@@ -1,0 +1,78 @@
+"""Host-side mirror of the reference's op surface: argument rules that need no GPU."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import load_package
+
+
+def _cpu_args(B=4, N=6, L=5, K=3):
+    x = torch.zeros(B, N)
+    lookup = torch.zeros(L, K, dtype=torch.int32)
+    w = torch.zeros(L, K)
+    return x, lookup, w
+
+
+def test_same_names_as_the_reference_binding():
+    # sparse/ops/fixed_fan_in_ops.py:15-28
+    pkg = load_package()
+    for name in ("fan_in_sparse_matmul", "fan_in_sparse_matmul_tp", "fan_in_sparse_matmul_grad",
+                 "fan_in_sparse_matmul_grad_tp"):
+        assert callable(getattr(pkg, name))
+    import ecml23_sparse_amd        # alias registered by the package itself
+    assert ecml23_sparse_amd is pkg
+
+
+def test_no_cpu_fallback():
+    pkg = load_package()
+    x, lookup, w = _cpu_args()
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        pkg.fan_in_sparse_matmul(x, lookup, w)
+
+
+def test_shape_rules_of_the_op_shape_functions():
+    # tfsparse/cc/ops/fixed_fan_in_ops.cpp:14-53: rank 2 everywhere, lookup.shape == weights.shape,
+    # out_grad.shape == [B, L]
+    pkg = load_package()
+    ops = pkg.fixed_fan_in_ops
+    x, lookup, w = _cpu_args()
+    with pytest.raises(ValueError, match="rank 2"):
+        ops._check_inputs(x[0], lookup, w, False)
+    with pytest.raises(ValueError, match="equal shapes"):
+        ops._check_inputs(x, lookup[:, :2], w, False)
+    with pytest.raises(TypeError):
+        ops._check_inputs(x.double(), lookup, w, False)
+    with pytest.raises(TypeError):
+        ops._check_inputs(x, lookup.long(), w, False)
+
+
+def test_synthetic_lookup_laws():
+    pkg = load_package()
+    from ecml23_sparse_amd import synth
+    g = torch.Generator().manual_seed(1)
+    idx = synth.make_lookup(500, 32, 768, generator=g)
+    assert idx.dtype == torch.int32 and idx.shape == (500, 32)
+    assert int(idx.min()) >= 0 and int(idx.max()) < 768
+    srt = np.sort(idx.numpy(), axis=1)
+    assert (srt[:, 1:] != srt[:, :-1]).all()                      # distinct inside each row
+    wide = synth.make_lookup(300, 72, 65536, generator=g, sorted_rows=True).numpy()
+    assert (wide[:, 1:] > wide[:, :-1]).all()
+    rep = synth.make_lookup(200, 16, 8, distinct=False, generator=g).numpy()
+    assert (np.sort(rep, axis=1)[:, 1:] == np.sort(rep, axis=1)[:, :-1]).any()
+
+
+def test_synthetic_inputs_shapes_and_bytes():
+    load_package()
+    from ecml23_sparse_amd import synth
+    cfg = synth.CONFIGS["c2"]
+    t = synth.make_inputs(cfg, seed=42, num_units=1000)
+    assert t["features"].shape == (128, 768) and float(t["features"].min()) == 0.0
+    assert t["lookup"].shape == (1000, 32) and t["weights"].shape == (1000, 32) and t["out_grad"].shape == (128, 1000)
+    assert abs(float(t["weights"].std()) - 32 ** -0.5) < 0.01
+    tt = synth.make_inputs(cfg, seed=42, num_units=1000, transposed=True)
+    assert torch.equal(tt["features"].t(), t["features"])
+    b = synth.algorithmic_bytes(cfg)
+    # 515.0 MB per pass at 670,091 labels x fan-in 32 x 768 inputs x batch 128
+    assert b["forward"] == b["input_grad"] == b["weight_grad"] == 515_023_104
+    c3 = synth.make_inputs(synth.CONFIGS["c3"], num_units=10)["features"]
+    assert torch.allclose(c3.norm(dim=1), torch.ones(256), atol=1e-5) and float(c3.min()) >= 0

@@ -1,0 +1,204 @@
+"""Pins the CPU oracle (oracle/ffi_oracle.c) with evidence that does not come from the oracle:
+the reference's known-answer test, committed dense-formulation fixtures, the dense and
+scipy.sparse formulations on the reference's shape grid, and algebraic invariants chosen so that a
+dropped term, a wrong index or a transposed operand fails at least one of them."""
+import glob
+import json
+import os
+
+import numpy as np
+import pytest
+import scipy.sparse as sp
+
+import oracle
+from conftest import GOLDEN, REFERENCE_SHAPES, reference_law_inputs, rel_err
+
+SMALL_SHAPES = [s for s in REFERENCE_SHAPES if s[2] < 1_000_000]
+
+
+def test_known_answer_forward_exact():
+    # testing/test.cpp:13-47: exact equality, both layouts
+    with open(os.path.join(GOLDEN, "kat_forward.json")) as f:
+        kat = json.load(f)
+    x = np.array(kat["features"], dtype=np.float32)
+    lookup = np.array(kat["lookup"], dtype=np.int32)
+    w = np.array(kat["weights"], dtype=np.float32)
+    expected = np.array(kat["expected"], dtype=np.float32)
+    assert np.array_equal(oracle.forward(x, lookup, w), expected)
+    assert np.array_equal(oracle.forward(np.ascontiguousarray(x.T), lookup, w, transposed=True), expected)
+    assert np.array_equal(oracle.forward(x, lookup.astype(np.uint32), w), expected)
+
+
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "dense_*.npz"))))
+@pytest.mark.parametrize("transposed", [False, True])
+def test_golden_dense_fixtures(path, transposed):
+    z = np.load(path)
+    x, lookup, w, g = z["features"], z["lookup"], z["weights"], z["out_grad"]
+    xin = np.ascontiguousarray(x.T) if transposed else x
+    out = oracle.forward(xin, lookup, w, transposed=transposed)
+    gx, gw = oracle.backward(xin, lookup, w, g, transposed=transposed)
+    if transposed:
+        gx = gx.T
+    # the reference's own absolute gates (test_case_templates.h:82,139-140), two-sided here
+    assert np.abs(out - z["result"]).max() < 1e-5
+    assert np.abs(gx - z["feature_grad"]).max() < 1.5e-5
+    assert np.abs(gw - z["weight_grad"]).max() < 1.5e-5
+
+
+@pytest.mark.parametrize("shape", SMALL_SHAPES)
+@pytest.mark.parametrize("transposed", [False, True])
+def test_against_dense_formulation(shape, transposed):
+    # reference.cpp:15-82 restated in numpy float64; inputs follow the reference tests' law
+    B, N, L, K = shape
+    x, lookup, w, g = reference_law_inputs(B, N, L, K)
+    xin = np.ascontiguousarray(x.T) if transposed else x
+    out = oracle.forward(xin, lookup, w, transposed=transposed)
+    gx, gw = oracle.backward(xin, lookup, w, g, transposed=transposed)
+    d_out = oracle.dense_forward(xin, lookup, w, transposed=transposed)
+    d_gx, d_gw = oracle.dense_backward(xin, lookup, w, g, transposed=transposed)
+    assert out.shape == (B, L) and gx.shape == xin.shape and gw.shape == (L, K)
+    assert np.abs(out - d_out).max() < 1e-5
+    assert np.abs(gx - d_gx).max() < 1.5e-5
+    assert np.abs(gw - d_gw).max() < 1.5e-5
+
+
+def test_huge_label_count_against_scipy_sparse():
+    # (1, 32, 4_000_000, 4) of the reference grid; D is too big to hold densely, so the check is
+    # the CSR product of scipy.sparse, an independent library routine
+    B, N, L, K = REFERENCE_SHAPES[-1]
+    x, lookup, w, g = reference_law_inputs(B, N, L, K)
+    S = sp.csr_matrix((w.reshape(-1).astype(np.float64), lookup.reshape(-1), np.arange(0, L * K + 1, K)), shape=(L, N))
+    out = oracle.forward(x, lookup, w)
+    assert np.abs(out - (S @ x.astype(np.float64).T).T).max() < 1e-5
+    gx = oracle.input_grad(x, lookup, w, g)
+    ref_gx = (S.T @ g.astype(np.float64).T).T
+    assert rel_err(gx, ref_gx) < 1e-4          # about 250k terms per column: relative gate
+    gw = oracle.weight_grad(x, lookup, w, g)
+    ref_gw = x.astype(np.float64)[0][lookup] * g.astype(np.float64)[0][:, None]
+    assert np.abs(gw - ref_gw).max() < 1.5e-5
+
+
+@pytest.mark.parametrize("shape", [(17, 12, 63, 44), (127, 254, 513, 73)])
+def test_f64_variants_agree_with_dense(shape):
+    B, N, L, K = shape
+    x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=7)
+    d_out = oracle.dense_forward(x, lookup, w)
+    d_gx, d_gw = oracle.dense_backward(x, lookup, w, g)
+    assert np.allclose(oracle.forward(x, lookup, w, f64=True), d_out, rtol=0, atol=1e-12)
+    assert np.allclose(oracle.input_grad(x, lookup, w, g, f64=True), d_gx, rtol=0, atol=1e-12)
+    assert np.allclose(oracle.weight_grad(x, lookup, w, g, f64=True), d_gw, rtol=0, atol=1e-12)
+
+
+def test_adjoint_identity():
+    # the layer is linear in x and in W:  <out, g> = <x, gx> = <W, gW>
+    B, N, L, K = 33, 100, 257, 19
+    x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=3)
+    out = oracle.forward(x, lookup, w).astype(np.float64)
+    gx, gw = oracle.backward(x, lookup, w, g)
+    a = float((out * g).sum())
+    b = float((x.astype(np.float64) * gx).sum())
+    c = float((w.astype(np.float64) * gw).sum())
+    assert abs(a - b) < 1e-4 * abs(a) and abs(a - c) < 1e-4 * abs(a)
+
+
+def test_layouts_agree_bitwise():
+    # testing/test.cpp:91-166: [B,N] and [N,B] feature layouts give the same numbers
+    B, N, L, K = 12, 8, 32, 16
+    x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=5)
+    xt = np.ascontiguousarray(x.T)
+    assert np.array_equal(oracle.forward(x, lookup, w), oracle.forward(xt, lookup, w, transposed=True))
+    gx, gw = oracle.backward(x, lookup, w, g)
+    gxt, gwt = oracle.backward(xt, lookup, w, g, transposed=True)
+    assert np.array_equal(gx, gxt.T) and np.array_equal(gw, gwt)
+
+
+def test_duplicates_and_untouched_columns():
+    # duplicates inside a row accumulate (reference.cpp:19-25) and each copy gets the full weight
+    # gradient; columns no connection points at receive exactly zero input gradient
+    x = np.arange(1, 13, dtype=np.float32).reshape(2, 6)
+    lookup = np.array([[1, 1, 3], [0, 3, 3]], dtype=np.int32)       # columns 2, 4, 5 untouched
+    w = np.array([[1.0, 2.0, 4.0], [8.0, 16.0, 32.0]], dtype=np.float32)
+    g = np.array([[1.0, 10.0], [100.0, 1000.0]], dtype=np.float32)
+    out = oracle.forward(x, lookup, w)
+    assert np.array_equal(out, np.array([[3 * 2 + 4 * 4, 8 * 1 + 48 * 4], [3 * 8 + 4 * 10, 8 * 7 + 48 * 10]], dtype=np.float32))
+    gx, gw = oracle.backward(x, lookup, w, g)
+    assert np.array_equal(gx[:, [2, 4, 5]], np.zeros((2, 3), dtype=np.float32))
+    assert np.array_equal(gx[:, 1], np.array([3.0, 300.0], dtype=np.float32))
+    assert np.array_equal(gx[:, 3], np.array([4 * 1 + 48 * 10, 4 * 100 + 48 * 1000], dtype=np.float32))
+    assert np.array_equal(gx[:, 0], np.array([80.0, 8000.0], dtype=np.float32))
+    assert gw[0, 0] == gw[0, 1] == 2 * 1 + 8 * 100
+    assert gw[1, 1] == gw[1, 2] == 4 * 10 + 10 * 1000
+
+
+def test_identity_lookup_reduces_to_column_scaling():
+    # K = 1 and lookup[j] = j: out = x * w^T column-wise, gx = g * w^T, gw = sum_b x*g
+    B, N = 5, 9
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((B, N)).astype(np.float32)
+    w = rng.standard_normal((N, 1)).astype(np.float32)
+    g = rng.standard_normal((B, N)).astype(np.float32)
+    lookup = np.arange(N, dtype=np.int32).reshape(N, 1)
+    assert np.array_equal(oracle.forward(x, lookup, w), x * w.T)
+    gx, gw = oracle.backward(x, lookup, w, g)
+    assert np.array_equal(gx, g * w.T)
+    assert np.allclose(gw[:, 0], (x.astype(np.float64) * g).sum(0), rtol=1e-6, atol=1e-6)
+
+
+def test_permuting_a_row_only_reorders():
+    B, N, L, K = 9, 40, 21, 12
+    x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=9)
+    perm = np.random.default_rng(1).permutation(K)
+    out = oracle.forward(x, lookup, w)
+    out_p = oracle.forward(x, lookup[:, perm], w[:, perm])
+    assert np.abs(out - out_p).max() < 1e-5
+    gx, gw = oracle.backward(x, lookup, w, g)
+    gx_p, gw_p = oracle.backward(x, lookup[:, perm], w[:, perm], g)
+    assert np.abs(gx - gx_p).max() < 1.5e-5
+    assert np.array_equal(gw[:, perm], gw_p)      # each weight gradient is its own b-ordered sum
+
+
+def test_thread_count_does_not_change_results():
+    B, N, L, K = 16, 64, 1000, 8
+    x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=13)
+    one = (oracle.forward(x, lookup, w, threads=1),) + oracle.backward(x, lookup, w, g, threads=1)
+    many = (oracle.forward(x, lookup, w, threads=7),) + oracle.backward(x, lookup, w, g, threads=7)
+    for a, b in zip(one, many):
+        assert np.array_equal(a, b)
+
+
+def test_forward_accumulation_order_matches_reference_loop():
+    # forward.cpp:29-41: four strided partial sums over the 4-aligned part, tail into the first,
+    # then v0+v1+v2+v3.  Restated here in numpy float32 (no FMA), so agreement is to rounding only;
+    # magnitudes chosen so that a different association (e.g. one running sum) shows.
+    K = 11
+    x = np.array([[1e8, 1.0, -1e8, 1.0, 3.0, 1.0, 1.0, 1.0, 1.0, 1.0, 1.0]], dtype=np.float32)
+    lookup = np.arange(K, dtype=np.int32).reshape(1, K)
+    w = np.ones((1, K), dtype=np.float32)
+    v = np.zeros(4, dtype=np.float32)
+    for i in range(0, 8, 4):
+        for q in range(4):
+            v[q] = np.float32(v[q] + x[0, i + q] * w[0, i + q])
+    for i in range(8, K):
+        v[0] = np.float32(v[0] + x[0, i] * w[0, i])
+    expected = np.float32(np.float32(np.float32(v[0] + v[1]) + v[2]) + v[3])
+    assert oracle.forward(x, lookup, w)[0, 0] == expected
+    assert expected != np.float32(np.cumsum((x[0] * w[0]).astype(np.float32), dtype=np.float32)[-1])
+
+
+def test_bf16_rounding_closed_form():
+    vals = np.array([1.0, 1.00390625, 1.005859375, 1.001953125, -3.1415927, 0.0, 65504.0, 1e-40], dtype=np.float32)
+    r = oracle.round_bf16(vals)
+    # RNE on the top 16 bits: 1+2^-8 is a tie -> even (1.0); 1+3*2^-9 rounds up to 1+2^-7
+    assert r[0] == 1.0 and r[1] == 1.0 and r[2] == np.float32(1.0078125) and r[3] == 1.0
+    assert (r.view(np.uint32) & 0xFFFF == 0).all()
+    assert np.all(np.abs(r[:7] - vals[:7]) <= np.abs(vals[:7]) * 2.0 ** -8)
+
+
+def test_topk_matches_sort_with_lower_index_first():
+    rng = np.random.default_rng(2)
+    s = rng.integers(0, 20, (7, 300)).astype(np.float32)          # many ties
+    values, indices = oracle.topk(s, 5)
+    for b in range(s.shape[0]):
+        order = np.lexsort((np.arange(s.shape[1]), -s[b]))[:5]
+        assert np.array_equal(indices[b], order)
+        assert np.array_equal(values[b], s[b, order])
