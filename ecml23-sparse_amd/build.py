@@ -23,6 +23,7 @@ SOURCES = [
     "ffi_weight_grad.hip",
     "ffi_input_grad.hip",
     "ffi_plan.hip",
+    "ffi_util.hip",
 ]
 
 # gfx950 only.  Packed-fp32 VALU forms are switched off for all device code.

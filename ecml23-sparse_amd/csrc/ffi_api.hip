@@ -223,6 +223,7 @@ int ffi_cache_clear(void) {
             ++i;
         }
     }
+    workspace_clear(dev);
     return FFI_OK;
 }
 
@@ -233,7 +234,7 @@ size_t ffi_cache_bytes(void) {
     size_t total = 0;
     for (ffi_plan* p : g_cache)
         if (p->device == dev) total += p->bytes;
-    return total;
+    return total + workspace_bytes(dev);
 }
 
 int ffi_check_lookup(const int32_t* lookup, int64_t num_units, int64_t fan_in, int64_t num_features,

@@ -34,6 +34,17 @@ int hip_fail(hipError_t e);
         if (s__ != FFI_OK) return s__; \
     } while (0)
 
+// Library-owned device scratch, one buffer per (device, stream, slot), grown on demand and kept.
+// Work that uses a buffer is ordered by the stream it belongs to.
+enum WorkspaceSlot { kWsFeaturesT = 0, kWsPartials = 1, kWsSlots = 2 };
+int workspace_get(hipStream_t s, int slot, size_t bytes, void** out);
+void workspace_clear(int device);
+size_t workspace_bytes(int device);
+int device_cu_count();
+
+// dst[c][r] = src[r][c] for a row-major [rows, cols] matrix.
+int launch_transpose(const float* src, float* dst, int rows, int cols, hipStream_t s);
+
 // ---- launchers (each validates nothing; callers pass validated Dims) ---------------------------
 int launch_forward(const float* x, const int32_t* idx, const float* w, float* out, const Dims& d,
                    hipStream_t s);
