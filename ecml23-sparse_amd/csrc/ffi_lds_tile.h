@@ -42,15 +42,42 @@ __device__ __forceinline__ int xcd_contiguous_block(int block, int nblocks) {
     return (nblocks & 7) == 0 ? (block & 7) * (nblocks >> 3) + (block >> 3) : block;
 }
 
-// xs[r][c] = src[r*ld + c0 + c] for c < 32 (zero beyond `ncols`), r < rows.  src rows are read in
-// 128-byte pieces, LDS writes are conflict-free.
+// xs[r][c] = src[r*ld + c0 + c] for c < 32 (zero beyond column `ld`), r < rows.  src rows are read
+// in 128-byte pieces, LDS writes are conflict-free.
 __device__ __forceinline__ void stage_rows32(float* __restrict__ xs, const float* __restrict__ src, int rows,
                                              int ld, int c0) {
-    const int total = rows * kTileBatch;
-    for (int t = threadIdx.x; t < total; t += kTileThreads) {
-        const int r = t >> 5, c = t & 31;
-        xs[t] = (c0 + c < ld) ? src[(size_t)r * ld + c0 + c] : 0.f;
-    }
+    const int c = threadIdx.x & 31;
+    const bool in = c0 + c < ld;
+    const float* p = src + c0 + c;
+#pragma unroll 4
+    for (int r = threadIdx.x >> 5; r < rows; r += kTileThreads / 32)
+        xs[r * kTileBatch + c] = in ? p[(size_t)r * ld] : 0.f;
+}
+
+// Raw buffer resource over `bytes` bytes at p (gfx9 family: 32-bit data format word).  Loads
+// through it take a per-lane byte offset plus a wave-uniform (scalar) byte offset, and reads
+// beyond `bytes` return zero instead of faulting.
+using buffer_rsrc = __amdgpu_buffer_rsrc_t;
+__device__ __forceinline__ buffer_rsrc make_rsrc(const void* p, size_t bytes) {
+    const unsigned n = bytes > 0xfffffffeull ? 0xfffffffeu : (unsigned)bytes;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, n, 0x00020000);
+}
+__device__ __forceinline__ float buffer_load_f32(buffer_rsrc r, unsigned lane_off, unsigned wave_off) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, lane_off, wave_off, 0));
+}
+
+// v[b] = m[(b0+b)*ld + col] for b < 32 (zero beyond `rows`); rows of m are reached through the
+// scalar offset, `col` is the only per-lane address register.  m + b0*ld is rebased in 64 bits,
+// the remaining offsets (< 32*ld*4) must fit 32 bits: callers guarantee ld < 2^25.
+__device__ __forceinline__ void load_rows32(const float* __restrict__ m, int ld, int b0, int rows, unsigned col,
+                                            float (&v)[32]) {
+    const float* base = m + (size_t)b0 * (size_t)ld;
+    const int nrows = min(32, rows - b0);
+    const buffer_rsrc r = make_rsrc(base, (size_t)nrows * (size_t)ld * sizeof(float));
+    const unsigned lane_off = col * 4u;
+    const unsigned stride = (unsigned)ld * 4u;
+#pragma unroll
+    for (int b = 0; b < 32; ++b) v[b] = buffer_load_f32(r, lane_off, (unsigned)b * stride);
 }
 
 // Loads connections k0..k0+7 of one row: weights as they are, column ids scaled to LDS row byte
@@ -76,6 +103,37 @@ __device__ __forceinline__ void load_chunk8(const float* __restrict__ wrow, cons
         }
     }
 }
+
+// ---- lane-per-row gathers -------------------------------------------------------------------------
+// When every lane reads its OWN 128-byte row (row ids unrelated between lanes), bank conflicts are
+// avoided by skewing the order in which a lane walks the eight 16-byte chunks of its row: at step
+// c lane l reads chunk c ^ (l & 7).  Rows are 128-byte aligned, so the bank group depends on the
+// chunk number only and any eight consecutive lanes hit eight different bank groups.
+// Consequence: register group c of lane l holds batch entries 4*(c ^ (l&7)) .. +3.
+
+__device__ __forceinline__ void cond_swap(bool p, float& a, float& b) {
+    const float t = p ? b : a;
+    b = p ? a : b;
+    a = t;
+}
+
+// v[4c+i] <-> v[4(c ^ r)+i] for r in [0,8): its own inverse; three stages of conditional swaps.
+__device__ __forceinline__ void xor_permute_groups(float (&v)[32], int r) {
+    const bool b4 = r & 4, b2 = r & 2, b1 = r & 1;
+#pragma unroll
+    for (int e = 0; e < 32; ++e)
+        if (!(e & 16)) cond_swap(b4, v[e], v[e + 16]);
+#pragma unroll
+    for (int e = 0; e < 32; ++e)
+        if (!(e & 8)) cond_swap(b2, v[e], v[e + 8]);
+#pragma unroll
+    for (int e = 0; e < 32; ++e)
+        if (!(e & 4)) cond_swap(b1, v[e], v[e + 4]);
+}
+
+// Byte address (inside the tile) of the chunk read at step C, given base = row*128 | (lane&7)*16.
+template <int C>
+__device__ __forceinline__ unsigned skew_addr(unsigned base) { return C == 0 ? base : (base ^ (unsigned)(C * 16)); }
 
 #endif  // __HIPCC__
 
