@@ -37,10 +37,8 @@ int plan_alloc(int L, int K, int N, ffi_plan** out) {
     if (!p) return FFI_ERR_OUT_OF_MEMORY;
     if (hipGetDevice(&p->device) != hipSuccess) { delete p; return FFI_ERR_NO_DEVICE; }
     p->L = L; p->K = K; p->N = N;
-    const size_t total = (size_t)L * K;
-    bool ok = hipMalloc(&p->perm, total * sizeof(int32_t)) == hipSuccess &&
-              hipMalloc(&p->col_ptr, ((size_t)N + 1) * sizeof(int32_t)) == hipSuccess &&
-              hipMalloc(&p->d_scratch, 8 * sizeof(unsigned long long)) == hipSuccess &&
+    // the plan arrays themselves are sized and allocated by plan_build
+    bool ok = hipMalloc(&p->d_scratch, 8 * sizeof(unsigned long long)) == hipSuccess &&
               hipHostMalloc(&p->h_scratch, 8 * sizeof(unsigned long long)) == hipSuccess;
     if (!ok) {
         (void)hipGetLastError();
@@ -48,7 +46,6 @@ int plan_alloc(int L, int K, int N, ffi_plan** out) {
         delete p;
         return FFI_ERR_OUT_OF_MEMORY;
     }
-    p->bytes = total * sizeof(int32_t) + ((size_t)N + 1) * sizeof(int32_t) + 64;
     *out = p;
     return FFI_OK;
 }

@@ -1,11 +1,136 @@
 // Input gradient of the fixed-fan-in sparse layer for gfx950, atomics-free:
 //   gx[b,n] = sum over (j,k) with idx[j,k]==n of w[j,k] * g[b,j]
 // (semantics of tfsparse/cc/kernels/backward.cpp:39-73 in the reference).
+//
+// Narrow inputs use the tiled plan: it is the forward pass of the transposed sparse matrix, done
+// tile by tile.  A workgroup keeps gs[label in tile][32 batch rows] in LDS, thread n owns input
+// column n and walks the tile's connections of that column, gathering whole 128-byte rows of gs
+// (chunk order skewed per lane, see ffi_lds_tile.h) into 32 accumulators that live in registers
+// across all the tiles of the workgroup's label stream.  Streams are then summed in a fixed order.
 #include "ffi_internal.h"
+#include "ffi_lds_tile.h"
+
+#include <algorithm>
 
 namespace ffi {
 namespace {
 
+// ---- tiled plan ---------------------------------------------------------------------------------
+
+// wp[slot] = w at the connection stored in that slot (0 in padding slots): brings the weights into
+// the plan's slot order so that the main kernel reads them coalesced.  One workgroup per tile.
+__global__ void igrad_permute_weights_kernel(const unsigned* __restrict__ ent, const unsigned* __restrict__ slice_off,
+                                             const unsigned short* __restrict__ col_len, const float* __restrict__ w,
+                                             float* __restrict__ wp, int K, int tile_labels) {
+    const int t = blockIdx.x, nthreads = blockDim.x;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const size_t sl = (size_t)t * (nthreads >> 6) + wave;
+    const unsigned row0 = slice_off[sl], rows = slice_off[sl + 1] - row0;
+    const unsigned len = col_len[(size_t)t * nthreads + threadIdx.x];
+    const float* wt = w + (size_t)t * tile_labels * K;
+    for (unsigned i = 0; i < rows; ++i) {
+        const size_t slot = ((size_t)row0 + i) * 64 + lane;
+        wp[slot] = (i < len) ? wt[ent[slot] >> 10] : 0.f;
+    }
+}
+
+template <int C>
+__device__ __forceinline__ void igrad_step(const char* __restrict__ gs_bytes, unsigned base, float wv, float (&acc)[32]) {
+    const float4 v = *reinterpret_cast<const float4*>(gs_bytes + skew_addr<C>(base));
+    acc[4 * C + 0] = fmaf(wv, v.x, acc[4 * C + 0]);
+    acc[4 * C + 1] = fmaf(wv, v.y, acc[4 * C + 1]);
+    acc[4 * C + 2] = fmaf(wv, v.z, acc[4 * C + 2]);
+    acc[4 * C + 3] = fmaf(wv, v.w, acc[4 * C + 3]);
+}
+
+__device__ __forceinline__ void igrad_entry(const char* __restrict__ gs_bytes, unsigned e, float wv, unsigned skew,
+                                            float (&acc)[32]) {
+    const unsigned base = ((e & 1023u) << 7) | skew;
+    igrad_step<0>(gs_bytes, base, wv, acc); igrad_step<1>(gs_bytes, base, wv, acc);
+    igrad_step<2>(gs_bytes, base, wv, acc); igrad_step<3>(gs_bytes, base, wv, acc);
+    igrad_step<4>(gs_bytes, base, wv, acc); igrad_step<5>(gs_bytes, base, wv, acc);
+    igrad_step<6>(gs_bytes, base, wv, acc); igrad_step<7>(gs_bytes, base, wv, acc);
+}
+
+// partial[stream][n][b] over the stream's tiles.  grid = streams * batch tiles.
+__global__ __launch_bounds__(1024) void igrad_tile_kernel(const unsigned* __restrict__ ent, const float* __restrict__ wp,
+                                  const unsigned* __restrict__ slice_off, const unsigned short* __restrict__ col_len,
+                                  const float* __restrict__ g, float* __restrict__ partial, int B, int L,
+                                  int tile_labels, int tiles, int tiles_per_stream, int nbt) {
+    extern __shared__ __align__(16) float gs[];
+    char* gs_bytes = reinterpret_cast<char*>(gs);
+    const int nthreads = blockDim.x;
+    const int u = xcd_contiguous_block(blockIdx.x, gridDim.x);
+    const int bt = u % nbt, stream = u / nbt;
+    const int b0 = bt * kTileBatch;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const unsigned skew = (unsigned)(lane & 7) * 16u;
+    const int t_begin = stream * tiles_per_stream, t_end = min(t_begin + tiles_per_stream, tiles);
+
+    float acc[32];
+#pragma unroll
+    for (int i = 0; i < 32; ++i) acc[i] = 0.f;
+
+    for (int t = t_begin; t < t_end; ++t) {
+        const int j0 = t * tile_labels;
+        const int nl = min(tile_labels, L - j0);
+        __syncthreads();                       // the previous tile is no longer being read
+        // stage gs[jl][c] = g[b0+c][j0+jl]: coalesced loads along labels, then 16-byte LDS writes
+        // whose chunk order is skewed by the label id (no bank conflicts)
+        for (int jl = threadIdx.x; jl < nl; jl += nthreads) {
+            float gb[32];
+            load_rows32(g, L, b0, B, (unsigned)(j0 + jl), gb);
+            const int r = jl & 7;
+            xor_permute_groups(gb, r);
+            char* rowp = gs_bytes + ((unsigned)jl << 7);
+#pragma unroll
+            for (int c = 0; c < 8; ++c)
+                *reinterpret_cast<float4*>(rowp + ((c ^ r) << 4)) = make_float4(gb[4 * c], gb[4 * c + 1], gb[4 * c + 2], gb[4 * c + 3]);
+        }
+        __syncthreads();
+        const size_t sl = (size_t)t * (nthreads >> 6) + wave;
+        const unsigned row0 = __builtin_amdgcn_readfirstlane(slice_off[sl]);
+        const unsigned rows = __builtin_amdgcn_readfirstlane(slice_off[sl + 1]) - row0;
+        const unsigned len = col_len[(size_t)t * nthreads + threadIdx.x];
+        const unsigned* ep = ent + (size_t)row0 * 64 + lane;
+        const float* wpp = wp + (size_t)row0 * 64 + lane;
+        unsigned i = 0;
+        for (; i + 4 <= rows; i += 4) {
+            unsigned e4[4];
+            float w4[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) { e4[q] = ep[(size_t)(i + q) * 64]; w4[q] = wpp[(size_t)(i + q) * 64]; }
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                if (i + q < len) igrad_entry(gs_bytes, e4[q], w4[q], skew, acc);
+        }
+        for (; i < rows; ++i) {
+            const unsigned e = ep[(size_t)i * 64];
+            const float wv = wpp[(size_t)i * 64];
+            if (i < len) igrad_entry(gs_bytes, e, wv, skew, acc);
+        }
+    }
+    // back to natural batch order, then one 128-byte row per thread
+    xor_permute_groups(acc, lane & 7);
+    float* out = partial + ((size_t)stream * nthreads + threadIdx.x) * ((size_t)nbt * kTileBatch) + b0;
+#pragma unroll
+    for (int c = 0; c < 8; ++c)
+        *reinterpret_cast<float4*>(out + 4 * c) = make_float4(acc[4 * c], acc[4 * c + 1], acc[4 * c + 2], acc[4 * c + 3]);
+}
+
+// gx = sum over streams, ascending: a fixed order, so results are reproducible.
+template <bool TP>
+__global__ __launch_bounds__(256) void igrad_reduce_kernel(const float* __restrict__ partial, float* __restrict__ gx,
+                                                           int B, int N, int streams, int nthreads, int bpad) {
+    const int b = blockIdx.x * 256 + threadIdx.x;
+    const int n = blockIdx.y;
+    if (b >= B) return;
+    float v = 0.f;
+    for (int r = 0; r < streams; ++r) v += partial[((size_t)r * nthreads + n) * bpad + b];
+    if (TP) gx[(size_t)n * B + b] = v; else gx[(size_t)b * N + n] = v;
+}
+
+// ---- global plan --------------------------------------------------------------------------------
 constexpr int kIgBlock = 256;
 constexpr int kIgBatch = 4;
 
@@ -51,10 +176,38 @@ __global__ __launch_bounds__(kIgBlock) void igrad_column_block(const int32_t* __
     }
 }
 
+int launch_tiled(const ffi_plan* p, const float* w, const float* g, float* gx, int B, bool tp, hipStream_t s) {
+    const int nbt = (B + kTileBatch - 1) / kTileBatch;
+    const int cus = device_cu_count();
+    int streams = std::max(1, std::min(p->tiles, cus / std::max(1, nbt)));
+    const int tps = (p->tiles + streams - 1) / streams;
+    streams = (p->tiles + tps - 1) / tps;
+    const int bpad = nbt * kTileBatch;
+    const size_t slots = (size_t)p->total_rows * 64;
+    float* wp = nullptr;
+    float* partial = nullptr;
+    FFI_TRY(workspace_get(s, kWsFeaturesT, std::max<size_t>(slots, 1) * sizeof(float), (void**)&wp));
+    FFI_TRY(workspace_get(s, kWsPartials, (size_t)streams * p->threads * bpad * sizeof(float), (void**)&partial));
+    hipLaunchKernelGGL(igrad_permute_weights_kernel, dim3(p->tiles), dim3(p->threads), 0, s, p->ent, p->slice_off,
+                       p->col_len, w, wp, p->K, p->tile_labels);
+    const size_t lds = tile_lds_bytes(p->tile_labels);
+    FFI_HIP_TRY(hipFuncSetAttribute((const void*)igrad_tile_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(igrad_tile_kernel, dim3(streams * nbt), dim3(p->threads), lds, s, p->ent, wp, p->slice_off,
+                       p->col_len, g, partial, B, p->L, p->tile_labels, p->tiles, tps, nbt);
+    dim3 rgrid((B + 255) / 256, p->N);
+    if (tp)
+        hipLaunchKernelGGL(igrad_reduce_kernel<true>, rgrid, dim3(256), 0, s, partial, gx, B, p->N, streams, p->threads, bpad);
+    else
+        hipLaunchKernelGGL(igrad_reduce_kernel<false>, rgrid, dim3(256), 0, s, partial, gx, B, p->N, streams, p->threads, bpad);
+    FFI_HIP_TRY(hipGetLastError());
+    return FFI_OK;
+}
+
 }  // namespace
 
 int launch_input_grad(const ffi_plan* p, const float* w, const float* g, float* gx, int B, bool tp,
                       hipStream_t s) {
+    if (p->tiled) return launch_tiled(p, w, g, gx, B, tp, s);
     dim3 grid(p->N, (B + kIgBatch - 1) / kIgBatch);
     if (grid.y > 65535u) return FFI_ERR_TOO_LARGE;
     if (tp)

@@ -53,22 +53,42 @@ int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float
 
 }  // namespace ffi
 
-// Column-ordered ("CSC") view of one lookup matrix.
+// Column-ordered view of one lookup matrix, in one of two forms.
+//
+// tiled == true (narrow inputs): labels are cut into tiles of `tile_labels`; inside a tile the
+// connections are grouped by column, and the columns into slices of 64 (one per wavefront).  A
+// slice is stored slot-major: row i of the slice holds the i-th connection of each of its 64
+// columns (so a wavefront reads 256 contiguous bytes per step), padded to the longest column of
+// the slice.  Inside a column the connections are in ascending flat position, the order the
+// reference's CPU kernel accumulates in (tfsparse/cc/kernels/backward.cpp:64-72).
+//
+// tiled == false (any shape): a global CSC, perm[e] = flat position of the e-th connection in
+// (column, position) order, col_ptr[n]..col_ptr[n+1] the connections of column n.
 struct ffi_plan {
     int device = -1;
     int L = 0, K = 0, N = 0;
     const int32_t* lookup = nullptr;  // the buffer this plan was built from (cache key)
     unsigned long long fingerprint = 0;
-    // perm[e]: flat position j*K+k of the e-th entry in (column, position) order;
-    // col_ptr[n]..col_ptr[n+1]: the entries of column n.
+    bool tiled = false;
+    // tiled form
+    int tile_labels = 0;      // labels per tile (<= 1024)
+    int threads = 0;          // workgroup size of the kernels walking the plan: N rounded up to 64
+    int slices = 0;           // threads / 64
+    int tiles = 0;            // ceil(L / tile_labels)
+    long long total_rows = 0; // rows of 64 entries over all slices
+    unsigned* slice_off = nullptr;       // [tiles*slices + 1] first row of each slice
+    unsigned short* col_len = nullptr;   // [tiles][threads] connections of each column in each tile
+    unsigned* ent = nullptr;             // [total_rows*64]  (local position << 10) | local label
+    // global form
     int32_t* perm = nullptr;
     int32_t* col_ptr = nullptr;
-    unsigned long long* d_scratch = nullptr;  // fingerprint / flags (device)
+    unsigned long long* d_scratch = nullptr;  // fingerprint / counters (device)
     unsigned long long* h_scratch = nullptr;  // pinned mirror
     size_t bytes = 0;
 };
 
 namespace ffi {
+constexpr int kPlanTileLabels = 1024;     // local label ids fit 10 bits, a [1024][32] fp32 tile fits LDS
 int plan_build(ffi_plan* p, const int32_t* lookup, hipStream_t s);
 int plan_fingerprint(ffi_plan* p, const int32_t* lookup, hipStream_t s, unsigned long long* out,
                      unsigned long long* bad_ids);

@@ -1,9 +1,8 @@
 // Column-ordered view ("plan") of a lookup matrix, built on the device.
 //
 // The input gradient sums, for every input column n, over all connections (j,k) with
-// lookup[j,k] == n.  The plan lists those connections column by column, in ascending flat position
-// j*K+k inside a column, which is the order the reference's CPU kernel accumulates in
-// (tfsparse/cc/kernels/backward.cpp:64-72); walking it sequentially needs no atomics.
+// lookup[j,k] == n.  The plan lists those connections column by column so that they can be walked
+// sequentially, without atomics, in an order that never changes from run to run.
 #include "ffi_internal.h"
 
 #include <algorithm>
@@ -51,6 +50,85 @@ __global__ __launch_bounds__(kBlock) void zero_u64_kernel(unsigned long long* p,
     if (i < n) p[i] = 0;
 }
 
+// ---- tiled form ---------------------------------------------------------------------------------
+
+// One workgroup per label tile, one thread per column.  Counts the tile's connections per column
+// (integer LDS atomics: order-independent), stores them, and the longest column of each slice.
+__global__ void tile_count_kernel(const int32_t* __restrict__ idx, int L, int K, int tile_labels,
+                                  unsigned short* __restrict__ col_len, unsigned* __restrict__ slice_len) {
+    extern __shared__ unsigned cnt[];
+    const int t = blockIdx.x, nthreads = blockDim.x;
+    cnt[threadIdx.x] = 0;
+    __syncthreads();
+    const int j0 = t * tile_labels;
+    const int nl = min(tile_labels, L - j0);
+    const int* src = idx + (size_t)j0 * K;
+    const int total = nl * K;
+    for (int e = threadIdx.x; e < total; e += nthreads) atomicAdd(&cnt[(unsigned)src[e]], 1u);
+    __syncthreads();
+    unsigned c = cnt[threadIdx.x];
+    col_len[(size_t)t * nthreads + threadIdx.x] = (unsigned short)c;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) c = max(c, (unsigned)__shfl_xor((int)c, off));
+    if ((threadIdx.x & 63) == 0) slice_len[(size_t)t * (nthreads >> 6) + (threadIdx.x >> 6)] = c;
+}
+
+// Exclusive prefix sum of n values into off[0..n] by one workgroup (n is a few thousand).
+__global__ __launch_bounds__(1024) void slice_scan_kernel(const unsigned* __restrict__ len, unsigned* __restrict__ off,
+                                                           int n, unsigned long long* __restrict__ total_out) {
+    __shared__ unsigned long long part[1024];
+    const int per = (n + 1023) / 1024;
+    const int b = threadIdx.x * per, e = min(b + per, n);
+    unsigned long long sum = 0;
+    for (int i = b; i < e; ++i) sum += len[i];
+    part[threadIdx.x] = sum;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned long long run = 0;
+        for (int i = 0; i < 1024; ++i) { const unsigned long long v = part[i]; part[i] = run; run += v; }
+        *total_out = run;
+    }
+    __syncthreads();
+    unsigned long long run = part[threadIdx.x];
+    for (int i = b; i < e; ++i) { off[i] = (unsigned)run; run += len[i]; }
+    if (threadIdx.x == 1023) off[n] = (unsigned)(part[1023] + sum);
+}
+
+// One workgroup per label tile, one thread per column n.  The tile's column ids pass through LDS
+// in chunks; every thread scans them in flat-position order and appends the ones equal to its
+// column, so the connections of a column end up in ascending position: deterministic and stable
+// without any sort.  ent = (position inside the tile << 10) | label inside the tile.
+constexpr int kFillChunk = 8192;
+__global__ void tile_fill_kernel(const int32_t* __restrict__ idx, int L, int K, int tile_labels,
+                                 const unsigned* __restrict__ slice_off, unsigned* __restrict__ ent) {
+    __shared__ __align__(16) int keys[kFillChunk];
+    const int t = blockIdx.x, nthreads = blockDim.x;
+    const int j0 = t * tile_labels;
+    const int nl = min(tile_labels, L - j0);
+    const int* src = idx + (size_t)j0 * K;
+    const int total = nl * K;
+    const int mine = threadIdx.x;
+    const size_t row0 = slice_off[(size_t)t * (nthreads >> 6) + (threadIdx.x >> 6)];
+    unsigned* dst = ent + row0 * 64 + (threadIdx.x & 63);
+    unsigned count = 0;
+    int label = 0, kk = 0;       // label and connection slot of the entry under the cursor
+    for (int c0 = 0; c0 < total; c0 += kFillChunk) {
+        const int n = min(kFillChunk, total - c0);
+        __syncthreads();
+        for (int e = threadIdx.x; e < n; e += nthreads) keys[e] = src[c0 + e];
+        __syncthreads();
+        for (int e = 0; e < n; ++e) {
+            if (keys[e] == mine) {
+                dst[(size_t)count * 64] = ((unsigned)(c0 + e) << 10) | (unsigned)label;
+                ++count;
+            }
+            if (++kk == K) { kk = 0; ++label; }
+        }
+    }
+}
+
+// ---- global form --------------------------------------------------------------------------------
+
 // col_ptr[n] = first position in the sorted key array whose key is >= n (n in [0,N]).
 __global__ __launch_bounds__(kBlock) void col_ptr_kernel(const unsigned* __restrict__ sorted_keys,
                                                           int total, int N, int32_t* __restrict__ col_ptr) {
@@ -70,28 +148,70 @@ int bits_for(unsigned max_value) {
     return b;
 }
 
-}  // namespace
+void free_arrays(ffi_plan* p) {
+    if (p->perm) (void)hipFree(p->perm);
+    if (p->col_ptr) (void)hipFree(p->col_ptr);
+    if (p->slice_off) (void)hipFree(p->slice_off);
+    if (p->col_len) (void)hipFree(p->col_len);
+    if (p->ent) (void)hipFree(p->ent);
+    p->perm = nullptr; p->col_ptr = nullptr; p->slice_off = nullptr; p->col_len = nullptr; p->ent = nullptr;
+    p->tiled = false; p->total_rows = 0; p->bytes = 0;
+}
 
-int plan_fingerprint(ffi_plan* p, const int32_t* lookup, hipStream_t s, unsigned long long* out,
-                     unsigned long long* bad_ids) {
-    const size_t total = (size_t)p->L * p->K;
-    hipLaunchKernelGGL(zero_u64_kernel, dim3(1), dim3(kBlock), 0, s, p->d_scratch, 2);
-    const unsigned blocks = (unsigned)std::min<size_t>((total + kBlock - 1) / kBlock, 2048);
-    hipLaunchKernelGGL(fingerprint_kernel, dim3(blocks), dim3(kBlock), 0, s, lookup, total, (unsigned)p->N, p->d_scratch);
-    FFI_HIP_TRY(hipGetLastError());
-    FFI_HIP_TRY(hipMemcpyAsync(p->h_scratch, p->d_scratch, 2 * sizeof(unsigned long long), hipMemcpyDeviceToHost, s));
-    FFI_HIP_TRY(hipStreamSynchronize(s));
-    *out = p->h_scratch[0];
-    *bad_ids = p->h_scratch[1];
+template <class T>
+bool dev_alloc(T** ptr, size_t count) {
+    if (hipMalloc(ptr, std::max<size_t>(count, 1) * sizeof(T)) != hipSuccess) {
+        (void)hipGetLastError();
+        *ptr = nullptr;
+        return false;
+    }
+    return true;
+}
+
+// Builds the tiled form.  Returns FFI_OK with p->tiled == false if the padded size would exceed
+// three times the connection count (heavily skewed column usage): the caller then builds the
+// global form instead.
+int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
+    const int TL = std::min(kPlanTileLabels, p->L);
+    const int threads = ((p->N + 63) / 64) * 64;
+    const int slices = threads / 64;
+    const int tiles = (p->L + TL - 1) / TL;
+    const size_t nslices = (size_t)tiles * slices;
+    unsigned* slice_len = nullptr;
+    if (!dev_alloc(&p->slice_off, nslices + 1) || !dev_alloc(&p->col_len, (size_t)tiles * threads) ||
+        !dev_alloc(&slice_len, nslices)) {
+        if (slice_len) (void)hipFree(slice_len);
+        return FFI_ERR_OUT_OF_MEMORY;
+    }
+    hipLaunchKernelGGL(tile_count_kernel, dim3(tiles), dim3(threads), threads * sizeof(unsigned), s, lookup, p->L, p->K,
+                       TL, p->col_len, slice_len);
+    hipLaunchKernelGGL(slice_scan_kernel, dim3(1), dim3(1024), 0, s, slice_len, p->slice_off, (int)nslices,
+                       p->d_scratch + 2);
+    hipError_t e = hipGetLastError();
+    if (e == hipSuccess) e = hipMemcpyAsync(p->h_scratch + 2, p->d_scratch + 2, sizeof(unsigned long long), hipMemcpyDeviceToHost, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    (void)hipFree(slice_len);
+    if (e != hipSuccess) return hip_fail(e);
+    const unsigned long long rows = p->h_scratch[2];
+    const unsigned long long connections = (unsigned long long)p->L * p->K;
+    if (rows * 64ull > 3ull * connections + 64ull * nslices || rows >= 0xffffffffull) return FFI_OK;   // too skewed
+    if (!dev_alloc(&p->ent, (size_t)rows * 64)) return FFI_ERR_OUT_OF_MEMORY;
+    e = hipMemsetAsync(p->ent, 0, std::max<size_t>((size_t)rows * 64, 1) * sizeof(unsigned), s);
+    if (e != hipSuccess) return hip_fail(e);
+    hipLaunchKernelGGL(tile_fill_kernel, dim3(tiles), dim3(threads), 0, s, lookup, p->L, p->K, TL, p->slice_off, p->ent);
+    e = hipGetLastError();
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    if (e != hipSuccess) return hip_fail(e);
+    p->tiled = true;
+    p->tile_labels = TL; p->threads = threads; p->slices = slices; p->tiles = tiles;
+    p->total_rows = (long long)rows;
+    p->bytes = (size_t)rows * 64 * sizeof(unsigned) + (nslices + 1) * sizeof(unsigned) + (size_t)tiles * threads * sizeof(unsigned short);
     return FFI_OK;
 }
 
-int plan_build(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
+int build_global(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     const int total = p->L * p->K;  // validated to fit int32 by the caller
-    unsigned long long fp = 0, bad = 0;
-    FFI_TRY(plan_fingerprint(p, lookup, s, &fp, &bad));
-    if (bad != 0) return FFI_ERR_BAD_LOOKUP;
-
+    if (!dev_alloc(&p->perm, (size_t)total) || !dev_alloc(&p->col_ptr, (size_t)p->N + 1)) return FFI_ERR_OUT_OF_MEMORY;
     unsigned* sorted_keys = nullptr;
     void* temp = nullptr;
     size_t temp_bytes = 0;
@@ -101,6 +221,7 @@ int plan_build(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
         if (sorted_keys) (void)hipFree(sorted_keys);
         if (temp) (void)hipFree(temp);
     };
+    // stable LSD radix sort of (column id, flat position): positions stay ascending inside a column
     hipError_t e = rocprim::radix_sort_pairs(nullptr, temp_bytes, (const unsigned*)lookup, sorted_keys, positions,
                                              p->perm, (unsigned)total, 0, end_bit, s);
     if (e != hipSuccess) return hip_fail(e);
@@ -119,6 +240,44 @@ int plan_build(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     if (e == hipSuccess) e = hipStreamSynchronize(s);
     cleanup();
     if (e != hipSuccess) return hip_fail(e);
+    p->bytes = (size_t)total * sizeof(int32_t) + ((size_t)p->N + 1) * sizeof(int32_t);
+    return FFI_OK;
+}
+
+}  // namespace
+
+int plan_fingerprint(ffi_plan* p, const int32_t* lookup, hipStream_t s, unsigned long long* out,
+                     unsigned long long* bad_ids) {
+    const size_t total = (size_t)p->L * p->K;
+    hipLaunchKernelGGL(zero_u64_kernel, dim3(1), dim3(kBlock), 0, s, p->d_scratch, 2);
+    const unsigned blocks = (unsigned)std::min<size_t>((total + kBlock - 1) / kBlock, 2048);
+    hipLaunchKernelGGL(fingerprint_kernel, dim3(blocks), dim3(kBlock), 0, s, lookup, total, (unsigned)p->N, p->d_scratch);
+    FFI_HIP_TRY(hipGetLastError());
+    FFI_HIP_TRY(hipMemcpyAsync(p->h_scratch, p->d_scratch, 2 * sizeof(unsigned long long), hipMemcpyDeviceToHost, s));
+    FFI_HIP_TRY(hipStreamSynchronize(s));
+    *out = p->h_scratch[0];
+    *bad_ids = p->h_scratch[1];
+    return FFI_OK;
+}
+
+int plan_build(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
+    unsigned long long fp = 0, bad = 0;
+    FFI_TRY(plan_fingerprint(p, lookup, s, &fp, &bad));
+    if (bad != 0) return FFI_ERR_BAD_LOOKUP;   // also keeps the build kernels' LDS counters in range
+    // a rebuild replaces the arrays: whatever still reads the old ones must have drained
+    if (p->perm || p->ent) FFI_HIP_TRY(hipDeviceSynchronize());
+    free_arrays(p);
+    // tiled form: one thread per column (N <= 1024) and positions inside a tile in 22 bits
+    // (and 32 rows of out_grad within 32-bit byte offsets, as the kernels' buffer loads need)
+    if (p->N <= 1024 && (long long)kPlanTileLabels * p->K < (1ll << 22) && p->L < (1 << 25)) {
+        int st = build_tiled(p, lookup, s);
+        if (st != FFI_OK) { free_arrays(p); return st; }
+    }
+    if (!p->tiled) {
+        free_arrays(p);
+        int st = build_global(p, lookup, s);
+        if (st != FFI_OK) { free_arrays(p); return st; }
+    }
     p->lookup = lookup;
     p->fingerprint = fp;
     return FFI_OK;
@@ -126,12 +285,10 @@ int plan_build(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
 
 void plan_free(ffi_plan* p) {
     if (!p) return;
-    if (p->perm) (void)hipFree(p->perm);
-    if (p->col_ptr) (void)hipFree(p->col_ptr);
+    free_arrays(p);
     if (p->d_scratch) (void)hipFree(p->d_scratch);
     if (p->h_scratch) (void)hipHostFree(p->h_scratch);
-    p->perm = nullptr; p->col_ptr = nullptr; p->d_scratch = nullptr; p->h_scratch = nullptr;
-    p->bytes = 0;
+    p->d_scratch = nullptr; p->h_scratch = nullptr;
 }
 
 }  // namespace ffi

@@ -141,7 +141,8 @@ __global__ __launch_bounds__(kWgBlock) void wgrad_connection_lane(const float* _
 
 int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float* gw, const Dims& d,
                        hipStream_t s) {
-    if (tile_path_fits(d.N)) {
+    // (32 rows of out_grad must be reachable through 32-bit byte offsets)
+    if (tile_path_fits(d.N) && d.L < (1 << 25)) {
         const float* xT = x;
         if (!d.tp) {
             float* ws = nullptr;
