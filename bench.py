@@ -33,6 +33,9 @@ def parse_args():
     ap.add_argument("--seed", type=int, default=42)
     ap.add_argument("--cpu-labels", type=int, default=0, help="labels in the CPU-baseline sample (0 = auto)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-bytes", type=int, default=0,
+                    help="also run one plain device copy kernel of this many bytes (read N, write N): the "
+                         "known-size reference that rocprofv3 FETCH_SIZE/WRITE_SIZE readings are scaled by")
     return ap.parse_args()
 
 
@@ -114,6 +117,14 @@ def main():
     def step():
         check(lib.ffi_forward_f32(ptr(x), ptr(lookup), ptr(w), ptr(out), B, N, L, K, int(tp), sh))
         check(lib.ffi_backward_f32(ptr(x), ptr(lookup), ptr(w), ptr(g), ptr(gx), ptr(gw), B, N, L, K, int(tp), sh))
+
+    if args.copy_bytes:
+        src = torch.empty(args.copy_bytes // 4, dtype=torch.float32, device="cuda").fill_(1.0)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)                                  # one elementwise copy kernel: reads N bytes, writes N bytes
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         step()

@@ -10,6 +10,9 @@
 #include "ffi_internal.h"
 #include "ffi_lds_tile.h"
 
+#include <algorithm>
+#include <cstdlib>
+
 namespace ffi {
 namespace {
 
@@ -26,26 +29,54 @@ namespace {
 // keeps connections 8q..8q+7 of the current 32-connection chunk, and the value needed at step k
 // is taken from its owner with a quad_perm DPP operand (both quads of a label hold a copy).
 // ------------------------------------------------------------------------------------------------
+// The 32 connections of a chunk are handled as four octets.  The eight row reads of an octet are
+// issued back to back, and the reads of the next octet go out before the multiply-adds of the
+// current one, so every wavefront keeps 8-16 LDS requests in flight (with one or two, the LDS
+// pipe idles on latency).
+template <int Q, bool FULL>
+__device__ __forceinline__ void fwd_reads(const char* __restrict__ xs_bytes, const unsigned (&o8)[8], unsigned myoff,
+                                          int kvalid, float4 (&xv)[8]) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        if (FULL || (Q * 8 + i) < kvalid) {
+            const unsigned a = quad_bcast<Q>(o8[i]) + myoff;
+            xv[i] = *reinterpret_cast<const float4*>(xs_bytes + a);
+        }
+    }
+}
+
+template <int Q, bool FULL>
+__device__ __forceinline__ void fwd_fmas(const float (&w8)[8], int kvalid, const float4 (&xv)[8], float (&acc)[4]) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        if (FULL || (Q * 8 + i) < kvalid) {
+            const float wk = quad_bcast<Q>(w8[i]);
+            acc[0] = fmaf(wk, xv[i].x, acc[0]);
+            acc[1] = fmaf(wk, xv[i].y, acc[1]);
+            acc[2] = fmaf(wk, xv[i].z, acc[2]);
+            acc[3] = fmaf(wk, xv[i].w, acc[3]);
+        }
+    }
+}
+
 template <bool FULL>
 __device__ __forceinline__ void fwd_chunk(const char* __restrict__ xs_bytes, const float (&w8)[8],
                                           const unsigned (&o8)[8], unsigned myoff, int kvalid,
                                           float (&acc)[4]) {
-#define FFI_FWD_STEP(Q, I)                                                       \
-    if (FULL || (Q * 8 + I) < kvalid) {                                          \
-        const float wk = quad_bcast<Q>(w8[I]);                                   \
-        const unsigned a = quad_bcast<Q>(o8[I]) + myoff;                         \
-        const float4 xv = *reinterpret_cast<const float4*>(xs_bytes + a);        \
-        acc[0] = fmaf(wk, xv.x, acc[0]);                                         \
-        acc[1] = fmaf(wk, xv.y, acc[1]);                                         \
-        acc[2] = fmaf(wk, xv.z, acc[2]);                                         \
-        acc[3] = fmaf(wk, xv.w, acc[3]);                                         \
-    }
-#define FFI_FWD_ROW(Q) \
-    FFI_FWD_STEP(Q, 0) FFI_FWD_STEP(Q, 1) FFI_FWD_STEP(Q, 2) FFI_FWD_STEP(Q, 3) \
-    FFI_FWD_STEP(Q, 4) FFI_FWD_STEP(Q, 5) FFI_FWD_STEP(Q, 6) FFI_FWD_STEP(Q, 7)
-    FFI_FWD_ROW(0) FFI_FWD_ROW(1) FFI_FWD_ROW(2) FFI_FWD_ROW(3)
-#undef FFI_FWD_ROW
-#undef FFI_FWD_STEP
+    float4 xa[8], xb[8];
+    fwd_reads<0, FULL>(xs_bytes, o8, myoff, kvalid, xa);
+    fwd_reads<1, FULL>(xs_bytes, o8, myoff, kvalid, xb);
+    __builtin_amdgcn_sched_barrier(0);
+    fwd_fmas<0, FULL>(w8, kvalid, xa, acc);
+    __builtin_amdgcn_sched_barrier(0);
+    fwd_reads<2, FULL>(xs_bytes, o8, myoff, kvalid, xa);
+    __builtin_amdgcn_sched_barrier(0);
+    fwd_fmas<1, FULL>(w8, kvalid, xb, acc);
+    __builtin_amdgcn_sched_barrier(0);
+    fwd_reads<3, FULL>(xs_bytes, o8, myoff, kvalid, xb);
+    __builtin_amdgcn_sched_barrier(0);
+    fwd_fmas<2, FULL>(w8, kvalid, xa, acc);
+    fwd_fmas<3, FULL>(w8, kvalid, xb, acc);
 }
 
 template <bool VEC4>
@@ -59,7 +90,7 @@ __global__ __launch_bounds__(kTileThreads) void fwd_rows32_kernel(const float* _
     const int u = xcd_contiguous_block(blockIdx.x, gridDim.x);
     const int bt = u % nbt, stream = u / nbt;
     const int b0 = bt * kTileBatch;
-    stage_rows32(xs, xT, N, B, b0);
+    stage_rows32<kTileThreads>(xs, xT, N, B, b0);
     __syncthreads();
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -71,29 +102,152 @@ __global__ __launch_bounds__(kTileThreads) void fwd_rows32_kernel(const float* _
     const int g_end = min(g_begin + groups_per_stream, total_groups);
     const int nfull = K / 32, ktail = K - nfull * 32;
 
-    for (int grp = g_begin + wave; grp < g_end; grp += kTileThreads / 64) {
-        const int j = grp * kLabelsPerWave + g;
-        const bool valid = j < L;
-        const size_t row = (size_t)(valid ? j : L - 1) * K;   // keep every lane's loads in bounds
-        float acc[4] = {0.f, 0.f, 0.f, 0.f};
-        for (int ch = 0; ch < nfull; ++ch) {
-            float w8[8];
-            unsigned o8[8];
-            load_chunk8<VEC4, true>(w + row, idx + row, ch * 32 + sq * 8, K, w8, o8);
-            fwd_chunk<true>(xs_bytes, w8, o8, myoff, 32, acc);
-        }
-        if (ktail) {
-            float w8[8];
-            unsigned o8[8];
-            load_chunk8<VEC4, false>(w + row, idx + row, nfull * 32 + sq * 8, K, w8, o8);
-            fwd_chunk<false>(xs_bytes, w8, o8, myoff, ktail, acc);
-        }
-        if (valid) {
+    // Software pipeline over (label group, 32-connection chunk) steps: the W/idx registers of the
+    // next step are requested before the current step's multiply-adds, so global-load latency
+    // hides behind LDS work.
+    const int nchunks = nfull + (ktail ? 1 : 0);
+    const int stride = kTileThreads / 64;
+    int grp = g_begin + wave, ch = 0;
+    float w8[8];
+    unsigned o8[8];
+    auto row_of = [&](int gidx) -> size_t {
+        const int j = gidx * kLabelsPerWave + g;
+        return (size_t)(j < L ? j : L - 1) * K;            // keep every lane's loads in bounds
+    };
+    auto issue = [&](int gidx, int c, float (&wd)[8], unsigned (&od)[8]) {
+        const size_t row = row_of(gidx);
+        if (c < nfull) load_chunk8<VEC4, true>(w + row, idx + row, c * 32 + sq * 8, K, wd, od);
+        else load_chunk8<VEC4, false>(w + row, idx + row, c * 32 + sq * 8, K, wd, od);
+    };
+    if (grp < g_end) issue(grp, 0, w8, o8);
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    while (grp < g_end) {
+        int ngrp = grp, nch = ch + 1;
+        if (nch == nchunks) { nch = 0; ngrp = grp + stride; }
+        float w8n[8];
+        unsigned o8n[8];
+        const bool more = ngrp < g_end;
+#ifdef FFI_EXP_NOLOAD
+        if (more) { for (int i = 0; i < 8; ++i) { w8n[i] = w8[i] * 1.0001f; o8n[i] = (o8[i] + 128u * 7u) % (128u * (unsigned)N); } }
+#else
+        if (more) issue(ngrp, nch, w8n, o8n);
+#endif
+        if (ch < nfull) fwd_chunk<true>(xs_bytes, w8, o8, myoff, 32, acc);
+        else fwd_chunk<false>(xs_bytes, w8, o8, myoff, ktail, acc);
+        if (ch == nchunks - 1) {
+            const int j = grp * kLabelsPerWave + g;
+            if (j < L) {
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                const int b = b0 + 4 * s + c;
-                if (b < B) out[(size_t)b * L + j] = acc[c];
+                for (int c = 0; c < 4; ++c) {
+                    const int b = b0 + 4 * s + c;
+#ifdef FFI_EXP_NOSTORE
+                    if (b < B && acc[c] == 12345.678f) out[(size_t)b * L + j] = acc[c];
+#else
+                    if (b < B) out[(size_t)b * L + j] = acc[c];
+#endif
+                }
             }
+            acc[0] = acc[1] = acc[2] = acc[3] = 0.f;
+        }
+        if (more) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) { w8[i] = w8n[i]; o8[i] = o8n[i]; }
+        }
+        grp = ngrp; ch = nch;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Narrow-input kernel, lane-per-label form: thread <-> label, 32 accumulators (one per batch row of
+// the tile), W and idx of the label in registers.  Each lane reads whole 128-byte rows of xs with
+// the chunk order skewed by its lane id; the accumulators are brought back to natural batch order
+// before the stores, which are then full 256-byte rows of out per wavefront.
+// ------------------------------------------------------------------------------------------------
+template <int C>
+__device__ __forceinline__ void fwd_lane_step(const char* __restrict__ xs_bytes, unsigned base, float wv, float (&acc)[32]) {
+    const float4 v = *reinterpret_cast<const float4*>(xs_bytes + skew_addr<C>(base));
+    acc[4 * C + 0] = fmaf(wv, v.x, acc[4 * C + 0]);
+    acc[4 * C + 1] = fmaf(wv, v.y, acc[4 * C + 1]);
+    acc[4 * C + 2] = fmaf(wv, v.z, acc[4 * C + 2]);
+    acc[4 * C + 3] = fmaf(wv, v.w, acc[4 * C + 3]);
+}
+
+template <bool VEC4>
+__global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* __restrict__ xT,
+                                                                  const int32_t* __restrict__ idx,
+                                                                  const float* __restrict__ w,
+                                                                  float* __restrict__ out, int B, int N,
+                                                                  int L, int K, int nbt, int labels_per_stream) {
+    extern __shared__ __align__(16) float xs[];
+    const char* xs_bytes = reinterpret_cast<const char*>(xs);
+    const int u = xcd_contiguous_block(blockIdx.x, gridDim.x);
+    const int bt = u % nbt, stream = u / nbt;
+    const int b0 = bt * kTileBatch;
+    stage_rows32<kTileThreads>(xs, xT, N, B, b0);
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
+    const unsigned skew = (unsigned)(lane & 7) * 16u;
+    const int l_begin = stream * labels_per_stream;
+    const int l_end = min(l_begin + labels_per_stream, L);
+    const int nchunks = (K + 31) / 32;
+    // rows of out for this batch tile, reached through a scalar row offset plus the lane's label
+    const int nrows = min(kTileBatch, B - b0);
+    float* obase = out + (size_t)b0 * (size_t)L;
+    const buffer_rsrc orsrc = make_rsrc(obase, (size_t)nrows * (size_t)L * sizeof(float));
+
+    for (int base = l_begin; base < l_end; base += kTileThreads) {
+        const int j = base + (int)threadIdx.x;
+        const bool valid = j < l_end;
+        const int jj = valid ? j : l_end - 1;
+        const int32_t* irow = idx + (size_t)jj * K;
+        const float* wrow = w + (size_t)jj * K;
+        float acc[32];
+#pragma unroll
+        for (int i = 0; i < 32; ++i) acc[i] = 0.f;
+        for (int ch = 0; ch < nchunks; ++ch) {
+            const int k0 = ch * 32;
+            const bool full = VEC4 && k0 + 32 <= K;
+            unsigned idp[16];
+            float wv[32];
+            if (full) {
+#pragma unroll
+                for (int q = 0; q < 8; ++q) {
+                    const int4 v = *reinterpret_cast<const int4*>(irow + k0 + 4 * q);
+                    idp[2 * q + 0] = (unsigned)v.x | ((unsigned)v.y << 16);
+                    idp[2 * q + 1] = (unsigned)v.z | ((unsigned)v.w << 16);
+                    const float4 f = *reinterpret_cast<const float4*>(wrow + k0 + 4 * q);
+                    wv[4 * q] = f.x; wv[4 * q + 1] = f.y; wv[4 * q + 2] = f.z; wv[4 * q + 3] = f.w;
+                }
+            } else {
+#pragma unroll
+                for (int q = 0; q < 16; ++q) {
+                    const unsigned a = (k0 + 2 * q < K) ? (unsigned)irow[k0 + 2 * q] : 0u;
+                    const unsigned b = (k0 + 2 * q + 1 < K) ? (unsigned)irow[k0 + 2 * q + 1] : 0u;
+                    idp[q] = a | (b << 16);
+                }
+#pragma unroll
+                for (int k = 0; k < 32; ++k) wv[k] = (k0 + k < K) ? wrow[k0 + k] : 0.f;
+            }
+            const int kn = min(32, K - k0);
+#pragma unroll
+            for (int k = 0; k < 32; ++k) {
+                if (full || k < kn) {
+                    const unsigned id = (k & 1) ? (idp[k >> 1] >> 16) : (idp[k >> 1] & 0xffffu);
+                    const unsigned rb = (id << 7) | skew;
+                    fwd_lane_step<0>(xs_bytes, rb, wv[k], acc); fwd_lane_step<1>(xs_bytes, rb, wv[k], acc);
+                    fwd_lane_step<2>(xs_bytes, rb, wv[k], acc); fwd_lane_step<3>(xs_bytes, rb, wv[k], acc);
+                    fwd_lane_step<4>(xs_bytes, rb, wv[k], acc); fwd_lane_step<5>(xs_bytes, rb, wv[k], acc);
+                    fwd_lane_step<6>(xs_bytes, rb, wv[k], acc); fwd_lane_step<7>(xs_bytes, rb, wv[k], acc);
+                }
+            }
+        }
+        xor_permute_groups(acc, lane & 7);                 // back to natural batch order
+        if (valid) {
+            const unsigned lane_off = (unsigned)j * 4u;
+            const unsigned stride = (unsigned)L * 4u;
+#pragma unroll
+            for (int b = 0; b < 32; ++b)
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, acc[b]), orsrc, lane_off, (unsigned)b * stride, 0);
         }
     }
 }
@@ -148,10 +302,28 @@ int launch_forward(const float* x, const int32_t* idx, const float* w, float* ou
             FFI_TRY(launch_transpose(x, ws, d.B, d.N, s));   // [B,N] -> [N,B]
             xT = ws;
         }
-        TileGrid tg;
-        FFI_TRY(tile_grid(d.B, d.L, &tg));
         const size_t lds = tile_lds_bytes(d.N);
         const bool vec4 = (d.K % 4 == 0) && (((uintptr_t)w | (uintptr_t)idx) % 16 == 0);
+        static const bool use_quads = getenv("FFI_FWD_QUADS") != nullptr;
+        if (!use_quads && d.L < (1 << 25)) {
+            const int cus = device_cu_count();
+            const int nbt = (d.B + kTileBatch - 1) / kTileBatch;
+            int streams = std::max(1, cus / nbt);
+            int per_stream = (d.L + streams - 1) / streams;
+            streams = (d.L + per_stream - 1) / per_stream;
+            const int blocks = streams * nbt;
+            if (vec4) {
+                FFI_HIP_TRY(hipFuncSetAttribute((const void*)fwd_lane32_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+                hipLaunchKernelGGL(fwd_lane32_kernel<true>, dim3(blocks), dim3(kTileThreads), lds, s, xT, idx, w, out, d.B, d.N, d.L, d.K, nbt, per_stream);
+            } else {
+                FFI_HIP_TRY(hipFuncSetAttribute((const void*)fwd_lane32_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+                hipLaunchKernelGGL(fwd_lane32_kernel<false>, dim3(blocks), dim3(kTileThreads), lds, s, xT, idx, w, out, d.B, d.N, d.L, d.K, nbt, per_stream);
+            }
+            FFI_HIP_TRY(hipGetLastError());
+            return FFI_OK;
+        }
+        TileGrid tg;
+        FFI_TRY(tile_grid(d.B, d.L, &tg));
         if (vec4) {
             FFI_HIP_TRY(hipFuncSetAttribute((const void*)fwd_rows32_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
             hipLaunchKernelGGL(fwd_rows32_kernel<true>, dim3(tg.blocks), dim3(kTileThreads), lds, s, xT, idx, w, out, d.B, d.N, d.L, d.K, tg.nbt, tg.groups_per_stream);

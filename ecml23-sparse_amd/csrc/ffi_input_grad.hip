@@ -18,20 +18,33 @@ namespace {
 // ---- tiled plan ---------------------------------------------------------------------------------
 
 // wp[slot] = w at the connection stored in that slot (0 in padding slots): brings the weights into
-// the plan's slot order so that the main kernel reads them coalesced.  One workgroup per tile.
-__global__ void igrad_permute_weights_kernel(const unsigned* __restrict__ ent, const unsigned* __restrict__ slice_off,
-                                             const unsigned short* __restrict__ col_len, const float* __restrict__ w,
-                                             float* __restrict__ wp, int K, int tile_labels) {
-    const int t = blockIdx.x, nthreads = blockDim.x;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const size_t sl = (size_t)t * (nthreads >> 6) + wave;
+// the plan's slot order so that the main kernel reads them coalesced.  One wavefront per slice,
+// eight rows in flight per lane.
+constexpr int kPermBlock = 256;
+__global__ __launch_bounds__(kPermBlock) void igrad_permute_weights_kernel(
+    const unsigned* __restrict__ ent, const unsigned* __restrict__ slice_off, const unsigned short* __restrict__ col_len,
+    const float* __restrict__ w, float* __restrict__ wp, int K, int tile_labels, int slices, int nthreads, int nslices) {
+    const int sl = blockIdx.x * (kPermBlock / 64) + (threadIdx.x >> 6);
+    if (sl >= nslices) return;
+    const int lane = threadIdx.x & 63;
+    const int t = sl / slices, wave = sl - t * slices;
     const unsigned row0 = slice_off[sl], rows = slice_off[sl + 1] - row0;
-    const unsigned len = col_len[(size_t)t * nthreads + threadIdx.x];
+    const unsigned len = col_len[(size_t)t * nthreads + wave * 64 + lane];
     const float* wt = w + (size_t)t * tile_labels * K;
-    for (unsigned i = 0; i < rows; ++i) {
-        const size_t slot = ((size_t)row0 + i) * 64 + lane;
-        wp[slot] = (i < len) ? wt[ent[slot] >> 10] : 0.f;
+    const unsigned* ep = ent + (size_t)row0 * 64 + lane;
+    float* op = wp + (size_t)row0 * 64 + lane;
+    unsigned i = 0;
+    for (; i + 8 <= rows; i += 8) {
+        unsigned e8[8];
+        float v8[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) e8[q] = ep[(size_t)(i + q) * 64];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) v8[q] = (i + q < len) ? wt[e8[q] >> 10] : 0.f;
+#pragma unroll
+        for (int q = 0; q < 8; ++q) op[(size_t)(i + q) * 64] = v8[q];
     }
+    for (; i < rows; ++i) op[(size_t)i * 64] = (i < len) ? wt[ep[(size_t)i * 64] >> 10] : 0.f;
 }
 
 template <int C>
@@ -94,20 +107,31 @@ __global__ __launch_bounds__(1024) void igrad_tile_kernel(const unsigned* __rest
         const unsigned len = col_len[(size_t)t * nthreads + threadIdx.x];
         const unsigned* ep = ent + (size_t)row0 * 64 + lane;
         const float* wpp = wp + (size_t)row0 * 64 + lane;
-        unsigned i = 0;
-        for (; i + 4 <= rows; i += 4) {
-            unsigned e4[4];
-            float w4[4];
+        // slots are read four rows ahead of the multiply-adds that use them
+        constexpr int kAhead = 4;
+        unsigned e4[kAhead];
+        float w4[kAhead];
 #pragma unroll
-            for (int q = 0; q < 4; ++q) { e4[q] = ep[(size_t)(i + q) * 64]; w4[q] = wpp[(size_t)(i + q) * 64]; }
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-                if (i + q < len) igrad_entry(gs_bytes, e4[q], w4[q], skew, acc);
+        for (int q = 0; q < kAhead; ++q) {
+            const bool in = (unsigned)q < rows;
+            e4[q] = in ? ep[(size_t)q * 64] : 0u;
+            w4[q] = in ? wpp[(size_t)q * 64] : 0.f;
         }
-        for (; i < rows; ++i) {
-            const unsigned e = ep[(size_t)i * 64];
-            const float wv = wpp[(size_t)i * 64];
-            if (i < len) igrad_entry(gs_bytes, e, wv, skew, acc);
+        for (unsigned i = 0; i < rows; i += kAhead) {
+            unsigned en[kAhead];
+            float wn[kAhead];
+#pragma unroll
+            for (int q = 0; q < kAhead; ++q) {
+                const unsigned r = i + kAhead + q;
+                const bool in = r < rows;
+                en[q] = in ? ep[(size_t)r * 64] : 0u;
+                wn[q] = in ? wpp[(size_t)r * 64] : 0.f;
+            }
+#pragma unroll
+            for (int q = 0; q < kAhead; ++q)
+                if (i + q < len) igrad_entry(gs_bytes, e4[q], w4[q], skew, acc);
+#pragma unroll
+            for (int q = 0; q < kAhead; ++q) { e4[q] = en[q]; w4[q] = wn[q]; }
         }
     }
     // back to natural batch order, then one 128-byte row per thread
@@ -188,8 +212,10 @@ int launch_tiled(const ffi_plan* p, const float* w, const float* g, float* gx, i
     float* partial = nullptr;
     FFI_TRY(workspace_get(s, kWsFeaturesT, std::max<size_t>(slots, 1) * sizeof(float), (void**)&wp));
     FFI_TRY(workspace_get(s, kWsPartials, (size_t)streams * p->threads * bpad * sizeof(float), (void**)&partial));
-    hipLaunchKernelGGL(igrad_permute_weights_kernel, dim3(p->tiles), dim3(p->threads), 0, s, p->ent, p->slice_off,
-                       p->col_len, w, wp, p->K, p->tile_labels);
+    const int nslices = p->tiles * p->slices;
+    hipLaunchKernelGGL(igrad_permute_weights_kernel, dim3((nslices + kPermBlock / 64 - 1) / (kPermBlock / 64)),
+                       dim3(kPermBlock), 0, s, p->ent, p->slice_off, p->col_len, w, wp, p->K, p->tile_labels, p->slices,
+                       p->threads, nslices);
     const size_t lds = tile_lds_bytes(p->tile_labels);
     FFI_HIP_TRY(hipFuncSetAttribute((const void*)igrad_tile_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     hipLaunchKernelGGL(igrad_tile_kernel, dim3(streams * nbt), dim3(p->threads), lds, s, p->ent, wp, p->slice_off,

@@ -43,15 +43,39 @@ __device__ __forceinline__ int xcd_contiguous_block(int block, int nblocks) {
 }
 
 // xs[r][c] = src[r*ld + c0 + c] for c < 32 (zero beyond column `ld`), r < rows.  src rows are read
-// in 128-byte pieces, LDS writes are conflict-free.
+// in 128-byte pieces, LDS writes are conflict-free.  All of a thread's loads are issued before its
+// first LDS write, so the staging costs one memory round trip, not one per row.
+template <int THREADS>
 __device__ __forceinline__ void stage_rows32(float* __restrict__ xs, const float* __restrict__ src, int rows,
                                              int ld, int c0) {
-    const int c = threadIdx.x & 31;
-    const bool in = c0 + c < ld;
-    const float* p = src + c0 + c;
-#pragma unroll 4
-    for (int r = threadIdx.x >> 5; r < rows; r += kTileThreads / 32)
-        xs[r * kTileBatch + c] = in ? p[(size_t)r * ld] : 0.f;
+    const bool vec = (ld % 4 == 0) && (c0 + kTileBatch <= ld) && (((uintptr_t)src & 15) == 0);
+    if (vec) {
+        // thread -> (row, 16-byte chunk): 8 threads per row
+        constexpr int kRowsPerIter = THREADS / 8;
+        constexpr int kInFlight = 4;
+        const int q = threadIdx.x & 7;
+        const float* p = src + c0 + 4 * q;
+        for (int r0 = threadIdx.x >> 3; r0 < rows; r0 += kRowsPerIter * kInFlight) {
+            float4 v[kInFlight];
+#pragma unroll
+            for (int i = 0; i < kInFlight; ++i) {
+                const int r = r0 + i * kRowsPerIter;
+                v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (r < rows) v[i] = *reinterpret_cast<const float4*>(p + (size_t)r * ld);
+            }
+#pragma unroll
+            for (int i = 0; i < kInFlight; ++i) {
+                const int r = r0 + i * kRowsPerIter;
+                if (r < rows) *reinterpret_cast<float4*>(xs + r * kTileBatch + 4 * q) = v[i];
+            }
+        }
+    } else {
+        const int c = threadIdx.x & 31;
+        const bool in = c0 + c < ld;
+        const float* p = src + c0 + c;
+        for (int r = threadIdx.x >> 5; r < rows; r += THREADS / 32)
+            xs[r * kTileBatch + c] = in ? p[(size_t)r * ld] : 0.f;
+    }
 }
 
 // Raw buffer resource over `bytes` bytes at p (gfx9 family: 32-bit data format word).  Loads

@@ -16,32 +16,56 @@ namespace {
 
 constexpr int kBlock = 256;
 
-__device__ __forceinline__ unsigned long long mix64(unsigned long long v) {
-    v ^= v >> 30; v *= 0xbf58476d1ce4e5b9ull;
-    v ^= v >> 27; v *= 0x94d049bb133111ebull;
-    v ^= v >> 31;
+__device__ __forceinline__ unsigned mix32(unsigned v) {
+    v ^= v >> 16; v *= 0x7feb352du;
+    v ^= v >> 15; v *= 0x846ca68bu;
+    v ^= v >> 16;
     return v;
 }
 
-// Order-independent 64-bit content fingerprint: sum over positions of mix(position, id), plus the
-// number of ids outside [0,N).  Integer atomics only, so the value is reproducible.
+// Order-independent 64-bit content fingerprint: sum over positions p of mix(id_p + p * odd), plus
+// the number of ids outside [0,N).  Integer adds only, so the value does not depend on the order
+// of the atomics.  Four ids per load when the array allows it.
 __global__ __launch_bounds__(kBlock) void fingerprint_kernel(const int32_t* __restrict__ idx,
                                                               size_t total, unsigned N,
                                                               unsigned long long* __restrict__ out) {
-    unsigned long long h = 0, bad = 0;
-    for (size_t p = (size_t)blockIdx.x * kBlock + threadIdx.x; p < total; p += (size_t)gridDim.x * kBlock) {
+    unsigned long long h = 0;
+    unsigned bad = 0;
+    const size_t stride = (size_t)gridDim.x * kBlock;
+    const size_t tid = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    const bool vec = ((uintptr_t)idx & 15) == 0;
+    const size_t nvec = vec ? total / 4 : 0;
+    const int4* idx4 = reinterpret_cast<const int4*>(idx);
+    for (size_t q = tid; q < nvec; q += stride) {
+        const int4 v = idx4[q];
+        const unsigned p = (unsigned)(q * 4);
+        h += mix32((unsigned)v.x + p * 0x9e3779b1u);
+        h += mix32((unsigned)v.y + (p + 1) * 0x9e3779b1u);
+        h += mix32((unsigned)v.z + (p + 2) * 0x9e3779b1u);
+        h += mix32((unsigned)v.w + (p + 3) * 0x9e3779b1u);
+        bad += ((unsigned)v.x >= N) + ((unsigned)v.y >= N) + ((unsigned)v.z >= N) + ((unsigned)v.w >= N);
+    }
+    for (size_t p = nvec * 4 + tid; p < total; p += stride) {
         const unsigned id = (unsigned)idx[p];
-        h += mix64(((unsigned long long)p << 32) ^ id ^ 0x9e3779b97f4a7c15ull);
+        h += mix32(id + (unsigned)p * 0x9e3779b1u);
         bad += id >= N;
     }
+    unsigned long long b64 = bad;
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
         h += __shfl_down(h, off);
-        bad += __shfl_down(bad, off);
+        b64 += __shfl_down(b64, off);
     }
-    if ((threadIdx.x & 63) == 0) {
-        atomicAdd(&out[0], h);
-        if (bad) atomicAdd(&out[1], bad);
+    // one pair of atomics per workgroup: thousands of wavefronts adding to one address serialise
+    __shared__ unsigned long long part[2][kBlock / 64];
+    if ((threadIdx.x & 63) == 0) { part[0][threadIdx.x >> 6] = h; part[1][threadIdx.x >> 6] = b64; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned long long hs = 0, bs = 0;
+#pragma unroll
+        for (int i = 0; i < kBlock / 64; ++i) { hs += part[0][i]; bs += part[1][i]; }
+        atomicAdd(&out[0], hs);
+        if (bs) atomicAdd(&out[1], bs);
     }
 }
 
@@ -250,7 +274,7 @@ int plan_fingerprint(ffi_plan* p, const int32_t* lookup, hipStream_t s, unsigned
                      unsigned long long* bad_ids) {
     const size_t total = (size_t)p->L * p->K;
     hipLaunchKernelGGL(zero_u64_kernel, dim3(1), dim3(kBlock), 0, s, p->d_scratch, 2);
-    const unsigned blocks = (unsigned)std::min<size_t>((total + kBlock - 1) / kBlock, 2048);
+    const unsigned blocks = (unsigned)std::min<size_t>((total / 4 + kBlock - 1) / kBlock + 1, 2048);
     hipLaunchKernelGGL(fingerprint_kernel, dim3(blocks), dim3(kBlock), 0, s, lookup, total, (unsigned)p->N, p->d_scratch);
     FFI_HIP_TRY(hipGetLastError());
     FFI_HIP_TRY(hipMemcpyAsync(p->h_scratch, p->d_scratch, 2 * sizeof(unsigned long long), hipMemcpyDeviceToHost, s));

@@ -9,11 +9,13 @@ namespace {
 
 // ------------------------------------------------------------------------------------------------
 // Narrow-input kernel: lane <-> label, 32 connections of the label per pass held as 32 fp32
-// accumulators, xs[n][32 batch rows] in LDS.  For every batch tile the workgroup re-stages xs
-// (cheap: one 96 KB tile per 1024 labels x 32 connections x 32 rows of multiply-adds), so each
-// gw element is summed over the whole batch in registers and written exactly once: no atomics, no
-// partial buffers, bit-reproducible.  Each lane reads whole 128-byte rows with the chunk order
-// skewed by its lane id (see ffi_lds_tile.h), which keeps the gathers free of bank conflicts.
+// accumulators, xs[n][32 batch rows] in LDS.  A workgroup owns a range of labels and makes one
+// sweep over it per batch tile: xs is staged once per sweep, and inside a sweep there is no
+// barrier, so the wavefronts drift apart and the out_grad/idx loads of some overlap the LDS work of
+// the others.  The first sweep writes gw, every later sweep adds its partial sum to what the same
+// thread wrote before (plain read-modify-write: no atomics, fixed order, bit-reproducible).
+// Each lane reads whole 128-byte rows with the chunk order skewed by its lane id (see
+// ffi_lds_tile.h), and out_grad is permuted in registers to match.
 // ------------------------------------------------------------------------------------------------
 constexpr int kWgChunk = 32;   // connections per register pass
 
@@ -37,52 +39,62 @@ __global__ __launch_bounds__(kTileThreads) void wgrad_rows32_kernel(const float*
     extern __shared__ __align__(16) float xs[];
     const char* xs_bytes = reinterpret_cast<const char*>(xs);
     const int lane = threadIdx.x & 63;
-    unsigned skew = (unsigned)(lane & 7) * 16u;
+    const unsigned skew = (unsigned)(lane & 7) * 16u;
     const int l_begin = blockIdx.x * labels_per_block;
     const int l_end = min(l_begin + labels_per_block, L);
     const int nbt = (B + kTileBatch - 1) / kTileBatch;
     const int nchunks = (K + kWgChunk - 1) / kWgChunk;
 
-    for (int base = l_begin; base < l_end; base += kTileThreads) {
-        const int j = base + (int)threadIdx.x;
-        const bool valid = j < l_end;
-        const int jj = valid ? j : l_end - 1;              // keep loads in bounds
-        const int32_t* irow = idx + (size_t)jj * K;
-        for (int ch = 0; ch < nchunks; ++ch) {
-            const int k0 = ch * kWgChunk;
-            // column ids of this pass, two 16-bit ids per register (ids < 2^16 on this path)
-            unsigned idp[kWgChunk / 2];
-            if (VEC4 && k0 + kWgChunk <= K) {
+    for (int bt = 0; bt < nbt; ++bt) {
+        const int b0 = bt * kTileBatch;
+        __syncthreads();                                   // everyone is done with the previous tile
+        stage_rows32<kTileThreads>(xs, xT, N, B, b0);
+        __syncthreads();
+        for (int base = l_begin; base < l_end; base += kTileThreads) {
+            const int j = base + (int)threadIdx.x;
+            const bool valid = j < l_end;
+            const int jj = valid ? j : l_end - 1;          // keep loads in bounds
+            const int32_t* irow = idx + (size_t)jj * K;
+            float* grow = gw + (size_t)jj * K;
+            // out_grad of this label for the tile's 32 batch rows: coalesced across lanes
+            float gb[32];
+            load_rows32(g, L, b0, B, (unsigned)jj, gb);
+            xor_permute_groups(gb, lane & 7);              // match the skewed chunk order of the gathers
+            for (int ch = 0; ch < nchunks; ++ch) {
+                const int k0 = ch * kWgChunk;
+                const bool full = VEC4 && k0 + kWgChunk <= K;
+                // column ids of this pass, two 16-bit ids per register (ids < 2^16 on this path)
+                unsigned idp[kWgChunk / 2];
+                float acc[kWgChunk];
+                if (full) {
 #pragma unroll
-                for (int q = 0; q < kWgChunk / 4; ++q) {
-                    const int4 v = *reinterpret_cast<const int4*>(irow + k0 + 4 * q);
-                    idp[2 * q + 0] = (unsigned)v.x | ((unsigned)v.y << 16);
-                    idp[2 * q + 1] = (unsigned)v.z | ((unsigned)v.w << 16);
+                    for (int q = 0; q < kWgChunk / 4; ++q) {
+                        const int4 v = *reinterpret_cast<const int4*>(irow + k0 + 4 * q);
+                        idp[2 * q + 0] = (unsigned)v.x | ((unsigned)v.y << 16);
+                        idp[2 * q + 1] = (unsigned)v.z | ((unsigned)v.w << 16);
+                    }
+                } else {
+#pragma unroll
+                    for (int q = 0; q < kWgChunk / 2; ++q) {
+                        const unsigned a = (k0 + 2 * q < K) ? (unsigned)irow[k0 + 2 * q] : 0u;
+                        const unsigned b = (k0 + 2 * q + 1 < K) ? (unsigned)irow[k0 + 2 * q + 1] : 0u;
+                        idp[q] = a | (b << 16);
+                    }
                 }
-            } else {
+                // partial sums of the earlier batch tiles (written by this same thread)
+                if (bt == 0) {
 #pragma unroll
-                for (int q = 0; q < kWgChunk / 2; ++q) {
-                    const unsigned a = (k0 + 2 * q < K) ? (unsigned)irow[k0 + 2 * q] : 0u;
-                    const unsigned b = (k0 + 2 * q + 1 < K) ? (unsigned)irow[k0 + 2 * q + 1] : 0u;
-                    idp[q] = a | (b << 16);
+                    for (int k = 0; k < kWgChunk; ++k) acc[k] = 0.f;
+                } else if (full) {
+#pragma unroll
+                    for (int q = 0; q < kWgChunk / 4; ++q) {
+                        const float4 v = *reinterpret_cast<const float4*>(grow + k0 + 4 * q);
+                        acc[4 * q] = v.x; acc[4 * q + 1] = v.y; acc[4 * q + 2] = v.z; acc[4 * q + 3] = v.w;
+                    }
+                } else {
+#pragma unroll
+                    for (int k = 0; k < kWgChunk; ++k) acc[k] = (k0 + k < K) ? grow[k0 + k] : 0.f;
                 }
-            }
-            float acc[kWgChunk];
-#pragma unroll
-            for (int k = 0; k < kWgChunk; ++k) acc[k] = 0.f;
-
-            for (int bt = 0; bt < nbt; ++bt) {
-                const int b0 = bt * kTileBatch;
-                __syncthreads();                           // everyone is done with the previous tile
-                stage_rows32(xs, xT, N, B, b0);
-                // out_grad of this label for the tile's 32 batch rows: coalesced across lanes
-                float gb[32];
-                load_rows32(g, L, b0, B, (unsigned)jj, gb);
-                xor_permute_groups(gb, lane & 7);          // match the skewed chunk order of the gathers
-                __syncthreads();
-                // keep the 256 row addresses of this pass from being hoisted out of the batch-tile
-                // loop (they would be spilled): the compiler must treat `skew` as changing here
-                asm volatile("" : "+v"(skew));
 #pragma unroll
                 for (int k = 0; k < kWgChunk; ++k) {
                     const unsigned id = (k & 1) ? (idp[k >> 1] >> 16) : (idp[k >> 1] & 0xffffu);
@@ -95,19 +107,17 @@ __global__ __launch_bounds__(kTileThreads) void wgrad_rows32_kernel(const float*
                     wgrad_step<5>(xs_bytes, rb, gb, acc[k]);
                     wgrad_step<6>(xs_bytes, rb, gb, acc[k]);
                     wgrad_step<7>(xs_bytes, rb, gb, acc[k]);
-                    if ((k & 1) == 1) __builtin_amdgcn_sched_barrier(0);   // bound the scheduler's look-ahead
                 }
-            }
-            if (valid) {
-                float* orow = gw + (size_t)j * K + k0;
-                if (VEC4 && k0 + kWgChunk <= K) {
+                if (valid) {
+                    if (full) {
 #pragma unroll
-                    for (int q = 0; q < kWgChunk / 4; ++q)
-                        *reinterpret_cast<float4*>(orow + 4 * q) = make_float4(acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]);
-                } else {
+                        for (int q = 0; q < kWgChunk / 4; ++q)
+                            *reinterpret_cast<float4*>(grow + k0 + 4 * q) = make_float4(acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]);
+                    } else {
 #pragma unroll
-                    for (int k = 0; k < kWgChunk; ++k)
-                        if (k0 + k < K) orow[k] = acc[k];
+                        for (int k = 0; k < kWgChunk; ++k)
+                            if (k0 + k < K) grow[k0 + k] = acc[k];
+                    }
                 }
             }
         }
@@ -151,9 +161,8 @@ int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float
             xT = ws;
         }
         const int cus = device_cu_count();
-        // one workgroup per CU; label ranges are multiples of the workgroup size
-        int per_block = (d.L + cus - 1) / cus;
-        per_block = ((per_block + kTileThreads - 1) / kTileThreads) * kTileThreads;
+        // one workgroup per CU, equal label ranges (the last pass of a range may be partly filled)
+        const int per_block = (d.L + cus - 1) / cus;
         const int blocks = (d.L + per_block - 1) / per_block;
         const size_t lds = tile_lds_bytes(d.N);
         const bool vec4 = (d.K % 4 == 0) && (((uintptr_t)gw | (uintptr_t)idx) % 16 == 0);
