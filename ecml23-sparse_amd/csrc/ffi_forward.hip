@@ -196,6 +196,7 @@ __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* _
     const buffer_rsrc orsrc = make_rsrc(obase, (size_t)nrows * (size_t)L * sizeof(float));
 
     for (int base = l_begin; base < l_end; base += kTileThreads) {
+        if (base + (int)(threadIdx.x & ~63u) >= l_end) break;     // nothing left for this wavefront
         const int j = base + (int)threadIdx.x;
         const bool valid = j < l_end;
         const int jj = valid ? j : l_end - 1;

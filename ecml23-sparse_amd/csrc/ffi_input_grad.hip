@@ -18,33 +18,76 @@ namespace {
 // ---- tiled plan ---------------------------------------------------------------------------------
 
 // wp[slot] = w at the connection stored in that slot (0 in padding slots): brings the weights into
-// the plan's slot order so that the main kernel reads them coalesced.  One wavefront per slice,
-// eight rows in flight per lane.
-constexpr int kPermBlock = 256;
-__global__ __launch_bounds__(kPermBlock) void igrad_permute_weights_kernel(
+// the plan's slot order so that the main kernel reads them coalesced.  One workgroup per label
+// tile, one thread per column.  The tile's weights pass through LDS in pieces of kPermChunk floats
+// (read from HBM fully coalesced); a column's slots hold ascending positions, so each thread just
+// advances a cursor through its slots while their positions fall inside the staged piece.
+constexpr int kPermChunk = 16384;     // 64 KB of LDS: two workgroups fit on a CU and overlap each other
+__global__ __launch_bounds__(1024) void igrad_permute_weights_kernel(
     const unsigned* __restrict__ ent, const unsigned* __restrict__ slice_off, const unsigned short* __restrict__ col_len,
-    const float* __restrict__ w, float* __restrict__ wp, int K, int tile_labels, int slices, int nthreads, int nslices) {
-    const int sl = blockIdx.x * (kPermBlock / 64) + (threadIdx.x >> 6);
-    if (sl >= nslices) return;
-    const int lane = threadIdx.x & 63;
-    const int t = sl / slices, wave = sl - t * slices;
+    const float* __restrict__ w, float* __restrict__ wp, int L, int K, int tile_labels) {
+    __shared__ __align__(16) float ws[kPermChunk];
+    const int t = blockIdx.x, nthreads = blockDim.x;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const size_t sl = (size_t)t * (nthreads >> 6) + wave;
     const unsigned row0 = slice_off[sl], rows = slice_off[sl + 1] - row0;
-    const unsigned len = col_len[(size_t)t * nthreads + wave * 64 + lane];
+    const unsigned len = col_len[(size_t)t * nthreads + threadIdx.x];
+    const int nl = min(tile_labels, L - t * tile_labels);
+    const unsigned npos = (unsigned)nl * (unsigned)K;
     const float* wt = w + (size_t)t * tile_labels * K;
+    const bool vec = ((((uintptr_t)wt) & 15) == 0);
     const unsigned* ep = ent + (size_t)row0 * 64 + lane;
     float* op = wp + (size_t)row0 * 64 + lane;
-    unsigned i = 0;
-    for (; i + 8 <= rows; i += 8) {
-        unsigned e8[8];
-        float v8[8];
+    unsigned lo = 0;                 // wave-uniform: rows below lo are finished in every column of the slice
+    for (unsigned c0 = 0; c0 < npos; c0 += kPermChunk) {
+        const unsigned n = min((unsigned)kPermChunk, npos - c0);
+        __syncthreads();
+        if (vec) {
+            // all of a thread's loads go out before its first LDS write: one round trip per piece
+            const unsigned nv = n / 4;
+            const float4* src4 = reinterpret_cast<const float4*>(wt + c0);
+            float4* dst4 = reinterpret_cast<float4*>(ws);
+            for (unsigned q0 = threadIdx.x; q0 < nv; q0 += nthreads * 8) {
+                float4 v[8];
 #pragma unroll
-        for (int q = 0; q < 8; ++q) e8[q] = ep[(size_t)(i + q) * 64];
+                for (int r = 0; r < 8; ++r) v[r] = src4[min(q0 + r * nthreads, nv - 1)];
 #pragma unroll
-        for (int q = 0; q < 8; ++q) v8[q] = (i + q < len) ? wt[e8[q] >> 10] : 0.f;
+                for (int r = 0; r < 8; ++r)
+                    if (q0 + r * nthreads < nv) dst4[q0 + r * nthreads] = v[r];
+            }
+            for (unsigned r = nv * 4 + threadIdx.x; r < n; r += nthreads) ws[r] = wt[c0 + r];
+        } else {
+            for (unsigned q = threadIdx.x; q < n; q += nthreads) ws[q] = wt[c0 + q];
+        }
+        __syncthreads();
+        const unsigned hi = c0 + n;
+        // The wavefront walks the slice's rows together (every load is one coalesced 256-byte
+        // row), eight rows per step; a lane stores the slots whose position lies in the staged
+        // piece.  Positions ascend inside a column, so the walk of this piece stops at the first
+        // step in which no lane found one, and the next piece resumes at the first step in which
+        // some lane met a position beyond this piece.
+        unsigned resume = 0xffffffffu;
+        for (unsigned i = lo; i < rows; i += 8) {
+            unsigned e8[8];
 #pragma unroll
-        for (int q = 0; q < 8; ++q) op[(size_t)(i + q) * 64] = v8[q];
+            for (int q = 0; q < 8; ++q) e8[q] = ep[(size_t)min(i + q, rows - 1) * 64];
+            bool any_here = false, any_later = false;
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const unsigned pos = e8[q] >> 10;
+                const bool valid = i + q < len;
+                if (valid && pos >= c0 && pos < hi) {
+                    op[(size_t)(i + q) * 64] = ws[pos - c0];
+                    any_here = true;
+                }
+                any_later |= valid && pos >= hi;
+            }
+            if (resume == 0xffffffffu && __any(any_later)) resume = i;
+            if (!__any(any_here) && resume != 0xffffffffu) break;
+        }
+        lo = (resume == 0xffffffffu) ? rows : resume;
     }
-    for (; i < rows; ++i) op[(size_t)i * 64] = (i < len) ? wt[ep[(size_t)i * 64] >> 10] : 0.f;
+    for (unsigned r = len; r < rows; ++r) op[(size_t)r * 64] = 0.f;     // padding slots
 }
 
 template <int C>
@@ -111,21 +154,23 @@ __global__ __launch_bounds__(1024) void igrad_tile_kernel(const unsigned* __rest
         constexpr int kAhead = 4;
         unsigned e4[kAhead];
         float w4[kAhead];
+        // (row indices are clamped instead of predicated, so that the loads carry no branches)
+        if (rows == 0) continue;               // wave-uniform: no column of this slice is used in the tile
+        const unsigned last = rows - 1;
 #pragma unroll
         for (int q = 0; q < kAhead; ++q) {
-            const bool in = (unsigned)q < rows;
-            e4[q] = in ? ep[(size_t)q * 64] : 0u;
-            w4[q] = in ? wpp[(size_t)q * 64] : 0.f;
+            const unsigned r = min((unsigned)q, last);
+            e4[q] = ep[(size_t)r * 64];
+            w4[q] = wpp[(size_t)r * 64];
         }
         for (unsigned i = 0; i < rows; i += kAhead) {
             unsigned en[kAhead];
             float wn[kAhead];
 #pragma unroll
             for (int q = 0; q < kAhead; ++q) {
-                const unsigned r = i + kAhead + q;
-                const bool in = r < rows;
-                en[q] = in ? ep[(size_t)r * 64] : 0u;
-                wn[q] = in ? wpp[(size_t)r * 64] : 0.f;
+                const unsigned r = min(i + kAhead + q, last);
+                en[q] = ep[(size_t)r * 64];
+                wn[q] = wpp[(size_t)r * 64];
             }
 #pragma unroll
             for (int q = 0; q < kAhead; ++q)
@@ -212,10 +257,8 @@ int launch_tiled(const ffi_plan* p, const float* w, const float* g, float* gx, i
     float* partial = nullptr;
     FFI_TRY(workspace_get(s, kWsFeaturesT, std::max<size_t>(slots, 1) * sizeof(float), (void**)&wp));
     FFI_TRY(workspace_get(s, kWsPartials, (size_t)streams * p->threads * bpad * sizeof(float), (void**)&partial));
-    const int nslices = p->tiles * p->slices;
-    hipLaunchKernelGGL(igrad_permute_weights_kernel, dim3((nslices + kPermBlock / 64 - 1) / (kPermBlock / 64)),
-                       dim3(kPermBlock), 0, s, p->ent, p->slice_off, p->col_len, w, wp, p->K, p->tile_labels, p->slices,
-                       p->threads, nslices);
+    hipLaunchKernelGGL(igrad_permute_weights_kernel, dim3(p->tiles), dim3(p->threads), 0, s, p->ent, p->slice_off,
+                       p->col_len, w, wp, p->L, p->K, p->tile_labels);
     const size_t lds = tile_lds_bytes(p->tile_labels);
     FFI_HIP_TRY(hipFuncSetAttribute((const void*)igrad_tile_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     hipLaunchKernelGGL(igrad_tile_kernel, dim3(streams * nbt), dim3(p->threads), lds, s, p->ent, wp, p->slice_off,

@@ -51,6 +51,7 @@ __global__ __launch_bounds__(kTileThreads) void wgrad_rows32_kernel(const float*
         stage_rows32<kTileThreads>(xs, xT, N, B, b0);
         __syncthreads();
         for (int base = l_begin; base < l_end; base += kTileThreads) {
+            if (base + (int)(threadIdx.x & ~63u) >= l_end) break;   // nothing left for this wavefront
             const int j = base + (int)threadIdx.x;
             const bool valid = j < l_end;
             const int jj = valid ? j : l_end - 1;          // keep loads in bounds
