@@ -74,7 +74,7 @@ __global__ __launch_bounds__(1024) void igrad_permute_weights_kernel(
             bool any_here = false, any_later = false;
 #pragma unroll
             for (int q = 0; q < 8; ++q) {
-                const unsigned pos = e8[q] >> 10;
+                const unsigned pos = e8[q] >> kEntLabelBits;
                 const bool valid = i + q < len;
                 if (valid && pos >= c0 && pos < hi) {
                     op[(size_t)(i + q) * 64] = ws[pos - c0];
@@ -90,26 +90,34 @@ __global__ __launch_bounds__(1024) void igrad_permute_weights_kernel(
     for (unsigned r = len; r < rows; ++r) op[(size_t)r * 64] = 0.f;     // padding slots
 }
 
-template <int C>
-__device__ __forceinline__ void igrad_step(const char* __restrict__ gs_bytes, unsigned base, float wv, float (&acc)[32]) {
-    const float4 v = *reinterpret_cast<const float4*>(gs_bytes + skew_addr<C>(base));
-    acc[4 * C + 0] = fmaf(wv, v.x, acc[4 * C + 0]);
-    acc[4 * C + 1] = fmaf(wv, v.y, acc[4 * C + 1]);
-    acc[4 * C + 2] = fmaf(wv, v.z, acc[4 * C + 2]);
-    acc[4 * C + 3] = fmaf(wv, v.w, acc[4 * C + 3]);
+// The eight 16-byte reads of one row (chunk order skewed by the lane id) ...
+__device__ __forceinline__ void igrad_reads(const char* __restrict__ gs_bytes, unsigned e, unsigned skew, float4 (&v)[8]) {
+    const unsigned base = ((e & kEntLabelMask) << 7) | skew;
+    v[0] = *reinterpret_cast<const float4*>(gs_bytes + skew_addr<0>(base));
+    v[1] = *reinterpret_cast<const float4*>(gs_bytes + skew_addr<1>(base));
+    v[2] = *reinterpret_cast<const float4*>(gs_bytes + skew_addr<2>(base));
+    v[3] = *reinterpret_cast<const float4*>(gs_bytes + skew_addr<3>(base));
+    v[4] = *reinterpret_cast<const float4*>(gs_bytes + skew_addr<4>(base));
+    v[5] = *reinterpret_cast<const float4*>(gs_bytes + skew_addr<5>(base));
+    v[6] = *reinterpret_cast<const float4*>(gs_bytes + skew_addr<6>(base));
+    v[7] = *reinterpret_cast<const float4*>(gs_bytes + skew_addr<7>(base));
 }
-
-__device__ __forceinline__ void igrad_entry(const char* __restrict__ gs_bytes, unsigned e, float wv, unsigned skew,
-                                            float (&acc)[32]) {
-    const unsigned base = ((e & 1023u) << 7) | skew;
-    igrad_step<0>(gs_bytes, base, wv, acc); igrad_step<1>(gs_bytes, base, wv, acc);
-    igrad_step<2>(gs_bytes, base, wv, acc); igrad_step<3>(gs_bytes, base, wv, acc);
-    igrad_step<4>(gs_bytes, base, wv, acc); igrad_step<5>(gs_bytes, base, wv, acc);
-    igrad_step<6>(gs_bytes, base, wv, acc); igrad_step<7>(gs_bytes, base, wv, acc);
+// ... and the 32 multiply-adds that consume them.
+__device__ __forceinline__ void igrad_fmas(const float4 (&v)[8], float wv, float (&acc)[32]) {
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        acc[4 * c + 0] = fmaf(wv, v[c].x, acc[4 * c + 0]);
+        acc[4 * c + 1] = fmaf(wv, v[c].y, acc[4 * c + 1]);
+        acc[4 * c + 2] = fmaf(wv, v[c].z, acc[4 * c + 2]);
+        acc[4 * c + 3] = fmaf(wv, v[c].w, acc[4 * c + 3]);
+    }
 }
 
 // partial[stream][n][b] over the stream's tiles.  grid = streams * batch tiles.
-__global__ __launch_bounds__(1024) void igrad_tile_kernel(const unsigned* __restrict__ ent, const float* __restrict__ wp,
+// MAXT: largest workgroup the instantiation is launched with (sets the register budget);
+// LPT: labels of a tile staged per thread (tile_labels <= LPT * blockDim.x).
+template <int MAXT, int LPT>
+__global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned* __restrict__ ent, const float* __restrict__ wp,
                                   const unsigned* __restrict__ slice_off, const unsigned short* __restrict__ col_len,
                                   const float* __restrict__ g, float* __restrict__ partial, int B, int L,
                                   int tile_labels, int tiles, int tiles_per_stream, int nbt) {
@@ -130,33 +138,45 @@ __global__ __launch_bounds__(1024) void igrad_tile_kernel(const unsigned* __rest
     for (int t = t_begin; t < t_end; ++t) {
         const int j0 = t * tile_labels;
         const int nl = min(tile_labels, L - j0);
-        __syncthreads();                       // the previous tile is no longer being read
-        // stage gs[jl][c] = g[b0+c][j0+jl]: coalesced loads along labels, then 16-byte LDS writes
-        // whose chunk order is skewed by the label id (no bank conflicts)
-        for (int jl = threadIdx.x; jl < nl; jl += nthreads) {
-            float gb[32];
-            load_rows32(g, L, b0, B, (unsigned)(j0 + jl), gb);
-            const int r = jl & 7;
-            xor_permute_groups(gb, r);
-            char* rowp = gs_bytes + ((unsigned)jl << 7);
+        // out_grad rows of this tile: requested before the barrier, so the loads are in flight
+        // while the slower wavefronts finish the previous tile
+        float gbn[LPT][32];
 #pragma unroll
-            for (int c = 0; c < 8; ++c)
-                *reinterpret_cast<float4*>(rowp + ((c ^ r) << 4)) = make_float4(gb[4 * c], gb[4 * c + 1], gb[4 * c + 2], gb[4 * c + 3]);
+        for (int p = 0; p < LPT; ++p) {
+            const int jl = (int)threadIdx.x + p * nthreads;
+            if (jl < nl) load_rows32(g, L, b0, B, (unsigned)(j0 + jl), gbn[p]);
+        }
+        __syncthreads();                       // the previous tile is no longer being read
+        // row `tile_labels` is all zero: the target of padding slots
+        if (t == t_begin && threadIdx.x < 32) gs[tile_labels * kTileBatch + threadIdx.x] = 0.f;
+        // gs[jl][c] = g[b0+c][j0+jl]: the rows were loaded coalesced along labels; 16-byte LDS writes
+        // whose chunk order is skewed by the label id (no bank conflicts)
+#pragma unroll
+        for (int p = 0; p < LPT; ++p) {
+            const int jl = (int)threadIdx.x + p * nthreads;
+            if (jl < nl) {
+                const int r = jl & 7;
+                xor_permute_groups(gbn[p], r);
+                char* rowp = gs_bytes + ((unsigned)jl << 7);
+#pragma unroll
+                for (int c = 0; c < 8; ++c)
+                    *reinterpret_cast<float4*>(rowp + ((c ^ r) << 4)) =
+                        make_float4(gbn[p][4 * c], gbn[p][4 * c + 1], gbn[p][4 * c + 2], gbn[p][4 * c + 3]);
+            }
         }
         __syncthreads();
         const size_t sl = (size_t)t * (nthreads >> 6) + wave;
         const unsigned row0 = __builtin_amdgcn_readfirstlane(slice_off[sl]);
         const unsigned rows = __builtin_amdgcn_readfirstlane(slice_off[sl + 1]) - row0;
-        const unsigned len = col_len[(size_t)t * nthreads + threadIdx.x];
         const unsigned* ep = ent + (size_t)row0 * 64 + lane;
         const float* wpp = wp + (size_t)row0 * 64 + lane;
-        // slots are read four rows ahead of the multiply-adds that use them
+        if (rows == 0) continue;               // wave-uniform: no column of this slice is used in the tile
+        // Slots are fetched from memory kAhead rows ahead of the multiply-adds that use them (row
+        // indices clamped, not predicated, so the loads carry no branches).
         constexpr int kAhead = 4;
+        const unsigned last = rows - 1;
         unsigned e4[kAhead];
         float w4[kAhead];
-        // (row indices are clamped instead of predicated, so that the loads carry no branches)
-        if (rows == 0) continue;               // wave-uniform: no column of this slice is used in the tile
-        const unsigned last = rows - 1;
 #pragma unroll
         for (int q = 0; q < kAhead; ++q) {
             const unsigned r = min((unsigned)q, last);
@@ -172,9 +192,17 @@ __global__ __launch_bounds__(1024) void igrad_tile_kernel(const unsigned* __rest
                 en[q] = ep[(size_t)r * 64];
                 wn[q] = wpp[(size_t)r * 64];
             }
+            // branch-free: padding slots carry weight 0 and point at the all-zero LDS row, rows past
+            // the end of the slice are redirected there too
 #pragma unroll
-            for (int q = 0; q < kAhead; ++q)
-                if (i + q < len) igrad_entry(gs_bytes, e4[q], w4[q], skew, acc);
+            for (int q = 0; q < kAhead; ++q) {
+                const bool in = i + q < rows;                       // wave-uniform
+                const unsigned e = in ? e4[q] : (unsigned)tile_labels;
+                const float wv = in ? w4[q] : 0.f;
+                float4 xv[8];
+                igrad_reads(gs_bytes, e, skew, xv);
+                igrad_fmas(xv, wv, acc);
+            }
 #pragma unroll
             for (int q = 0; q < kAhead; ++q) { e4[q] = en[q]; w4[q] = wn[q]; }
         }
@@ -259,10 +287,22 @@ int launch_tiled(const ffi_plan* p, const float* w, const float* g, float* gx, i
     FFI_TRY(workspace_get(s, kWsPartials, (size_t)streams * p->threads * bpad * sizeof(float), (void**)&partial));
     hipLaunchKernelGGL(igrad_permute_weights_kernel, dim3(p->tiles), dim3(p->threads), 0, s, p->ent, p->slice_off,
                        p->col_len, w, wp, p->L, p->K, p->tile_labels);
-    const size_t lds = tile_lds_bytes(p->tile_labels);
-    FFI_HIP_TRY(hipFuncSetAttribute((const void*)igrad_tile_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(igrad_tile_kernel, dim3(streams * nbt), dim3(p->threads), lds, s, p->ent, wp, p->slice_off,
-                       p->col_len, g, partial, B, p->L, p->tile_labels, p->tiles, tps, nbt);
+    const size_t lds = tile_lds_bytes(p->tile_labels + 1);      // + the all-zero row
+    const dim3 grid(streams * nbt), block(p->threads);
+#define FFI_LAUNCH_TILE(MAXT, LPT)                                                                                      \
+    do {                                                                                                                \
+        FFI_HIP_TRY(hipFuncSetAttribute((const void*)igrad_tile_kernel<MAXT, LPT>,                                      \
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));                        \
+        hipLaunchKernelGGL((igrad_tile_kernel<MAXT, LPT>), grid, block, lds, s, p->ent, wp, p->slice_off, p->col_len, g, \
+                           partial, B, p->L, p->tile_labels, p->tiles, tps, nbt);                                       \
+    } while (0)
+    // the plan sizes its tiles so that one of these fits: tile_labels <= LPT * threads
+    if (p->threads <= 768) {
+        if (p->tile_labels <= p->threads) FFI_LAUNCH_TILE(768, 1); else FFI_LAUNCH_TILE(768, 2);
+    } else {
+        FFI_LAUNCH_TILE(1024, 1);
+    }
+#undef FFI_LAUNCH_TILE
     dim3 rgrid((B + 255) / 256, p->N);
     if (tp)
         hipLaunchKernelGGL(igrad_reduce_kernel<true>, rgrid, dim3(256), 0, s, partial, gx, B, p->N, streams, p->threads, bpad);

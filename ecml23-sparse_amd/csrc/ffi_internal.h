@@ -78,7 +78,8 @@ struct ffi_plan {
     long long total_rows = 0; // rows of 64 entries over all slices
     unsigned* slice_off = nullptr;       // [tiles*slices + 1] first row of each slice
     unsigned short* col_len = nullptr;   // [tiles][threads] connections of each column in each tile
-    unsigned* ent = nullptr;             // [total_rows*64]  (local position << 10) | local label
+    unsigned* ent = nullptr;             // [total_rows*64]  (position in tile << 11) | label in tile;
+                                         // padding slots hold label == tile_labels (an all-zero row)
     // global form
     int32_t* perm = nullptr;
     int32_t* col_ptr = nullptr;
@@ -88,7 +89,9 @@ struct ffi_plan {
 };
 
 namespace ffi {
-constexpr int kPlanTileLabels = 1024;     // local label ids fit 10 bits, a [1024][32] fp32 tile fits LDS
+constexpr int kPlanTileLabels = 1024;     // a [1024+1][32] fp32 tile fits LDS
+constexpr int kEntLabelBits = 11;         // label-in-tile field of a plan slot (values 0..1024)
+constexpr unsigned kEntLabelMask = (1u << kEntLabelBits) - 1;
 int plan_build(ffi_plan* p, const int32_t* lookup, hipStream_t s);
 int plan_fingerprint(ffi_plan* p, const int32_t* lookup, hipStream_t s, unsigned long long* out,
                      unsigned long long* bad_ids);

@@ -69,6 +69,10 @@ __global__ __launch_bounds__(kBlock) void fingerprint_kernel(const int32_t* __re
     }
 }
 
+__global__ __launch_bounds__(kBlock) void fill_u32_kernel(unsigned* p, size_t n, unsigned value) {
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) p[i] = value;
+}
+
 __global__ __launch_bounds__(kBlock) void zero_u64_kernel(unsigned long long* p, int n) {
     const int i = blockIdx.x * kBlock + threadIdx.x;
     if (i < n) p[i] = 0;
@@ -121,7 +125,7 @@ __global__ __launch_bounds__(1024) void slice_scan_kernel(const unsigned* __rest
 // One workgroup per label tile, one thread per column n.  The tile's column ids pass through LDS
 // in chunks; every thread scans them in flat-position order and appends the ones equal to its
 // column, so the connections of a column end up in ascending position: deterministic and stable
-// without any sort.  ent = (position inside the tile << 10) | label inside the tile.
+// without any sort.  ent = (position inside the tile << 11) | label inside the tile.
 constexpr int kFillChunk = 8192;
 __global__ void tile_fill_kernel(const int32_t* __restrict__ idx, int L, int K, int tile_labels,
                                  const unsigned* __restrict__ slice_off, unsigned* __restrict__ ent) {
@@ -143,7 +147,7 @@ __global__ void tile_fill_kernel(const int32_t* __restrict__ idx, int L, int K, 
         __syncthreads();
         for (int e = 0; e < n; ++e) {
             if (keys[e] == mine) {
-                dst[(size_t)count * 64] = ((unsigned)(c0 + e) << 10) | (unsigned)label;
+                dst[(size_t)count * 64] = ((unsigned)(c0 + e) << kEntLabelBits) | (unsigned)label;
                 ++count;
             }
             if (++kk == K) { kk = 0; ++label; }
@@ -196,8 +200,10 @@ bool dev_alloc(T** ptr, size_t count) {
 // three times the connection count (heavily skewed column usage): the caller then builds the
 // global form instead.
 int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
-    const int TL = std::min(kPlanTileLabels, p->L);
     const int threads = ((p->N + 63) / 64) * 64;
+    // every thread of the kernel that walks the plan stages at most two labels of a tile (one when
+    // the workgroup is larger than 768 threads and registers are scarcer)
+    const int TL = std::min(std::min(kPlanTileLabels, p->L), threads > 768 ? threads : 2 * threads);
     const int slices = threads / 64;
     const int tiles = (p->L + TL - 1) / TL;
     const size_t nslices = (size_t)tiles * slices;
@@ -220,8 +226,8 @@ int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     const unsigned long long connections = (unsigned long long)p->L * p->K;
     if (rows * 64ull > 3ull * connections + 64ull * nslices || rows >= 0xffffffffull) return FFI_OK;   // too skewed
     if (!dev_alloc(&p->ent, (size_t)rows * 64)) return FFI_ERR_OUT_OF_MEMORY;
-    e = hipMemsetAsync(p->ent, 0, std::max<size_t>((size_t)rows * 64, 1) * sizeof(unsigned), s);
-    if (e != hipSuccess) return hip_fail(e);
+    // every slot starts as padding: position 0, label TL (the all-zero row of the walking kernel)
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(1024), dim3(kBlock), 0, s, p->ent, (size_t)rows * 64, (unsigned)TL);
     hipLaunchKernelGGL(tile_fill_kernel, dim3(tiles), dim3(threads), 0, s, lookup, p->L, p->K, TL, p->slice_off, p->ent);
     e = hipGetLastError();
     if (e == hipSuccess) e = hipStreamSynchronize(s);
@@ -291,9 +297,9 @@ int plan_build(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     // a rebuild replaces the arrays: whatever still reads the old ones must have drained
     if (p->perm || p->ent) FFI_HIP_TRY(hipDeviceSynchronize());
     free_arrays(p);
-    // tiled form: one thread per column (N <= 1024) and positions inside a tile in 22 bits
+    // tiled form: one thread per column (N <= 1024) and positions inside a tile in 21 bits
     // (and 32 rows of out_grad within 32-bit byte offsets, as the kernels' buffer loads need)
-    if (p->N <= 1024 && (long long)kPlanTileLabels * p->K < (1ll << 22) && p->L < (1 << 25)) {
+    if (p->N <= 1024 && (long long)kPlanTileLabels * p->K < (1ll << (32 - kEntLabelBits)) && p->L < (1 << 25)) {
         int st = build_tiled(p, lookup, s);
         if (st != FFI_OK) { free_arrays(p); return st; }
     }

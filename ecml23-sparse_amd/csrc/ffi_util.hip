@@ -1,4 +1,4 @@
-// Small helpers: workspace pool, device properties, matrix transpose, LDS-tile launch geometry.
+// Small helpers: workspace pool, device properties, matrix transpose.
 #include "ffi_internal.h"
 #include "ffi_lds_tile.h"
 
@@ -104,20 +104,6 @@ int launch_transpose(const float* src, float* dst, int rows, int cols, hipStream
     if (grid.y > 65535u) return FFI_ERR_TOO_LARGE;
     hipLaunchKernelGGL(transpose_kernel, grid, dim3(kTrTile * 8), 0, s, src, dst, rows, cols);
     FFI_HIP_TRY(hipGetLastError());
-    return FFI_OK;
-}
-
-int tile_grid(int B, int L, TileGrid* out) {
-    const int cus = device_cu_count();
-    const int nbt = (B + kTileBatch - 1) / kTileBatch;
-    const int total_groups = (L + kLabelsPerWave - 1) / kLabelsPerWave;
-    const int waves = kTileThreads / 64;
-    int streams = std::max(1, cus / nbt);
-    streams = std::min(streams, std::max(1, (total_groups + waves - 1) / waves));
-    out->nbt = nbt;
-    out->groups_per_stream = (total_groups + streams - 1) / streams;
-    streams = (total_groups + out->groups_per_stream - 1) / out->groups_per_stream;
-    out->blocks = nbt * streams;
     return FFI_OK;
 }
 

@@ -131,6 +131,77 @@ def test_layouts_agree(ffi, shape):
     assert np.abs(gx - gxt.T).max() < 1.5e-5 and np.abs(gw - gwt).max() < 1.5e-5
 
 
+# shapes that steer the library through each of its code paths:
+#   narrow inputs (LDS tile kernels), wide inputs (generic kernels), the tiled and the global plan,
+#   partly filled batch tiles, fan-ins below / across / beyond the 32-connection register chunk,
+#   fewer labels than one tile, more than 1024 columns (global plan with tile forward/weight-grad)
+PATH_SHAPES = [
+    (300, 700, 5000, 32),      # 10 batch tiles, the last one partly filled
+    (33, 96, 9, 5),            # fewer labels than lanes, odd fan-in
+    (64, 1100, 3000, 12),      # N > 1024: tile forward / weight-grad, global plan
+    (40, 1216, 2500, 36),      # largest N that still fits the LDS tile
+    (48, 1300, 2000, 20),      # wide: generic kernels
+    (7, 64, 70000, 3),         # many tiles of a tiny column set
+    (128, 512, 4100, 100),     # four register chunks per label, tail of 4
+]
+
+
+@pytest.mark.parametrize("shape", PATH_SHAPES)
+@pytest.mark.parametrize("transposed", [False, True])
+def test_code_paths(ffi, shape, transposed):
+    B, N, L, K = shape
+    x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=B + N)
+    xin = np.ascontiguousarray(x.T) if transposed else x
+    print(f"case shape={shape} transposed={transposed}", flush=True)
+    out = hip_forward(ffi, xin, lookup, w, transposed)
+    gx, gw = hip_backward(ffi, xin, lookup, w, g, transposed)
+    assert rel_err(out, oracle.forward(xin, lookup, w, transposed=transposed)) <= FWD_RTOL
+    o_gx, o_gw = oracle.backward(xin, lookup, w, g, transposed=transposed)
+    assert rel_err(gw, o_gw) <= GRAD_RTOL
+    assert rel_err(gx, o_gx) <= GRAD_RTOL
+
+
+def test_skewed_lookup_uses_the_global_plan(ffi):
+    # every connection points at one of two columns: the padded tiled plan would explode, the
+    # library must fall back to the global column order and still be exact to tolerance
+    B, N, L, K = 40, 200, 6000, 8
+    x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=77)
+    lookup = np.where(lookup % 2 == 0, 3, 150).astype(np.int32)
+    gx, gw = hip_backward(ffi, x, lookup, w, g, False)
+    t_gx = oracle.input_grad(x, lookup, w, g, f64=True)
+    assert rel_err(gx, t_gx) <= GRAD_RTOL
+    assert np.array_equal(gx[:, [0, 1, 2, 4, 149, 151]], np.zeros((B, 6), dtype=np.float32))
+    assert rel_err(gw, oracle.weight_grad(x, lookup, w, g)) <= GRAD_RTOL
+    assert rel_err(hip_forward(ffi, x, lookup, w, False), oracle.forward(x, lookup, w)) <= FWD_RTOL
+
+
+def test_unaligned_buffers(ffi):
+    # pointers that are only 4-byte aligned take the scalar-load variants of the kernels
+    B, N, L, K = 64, 128, 1500, 32
+    x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=88)
+    lib = ffi._lib.lib()
+
+    def shifted(a):
+        flat = torch.empty(a.size + 1, dtype=torch.from_numpy(a).dtype, device="cuda")
+        view = flat[1:].view(*a.shape)
+        view.copy_(torch.from_numpy(a))
+        return flat, view
+
+    keep = [shifted(a) for a in (x, lookup, w, g)]
+    dx, dl, dw, dg = (v for _, v in keep)
+    assert dw.data_ptr() % 16 == 4
+    fo, out = shifted(np.zeros((B, L), np.float32))
+    fgx, gx = shifted(np.zeros((B, N), np.float32))
+    fgw, gw = shifted(np.zeros((L, K), np.float32))
+    ffi._lib.check(lib.ffi_forward_f32(dx.data_ptr(), dl.data_ptr(), dw.data_ptr(), out.data_ptr(), B, N, L, K, 0, stream()))
+    ffi._lib.check(lib.ffi_backward_f32(dx.data_ptr(), dl.data_ptr(), dw.data_ptr(), dg.data_ptr(), gx.data_ptr(),
+                                        gw.data_ptr(), B, N, L, K, 0, stream()))
+    torch.cuda.synchronize()
+    assert rel_err(out.cpu().numpy(), oracle.forward(x, lookup, w)) <= FWD_RTOL
+    o_gx, o_gw = oracle.backward(x, lookup, w, g)
+    assert rel_err(gx.cpu().numpy(), o_gx) <= GRAD_RTOL and rel_err(gw.cpu().numpy(), o_gw) <= GRAD_RTOL
+
+
 SCALED_CONFIGS = [
     # (config, labels used here) — same B, N, K and input laws as the benchmark configurations,
     # label count cut so that the CPU oracle finishes in seconds
