@@ -24,6 +24,7 @@ SOURCES = [
     "ffi_input_grad.hip",
     "ffi_plan.hip",
     "ffi_util.hip",
+    "ffi_wide.hip",
 ]
 
 # gfx950 only.  Packed-fp32 VALU forms are switched off for all device code.

@@ -50,6 +50,9 @@ int launch_forward(const float* x, const int32_t* idx, const float* w, float* ou
                    hipStream_t s);
 int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float* gw, const Dims& d,
                        hipStream_t s);
+// any shape (the tile kernels cover narrow inputs only)
+int launch_forward_wide(const float* x, const int32_t* idx, const float* w, float* out, const Dims& d, hipStream_t s);
+int launch_weight_grad_wide(const float* x, const int32_t* idx, const float* g, float* gw, const Dims& d, hipStream_t s);
 
 }  // namespace ffi
 
@@ -62,8 +65,9 @@ int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float
 // the slice.  Inside a column the connections are in ascending flat position, the order the
 // reference's CPU kernel accumulates in (tfsparse/cc/kernels/backward.cpp:64-72).
 //
-// tiled == false (any shape): a global CSC, perm[e] = flat position of the e-th connection in
-// (column, position) order, col_ptr[n]..col_ptr[n+1] the connections of column n.
+// tiled == false (any shape): a CSC per block of `block_labels` labels.  perm[e] = flat position of
+// the e-th connection in (label block, column, position) order;
+// col_ptr[blk*N + n] .. col_ptr[blk*N + n + 1] are the connections of column n inside block blk.
 struct ffi_plan {
     int device = -1;
     int L = 0, K = 0, N = 0;
@@ -80,7 +84,9 @@ struct ffi_plan {
     unsigned short* col_len = nullptr;   // [tiles][threads] connections of each column in each tile
     unsigned* ent = nullptr;             // [total_rows*64]  (position in tile << 11) | label in tile;
                                          // padding slots hold label == tile_labels (an all-zero row)
-    // global form
+    // blocked global form
+    int block_labels = 0;     // labels per block (bounds the part of out_grad that is live at a time)
+    int nblocks = 0;
     int32_t* perm = nullptr;
     int32_t* col_ptr = nullptr;
     unsigned long long* d_scratch = nullptr;  // fingerprint / counters (device)
@@ -98,6 +104,7 @@ int plan_fingerprint(ffi_plan* p, const int32_t* lookup, hipStream_t s, unsigned
 void plan_free(ffi_plan* p);
 int launch_input_grad(const ffi_plan* p, const float* w, const float* g, float* gx, int B, bool tp,
                       hipStream_t s);
+int launch_input_grad_wide(const ffi_plan* p, const float* w, const float* g, float* gx, int B, bool tp, hipStream_t s);
 }  // namespace ffi
 
 #endif  // FFI_INTERNAL_H

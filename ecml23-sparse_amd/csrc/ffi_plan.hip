@@ -155,9 +155,9 @@ __global__ void tile_fill_kernel(const int32_t* __restrict__ idx, int L, int K, 
     }
 }
 
-// ---- global form --------------------------------------------------------------------------------
+// ---- blocked global form ------------------------------------------------------------------------
 
-// col_ptr[n] = first position in the sorted key array whose key is >= n (n in [0,N]).
+// col_ptr[n] = first position in the sorted key array whose key is >= n (n in [0,N]; N = number of keys).
 __global__ __launch_bounds__(kBlock) void col_ptr_kernel(const unsigned* __restrict__ sorted_keys,
                                                           int total, int N, int32_t* __restrict__ col_ptr) {
     const int n = blockIdx.x * kBlock + threadIdx.x;
@@ -239,38 +239,58 @@ int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     return FFI_OK;
 }
 
+// key[p] = (label block of p) * N + column id of p
+__global__ __launch_bounds__(kBlock) void block_key_kernel(const int32_t* __restrict__ idx, int total, int K, int N,
+                                                           int block_labels, unsigned* __restrict__ key) {
+    const int p = blockIdx.x * kBlock + threadIdx.x;
+    if (p >= total) return;
+    const int j = p / K;
+    key[p] = (unsigned)(j / block_labels) * (unsigned)N + (unsigned)idx[p];
+}
+
+constexpr int kPlanBlockLabels = 65536;
+
 int build_global(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     const int total = p->L * p->K;  // validated to fit int32 by the caller
-    if (!dev_alloc(&p->perm, (size_t)total) || !dev_alloc(&p->col_ptr, (size_t)p->N + 1)) return FFI_ERR_OUT_OF_MEMORY;
+    const int nblocks = (p->L + kPlanBlockLabels - 1) / kPlanBlockLabels;
+    const long long nkeys = (long long)nblocks * p->N;
+    if (nkeys >= (1ll << 31)) return FFI_ERR_TOO_LARGE;
+    if (!dev_alloc(&p->perm, (size_t)total) || !dev_alloc(&p->col_ptr, (size_t)nkeys + 1)) return FFI_ERR_OUT_OF_MEMORY;
+    unsigned* keys = nullptr;
     unsigned* sorted_keys = nullptr;
     void* temp = nullptr;
     size_t temp_bytes = 0;
-    const int end_bit = bits_for((unsigned)(p->N - 1));
+    const int end_bit = bits_for((unsigned)(nkeys - 1));
     rocprim::counting_iterator<int32_t> positions(0);
     auto cleanup = [&]() {
+        if (keys) (void)hipFree(keys);
         if (sorted_keys) (void)hipFree(sorted_keys);
         if (temp) (void)hipFree(temp);
     };
-    // stable LSD radix sort of (column id, flat position): positions stay ascending inside a column
-    hipError_t e = rocprim::radix_sort_pairs(nullptr, temp_bytes, (const unsigned*)lookup, sorted_keys, positions,
-                                             p->perm, (unsigned)total, 0, end_bit, s);
+    // stable LSD radix sort of ((block, column), flat position): positions stay ascending inside a column
+    hipError_t e = rocprim::radix_sort_pairs(nullptr, temp_bytes, keys, sorted_keys, positions, p->perm, (unsigned)total, 0,
+                                             end_bit, s);
     if (e != hipSuccess) return hip_fail(e);
-    if (hipMalloc(&sorted_keys, (size_t)total * sizeof(unsigned)) != hipSuccess ||
+    if (hipMalloc(&keys, (size_t)total * sizeof(unsigned)) != hipSuccess ||
+        hipMalloc(&sorted_keys, (size_t)total * sizeof(unsigned)) != hipSuccess ||
         hipMalloc(&temp, temp_bytes ? temp_bytes : 4) != hipSuccess) {
         (void)hipGetLastError();
         cleanup();
         return FFI_ERR_OUT_OF_MEMORY;
     }
-    e = rocprim::radix_sort_pairs(temp, temp_bytes, (const unsigned*)lookup, sorted_keys, positions, p->perm,
-                                  (unsigned)total, 0, end_bit, s);
+    hipLaunchKernelGGL(block_key_kernel, dim3((total + kBlock - 1) / kBlock), dim3(kBlock), 0, s, lookup, total, p->K, p->N,
+                       kPlanBlockLabels, keys);
+    e = rocprim::radix_sort_pairs(temp, temp_bytes, keys, sorted_keys, positions, p->perm, (unsigned)total, 0, end_bit, s);
     if (e != hipSuccess) { cleanup(); return hip_fail(e); }
-    hipLaunchKernelGGL(col_ptr_kernel, dim3((p->N + 1 + kBlock - 1) / kBlock), dim3(kBlock), 0, s, sorted_keys, total,
-                       p->N, p->col_ptr);
+    hipLaunchKernelGGL(col_ptr_kernel, dim3((unsigned)((nkeys + 1 + kBlock - 1) / kBlock)), dim3(kBlock), 0, s, sorted_keys,
+                       total, (int)nkeys, p->col_ptr);
     e = hipGetLastError();
     if (e == hipSuccess) e = hipStreamSynchronize(s);
     cleanup();
     if (e != hipSuccess) return hip_fail(e);
-    p->bytes = (size_t)total * sizeof(int32_t) + ((size_t)p->N + 1) * sizeof(int32_t);
+    p->block_labels = kPlanBlockLabels;
+    p->nblocks = nblocks;
+    p->bytes = (size_t)total * sizeof(int32_t) + ((size_t)nkeys + 1) * sizeof(int32_t);
     return FFI_OK;
 }
 
