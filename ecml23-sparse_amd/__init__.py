@@ -19,6 +19,9 @@ from .fixed_fan_in_ops import (  # noqa: E402
     fan_in_sparse_matmul_grad_tp,
     FanInSparseMatmul,
     FanInSparseMatmulTp,
+    fan_in_sparse_matmul_bf16,
+    fan_in_sparse_topk_bf16,
+    topk_scores,
 )
 
 __all__ = [
@@ -28,4 +31,7 @@ __all__ = [
     "fan_in_sparse_matmul_grad_tp",
     "FanInSparseMatmul",
     "FanInSparseMatmulTp",
+    "fan_in_sparse_matmul_bf16",
+    "fan_in_sparse_topk_bf16",
+    "topk_scores",
 ]

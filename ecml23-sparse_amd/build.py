@@ -25,6 +25,7 @@ SOURCES = [
     "ffi_plan.hip",
     "ffi_util.hip",
     "ffi_wide.hip",
+    "ffi_bf16.hip",
 ]
 
 # gfx950 only.  Packed-fp32 VALU forms are switched off for all device code.

@@ -166,6 +166,32 @@ int ffi_backward_f32(const float* features, const int32_t* lookup, const float* 
     return FFI_OK;
 }
 
+int ffi_forward_bf16_f32(const uint16_t* features, const int32_t* lookup, const uint16_t* weights, float* result,
+                         int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in, int transposed,
+                         ffi_stream_t stream) {
+    if (!features || !lookup || !weights || !result) return FFI_ERR_NULL_POINTER;
+    Dims d;
+    FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
+    return launch_forward_bf16(features, lookup, weights, result, d, (hipStream_t)stream);
+}
+
+int ffi_forward_topk_bf16(const uint16_t* features, const int32_t* lookup, const uint16_t* weights, float* topk_values,
+                          int32_t* topk_indices, int64_t batch, int64_t num_features, int64_t num_units,
+                          int64_t fan_in, int k, int transposed, ffi_stream_t stream) {
+    if (!features || !lookup || !weights || !topk_values || !topk_indices) return FFI_ERR_NULL_POINTER;
+    Dims d;
+    FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
+    return launch_forward_topk_bf16(features, lookup, weights, topk_values, topk_indices, k, d, (hipStream_t)stream);
+}
+
+int ffi_topk_f32(const float* scores, int64_t batch, int64_t num_units, int k, float* topk_values, int32_t* topk_indices,
+                 ffi_stream_t stream) {
+    if (!scores || !topk_values || !topk_indices) return FFI_ERR_NULL_POINTER;
+    if (batch <= 0 || num_units <= 0) return FFI_ERR_BAD_SHAPE;
+    if (batch >= INT32_MAX || num_units >= INT32_MAX) return FFI_ERR_TOO_LARGE;
+    return launch_topk_f32(scores, (int)batch, (int)num_units, k, topk_values, topk_indices, (hipStream_t)stream);
+}
+
 int ffi_plan_create(const int32_t* lookup, int64_t num_units, int64_t fan_in, int64_t num_features,
                     int64_t batch_hint, ffi_stream_t stream, ffi_plan** plan) {
     if (!lookup || !plan) return FFI_ERR_NULL_POINTER;

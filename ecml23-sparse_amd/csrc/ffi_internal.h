@@ -42,6 +42,13 @@ void workspace_clear(int device);
 size_t workspace_bytes(int device);
 int device_cu_count();
 
+// inference variant: bf16 features / weights (raw 16-bit patterns), fp32 accumulation
+int launch_forward_bf16(const unsigned short* features, const int32_t* idx, const unsigned short* w, float* out,
+                        const Dims& d, hipStream_t s);
+int launch_forward_topk_bf16(const unsigned short* features, const int32_t* idx, const unsigned short* w, float* values,
+                             int32_t* indices, int k, const Dims& d, hipStream_t s);
+int launch_topk_f32(const float* scores, int B, int L, int k, float* values, int32_t* indices, hipStream_t s);
+
 // dst[c][r] = src[r][c] for a row-major [rows, cols] matrix.
 int launch_transpose(const float* src, float* dst, int rows, int cols, hipStream_t s);
 

@@ -122,3 +122,72 @@ def fan_in_sparse_matmul(features, lookup, weights):
 def fan_in_sparse_matmul_tp(features, lookup, weights):
     """Op FanInSparseMatmulTp: as above with features given as ``[N,B]``; result is ``[B,L]``."""
     return FanInSparseMatmulTp.apply(features, lookup, weights)
+
+
+# ------------------------------------------------------------------------------------------------
+# Inference variant: bf16 features and weights, fp32 accumulation, optional fused top-k.
+# The reference registers its ops for float only (tfsparse/cc/kernels/register.cpp:79-109) and takes
+# top-k through tf.nn.top_k in its metrics (sparse/metrics.py:19); these functions have no op there.
+# ------------------------------------------------------------------------------------------------
+def _check_bf16_inputs(features, lookup, weights, transposed):
+    for name, t in (("features", features), ("lookup", lookup), ("weights", weights)):
+        if t.dim() != 2:
+            raise ValueError(f"{name} must have rank 2, got shape {tuple(t.shape)}")
+    if tuple(lookup.shape) != tuple(weights.shape):
+        raise ValueError(f"lookup {tuple(lookup.shape)} and weights {tuple(weights.shape)} must have equal shapes")
+    if features.dtype != torch.bfloat16 or weights.dtype != torch.bfloat16:
+        raise TypeError("features and weights must be bfloat16")
+    if lookup.dtype not in _INDEX_DTYPES:
+        raise TypeError("lookup must be int32 or uint32")
+    if not features.is_cuda:
+        raise RuntimeError("the HIP path needs device tensors; there is no CPU fallback in this package")
+    if lookup.device != features.device or weights.device != features.device:
+        raise RuntimeError("features, lookup and weights must live on the same device")
+    batch = features.shape[1] if transposed else features.shape[0]
+    num_features = features.shape[0] if transposed else features.shape[1]
+    num_units, fan_in = lookup.shape
+    return batch, num_features, num_units, fan_in
+
+
+def fan_in_sparse_matmul_bf16(features, lookup, weights, transposed=False):
+    """Scores ``[B,L]`` in fp32 from bf16 features (``[B,N]``, or ``[N,B]`` if ``transposed``) and weights."""
+    batch, num_features, num_units, fan_in = _check_bf16_inputs(features, lookup, weights, transposed)
+    features, lookup, weights = features.contiguous(), lookup.contiguous(), weights.contiguous()
+    with torch.cuda.device(features.device):
+        result = torch.empty((batch, num_units), dtype=torch.float32, device=features.device)
+        _lib.check(_lib.lib().ffi_forward_bf16_f32(
+            features.data_ptr(), lookup.data_ptr(), weights.data_ptr(), result.data_ptr(),
+            batch, num_features, num_units, fan_in, int(transposed), _stream_handle(features.device)))
+    return result
+
+
+def fan_in_sparse_topk_bf16(features, lookup, weights, k=5, transposed=False):
+    """``(values [B,k] fp32, labels [B,k] int32)`` of the k best scores per sample, best first.
+
+    Equal scores are ordered by ascending label; the score matrix is never materialised.
+    """
+    batch, num_features, num_units, fan_in = _check_bf16_inputs(features, lookup, weights, transposed)
+    features, lookup, weights = features.contiguous(), lookup.contiguous(), weights.contiguous()
+    with torch.cuda.device(features.device):
+        values = torch.empty((batch, k), dtype=torch.float32, device=features.device)
+        labels = torch.empty((batch, k), dtype=torch.int32, device=features.device)
+        _lib.check(_lib.lib().ffi_forward_topk_bf16(
+            features.data_ptr(), lookup.data_ptr(), weights.data_ptr(), values.data_ptr(), labels.data_ptr(),
+            batch, num_features, num_units, fan_in, int(k), int(transposed), _stream_handle(features.device)))
+    return values, labels
+
+
+def topk_scores(scores, k=5):
+    """Per-row top-k of an fp32 ``[B,L]`` score matrix, same ordering rule as above."""
+    if scores.dim() != 2 or scores.dtype != torch.float32:
+        raise TypeError("scores must be a float32 matrix")
+    if not scores.is_cuda:
+        raise RuntimeError("the HIP path needs device tensors; there is no CPU fallback in this package")
+    scores = scores.contiguous()
+    batch, num_units = scores.shape
+    with torch.cuda.device(scores.device):
+        values = torch.empty((batch, k), dtype=torch.float32, device=scores.device)
+        labels = torch.empty((batch, k), dtype=torch.int32, device=scores.device)
+        _lib.check(_lib.lib().ffi_topk_f32(scores.data_ptr(), batch, num_units, int(k), values.data_ptr(),
+                                           labels.data_ptr(), _stream_handle(scores.device)))
+    return values, labels

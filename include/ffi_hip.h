@@ -118,6 +118,30 @@ size_t ffi_cache_bytes(void);
 int ffi_check_lookup(const int32_t* lookup, int64_t num_units, int64_t fan_in, int64_t num_features,
                      ffi_stream_t stream);
 
+/*
+ * Inference variant (no counterpart in the reference, whose ops are registered for float only,
+ * tfsparse/cc/kernels/register.cpp:79-109): features and weights are bfloat16 (raw 16-bit
+ * patterns, same layouts as above), products are accumulated in fp32, result is fp32.
+ */
+int ffi_forward_bf16_f32(const uint16_t* features, const int32_t* lookup, const uint16_t* weights, float* result,
+                         int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in,
+                         int transposed, ffi_stream_t stream);
+
+/*
+ * The same forward pass fused with a per-sample top-k (1 <= k <= 8): topk_values / topk_indices are
+ * [batch, k], scores descending, equal scores ordered by ascending label (the rule of tf.nn.top_k,
+ * which the reference uses in sparse/metrics.py:19).  The [batch, num_units] score matrix is never
+ * written.  Rows with fewer than k labels are padded with (-inf, -1).
+ */
+int ffi_forward_topk_bf16(const uint16_t* features, const int32_t* lookup, const uint16_t* weights,
+                          float* topk_values, int32_t* topk_indices,
+                          int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in,
+                          int k, int transposed, ffi_stream_t stream);
+
+/* Per-row top-k (1 <= k <= 8) of an fp32 score matrix scores[batch, num_units], same ordering rule. */
+int ffi_topk_f32(const float* scores, int64_t batch, int64_t num_units, int k,
+                 float* topk_values, int32_t* topk_indices, ffi_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
