@@ -26,14 +26,14 @@ __device__ __forceinline__ int xcd_contiguous_block(int block, int nblocks) {
 // xs[r][c] = src[r*ld + c0 + c] for c < 32 (zero beyond column `ld`), r < rows.  src rows are read
 // in 128-byte pieces, LDS writes are conflict-free.  All of a thread's loads are issued before its
 // first LDS write, so the staging costs one memory round trip, not one per row.
-template <int THREADS>
+template <int THREADS, int INFLIGHT = 4>
 __device__ __forceinline__ void stage_rows32(float* __restrict__ xs, const float* __restrict__ src, int rows,
                                              int ld, int c0) {
     const bool vec = (ld % 4 == 0) && (c0 + kTileBatch <= ld) && (((uintptr_t)src & 15) == 0);
     if (vec) {
         // thread -> (row, 16-byte chunk): 8 threads per row
         constexpr int kRowsPerIter = THREADS / 8;
-        constexpr int kInFlight = 4;
+        constexpr int kInFlight = INFLIGHT;
         const int q = threadIdx.x & 7;
         const float* p = src + c0 + 4 * q;
         for (int r0 = threadIdx.x >> 3; r0 < rows; r0 += kRowsPerIter * kInFlight) {

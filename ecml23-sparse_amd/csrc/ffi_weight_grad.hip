@@ -4,122 +4,137 @@
 #include "ffi_internal.h"
 #include "ffi_lds_tile.h"
 
+#include <algorithm>
+
 namespace ffi {
 namespace {
 
 // ------------------------------------------------------------------------------------------------
-// Narrow-input kernel: lane <-> label, 32 connections of the label per pass held as 32 fp32
-// accumulators, xs[n][32 batch rows] in LDS.  A workgroup owns a range of labels and makes one
-// sweep over it per batch tile: xs is staged once per sweep, and inside a sweep there is no
-// barrier, so the wavefronts drift apart and the out_grad/idx loads of some overlap the LDS work of
-// the others.  The first sweep writes gw, every later sweep adds its partial sum to what the same
-// thread wrote before (plain read-modify-write: no atomics, fixed order, bit-reproducible).
-// Each lane reads whole 128-byte rows with the chunk order skewed by its lane id (see
+// Narrow-input kernel, register-resident partial sums.  xs[n][32 batch rows] of one batch tile sits
+// in LDS.  A unit is (label, chunk of 32 connections); lane <-> unit.  A thread owns up to kResUnits
+// units for the whole kernel and keeps their 32 partial sums each in registers across ALL batch
+// tiles, so gw is written exactly once and never read (no atomics, fixed order, bit-reproducible);
+// per batch tile the workgroup re-stages xs and every thread re-reads the ids and the out_grad
+// column of its units.  512 threads per workgroup (two wavefronts per SIMD) leave 256 registers
+// per thread for this.  Inside a batch tile there is no barrier, so the wavefronts drift apart and
+// the loads of some overlap the LDS work of the others.  Workgroups [0,n1) own upb1 units each, the
+// others upb2 each: one launch covers a first round of full workgroups and a second set that shares
+// the remainder evenly.
+// Each lane reads whole 128-byte rows of xs with the chunk order skewed by its lane id (see
 // ffi_lds_tile.h), and out_grad is permuted in registers to match.
 // ------------------------------------------------------------------------------------------------
-constexpr int kWgChunk = 32;   // connections per register pass
+constexpr int kWgChunk = 32;        // connections per unit
+constexpr int kResThreads = 512;
+constexpr int kResUnits = 4;        // units per thread
 
-// acc += <row chunk C, gb group C>
-template <int C>
-__device__ __forceinline__ void wgrad_step(const char* __restrict__ xs_bytes, unsigned base, const float (&gb)[32],
-                                           float& acc) {
-    const float4 xv = *reinterpret_cast<const float4*>(xs_bytes + skew_addr<C>(base));
-    acc = fmaf(xv.x, gb[4 * C + 0], acc);
-    acc = fmaf(xv.y, gb[4 * C + 1], acc);
-    acc = fmaf(xv.z, gb[4 * C + 2], acc);
-    acc = fmaf(xv.w, gb[4 * C + 3], acc);
+// The eight 16-byte reads of one row, all issued before the first use ...
+__device__ __forceinline__ void wgrad_reads(const char* __restrict__ xs_bytes, unsigned base, float4 (&v)[8]) {
+    v[0] = *reinterpret_cast<const float4*>(xs_bytes + skew_addr<0>(base));
+    v[1] = *reinterpret_cast<const float4*>(xs_bytes + skew_addr<1>(base));
+    v[2] = *reinterpret_cast<const float4*>(xs_bytes + skew_addr<2>(base));
+    v[3] = *reinterpret_cast<const float4*>(xs_bytes + skew_addr<3>(base));
+    v[4] = *reinterpret_cast<const float4*>(xs_bytes + skew_addr<4>(base));
+    v[5] = *reinterpret_cast<const float4*>(xs_bytes + skew_addr<5>(base));
+    v[6] = *reinterpret_cast<const float4*>(xs_bytes + skew_addr<6>(base));
+    v[7] = *reinterpret_cast<const float4*>(xs_bytes + skew_addr<7>(base));
+}
+// ... and their dot product with the (equally skewed) out_grad values.
+__device__ __forceinline__ float wgrad_dot(const float4 (&v)[8], const float (&gb)[32], float acc) {
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        acc = fmaf(v[c].x, gb[4 * c + 0], acc);
+        acc = fmaf(v[c].y, gb[4 * c + 1], acc);
+        acc = fmaf(v[c].z, gb[4 * c + 2], acc);
+        acc = fmaf(v[c].w, gb[4 * c + 3], acc);
+    }
+    return acc;
 }
 
 template <bool VEC4>
-__global__ __launch_bounds__(kTileThreads) void wgrad_rows32_kernel(const float* __restrict__ xT,
-                                                                    const int32_t* __restrict__ idx,
-                                                                    const float* __restrict__ g,
-                                                                    float* __restrict__ gw, int B, int N,
-                                                                    int L, int K, int labels_per_block) {
+__global__ __launch_bounds__(kResThreads) void wgrad_resident_kernel(const float* __restrict__ xT,
+                                                                     const int32_t* __restrict__ idx,
+                                                                     const float* __restrict__ g,
+                                                                     float* __restrict__ gw, int B, int N,
+                                                                     int L, int K, int nchunks, int n1, int upb1,
+                                                                     int upb2) {
     extern __shared__ __align__(16) float xs[];
     const char* xs_bytes = reinterpret_cast<const char*>(xs);
     const int lane = threadIdx.x & 63;
-    const unsigned skew = (unsigned)(lane & 7) * 16u;
-    const int l_begin = blockIdx.x * labels_per_block;
-    const int l_end = min(l_begin + labels_per_block, L);
+    const int blk = blockIdx.x;
+    const long long total_units = (long long)L * nchunks;
+    const long long u_begin = blk < n1 ? (long long)blk * upb1 : (long long)n1 * upb1 + (long long)(blk - n1) * upb2;
+    const long long u_end = min(u_begin + (blk < n1 ? upb1 : upb2), total_units);
     const int nbt = (B + kTileBatch - 1) / kTileBatch;
-    const int nchunks = (K + kWgChunk - 1) / kWgChunk;
+
+    float res[kResUnits][kWgChunk];
+#pragma unroll
+    for (int q = 0; q < kResUnits; ++q)
+#pragma unroll
+        for (int k = 0; k < kWgChunk; ++k) res[q][k] = 0.f;
 
     for (int bt = 0; bt < nbt; ++bt) {
         const int b0 = bt * kTileBatch;
         __syncthreads();                                   // everyone is done with the previous tile
-        stage_rows32<kTileThreads>(xs, xT, N, B, b0);
+        stage_rows32<kResThreads, 8>(xs, xT, N, B, b0);
         __syncthreads();
-        for (int base = l_begin; base < l_end; base += kTileThreads) {
-            if (base + (int)(threadIdx.x & ~63u) >= l_end) break;   // nothing left for this wavefront
-            const int j = base + (int)threadIdx.x;
-            const bool valid = j < l_end;
-            const int jj = valid ? j : l_end - 1;          // keep loads in bounds
-            const int32_t* irow = idx + (size_t)jj * K;
-            float* grow = gw + (size_t)jj * K;
-            // out_grad of this label for the tile's 32 batch rows: coalesced across lanes
-            float gb[32];
-            load_rows32(g, L, b0, B, (unsigned)jj, gb);
-            xor_permute_groups(gb, lane & 7);              // match the skewed chunk order of the gathers
-            for (int ch = 0; ch < nchunks; ++ch) {
-                const int k0 = ch * kWgChunk;
-                const bool full = VEC4 && k0 + kWgChunk <= K;
-                // column ids of this pass, two 16-bit ids per register (ids < 2^16 on this path)
+        unsigned skew = (unsigned)(lane & 7) * 16u;
+        asm volatile("" : "+v"(skew));                     // keep the LDS addresses out of loop-invariant hoisting
+#pragma unroll
+        for (int q = 0; q < kResUnits; ++q) {
+            const long long ubase = u_begin + (long long)q * kResThreads;
+            if (ubase + (long long)(threadIdx.x & ~63u) < u_end) {          // the wavefront has units in this round
+                const long long u = min(ubase + (long long)threadIdx.x, u_end - 1);   // clamped: loads stay in bounds
+                const int j = (int)(u / nchunks);
+                const int k0 = (int)(u - (long long)j * nchunks) * kWgChunk;
+                const int32_t* irow = idx + (size_t)j * K + k0;
+                // out_grad of this label for the tile's 32 batch rows: coalesced across lanes
+                float gb[32];
+                load_rows32(g, L, b0, B, (unsigned)j, gb);
+                // column ids of the unit, two 16-bit ids per register (ids < 2^16 on this path)
                 unsigned idp[kWgChunk / 2];
-                float acc[kWgChunk];
-                if (full) {
+                if (VEC4 && k0 + kWgChunk <= K) {
 #pragma unroll
-                    for (int q = 0; q < kWgChunk / 4; ++q) {
-                        const int4 v = *reinterpret_cast<const int4*>(irow + k0 + 4 * q);
-                        idp[2 * q + 0] = (unsigned)v.x | ((unsigned)v.y << 16);
-                        idp[2 * q + 1] = (unsigned)v.z | ((unsigned)v.w << 16);
+                    for (int t = 0; t < kWgChunk / 4; ++t) {
+                        const int4 v = *reinterpret_cast<const int4*>(irow + 4 * t);
+                        idp[2 * t + 0] = (unsigned)v.x | ((unsigned)v.y << 16);
+                        idp[2 * t + 1] = (unsigned)v.z | ((unsigned)v.w << 16);
                     }
                 } else {
 #pragma unroll
-                    for (int q = 0; q < kWgChunk / 2; ++q) {
-                        const unsigned a = (k0 + 2 * q < K) ? (unsigned)irow[k0 + 2 * q] : 0u;
-                        const unsigned b = (k0 + 2 * q + 1 < K) ? (unsigned)irow[k0 + 2 * q + 1] : 0u;
-                        idp[q] = a | (b << 16);
+                    for (int t = 0; t < kWgChunk / 2; ++t) {
+                        const unsigned a = (k0 + 2 * t < K) ? (unsigned)irow[2 * t] : 0u;
+                        const unsigned b = (k0 + 2 * t + 1 < K) ? (unsigned)irow[2 * t + 1] : 0u;
+                        idp[t] = a | (b << 16);
                     }
                 }
-                // partial sums of the earlier batch tiles (written by this same thread)
-                if (bt == 0) {
-#pragma unroll
-                    for (int k = 0; k < kWgChunk; ++k) acc[k] = 0.f;
-                } else if (full) {
-#pragma unroll
-                    for (int q = 0; q < kWgChunk / 4; ++q) {
-                        const float4 v = *reinterpret_cast<const float4*>(grow + k0 + 4 * q);
-                        acc[4 * q] = v.x; acc[4 * q + 1] = v.y; acc[4 * q + 2] = v.z; acc[4 * q + 3] = v.w;
-                    }
-                } else {
-#pragma unroll
-                    for (int k = 0; k < kWgChunk; ++k) acc[k] = (k0 + k < K) ? grow[k0 + k] : 0.f;
-                }
+                xor_permute_groups(gb, lane & 7);          // match the skewed chunk order of the gathers
 #pragma unroll
                 for (int k = 0; k < kWgChunk; ++k) {
                     const unsigned id = (k & 1) ? (idp[k >> 1] >> 16) : (idp[k >> 1] & 0xffffu);
-                    const unsigned rb = (id << 7) | skew;
-                    wgrad_step<0>(xs_bytes, rb, gb, acc[k]);
-                    wgrad_step<1>(xs_bytes, rb, gb, acc[k]);
-                    wgrad_step<2>(xs_bytes, rb, gb, acc[k]);
-                    wgrad_step<3>(xs_bytes, rb, gb, acc[k]);
-                    wgrad_step<4>(xs_bytes, rb, gb, acc[k]);
-                    wgrad_step<5>(xs_bytes, rb, gb, acc[k]);
-                    wgrad_step<6>(xs_bytes, rb, gb, acc[k]);
-                    wgrad_step<7>(xs_bytes, rb, gb, acc[k]);
+                    float4 xv[8];
+                    wgrad_reads(xs_bytes, (id << 7) | skew, xv);
+                    __builtin_amdgcn_sched_barrier(0);
+                    res[q][k] = wgrad_dot(xv, gb, res[q][k]);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
-                if (valid) {
-                    if (full) {
+            }
+        }
+    }
 #pragma unroll
-                        for (int q = 0; q < kWgChunk / 4; ++q)
-                            *reinterpret_cast<float4*>(grow + k0 + 4 * q) = make_float4(acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]);
-                    } else {
+    for (int q = 0; q < kResUnits; ++q) {
+        const long long u = u_begin + (long long)q * kResThreads + threadIdx.x;
+        if (u < u_end) {
+            const int j = (int)(u / nchunks);
+            const int k0 = (int)(u - (long long)j * nchunks) * kWgChunk;
+            float* grow = gw + (size_t)j * K + k0;
+            if (VEC4 && k0 + kWgChunk <= K) {
 #pragma unroll
-                        for (int k = 0; k < kWgChunk; ++k)
-                            if (k0 + k < K) grow[k0 + k] = acc[k];
-                    }
-                }
+                for (int t = 0; t < kWgChunk / 4; ++t)
+                    *reinterpret_cast<float4*>(grow + 4 * t) = make_float4(res[q][4 * t], res[q][4 * t + 1], res[q][4 * t + 2], res[q][4 * t + 3]);
+            } else {
+#pragma unroll
+                for (int k = 0; k < kWgChunk; ++k)
+                    if (k0 + k < K) grow[k] = res[q][k];
             }
         }
     }
@@ -139,17 +154,30 @@ int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float
             xT = ws;
         }
         const int cus = device_cu_count();
-        // one workgroup per CU, equal label ranges (the last pass of a range may be partly filled)
-        const int per_block = (d.L + cus - 1) / cus;
-        const int blocks = (d.L + per_block - 1) / per_block;
+        // A first round of full workgroups (kResUnits units per thread), one per CU, as long as whole rounds
+        // fit; what is left is shared evenly by a second set of workgroups in the same launch.
+        const int nchunks = (d.K + kWgChunk - 1) / kWgChunk;
+        const long long units = (long long)d.L * nchunks;
+        const long long cap = (long long)kResUnits * kResThreads;      // units a workgroup can hold
+        const int n1 = (int)(units / (cap * cus)) * cus;
+        const long long rest = units - (long long)n1 * cap;
+        int n2 = 0, upb2 = 0;
+        if (rest > 0) {
+            const long long rounds = (rest + cap * cus - 1) / (cap * cus);
+            n2 = (int)std::min<long long>(rounds * cus, (rest + 63) / 64);
+            upb2 = (int)((rest + n2 - 1) / n2);
+            n2 = (int)((rest + upb2 - 1) / upb2);
+        }
+        const unsigned blocks = (unsigned)(n1 + n2);
+        const int upb = (int)cap;
         const size_t lds = tile_lds_bytes(d.N);
         const bool vec4 = (d.K % 4 == 0) && (((uintptr_t)gw | (uintptr_t)idx) % 16 == 0);
         if (vec4) {
-            FFI_HIP_TRY(hipFuncSetAttribute((const void*)wgrad_rows32_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-            hipLaunchKernelGGL(wgrad_rows32_kernel<true>, dim3(blocks), dim3(kTileThreads), lds, s, xT, idx, g, gw, d.B, d.N, d.L, d.K, per_block);
+            FFI_HIP_TRY(hipFuncSetAttribute((const void*)wgrad_resident_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+            hipLaunchKernelGGL(wgrad_resident_kernel<true>, dim3(blocks), dim3(kResThreads), lds, s, xT, idx, g, gw, d.B, d.N, d.L, d.K, nchunks, n1, upb, upb2);
         } else {
-            FFI_HIP_TRY(hipFuncSetAttribute((const void*)wgrad_rows32_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-            hipLaunchKernelGGL(wgrad_rows32_kernel<false>, dim3(blocks), dim3(kTileThreads), lds, s, xT, idx, g, gw, d.B, d.N, d.L, d.K, per_block);
+            FFI_HIP_TRY(hipFuncSetAttribute((const void*)wgrad_resident_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+            hipLaunchKernelGGL(wgrad_resident_kernel<false>, dim3(blocks), dim3(kResThreads), lds, s, xT, idx, g, gw, d.B, d.N, d.L, d.K, nchunks, n1, upb, upb2);
         }
         FFI_HIP_TRY(hipGetLastError());
         return FFI_OK;
