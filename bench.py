@@ -25,13 +25,13 @@ HBM_PEAK_GBPS = 8000.0        # MI355X published HBM3E peak
 # runs of this file (the factors are what the same counters read for a plain copy kernel of known
 # size); the summary with the commands is profiles/ffi_c2_counters.txt.  None where not measured.
 MEASURED_TRAFFIC_BYTES = {
-    "c2": {"forward": 557.9e6, "weight_grad": 1344.4e6, "input_grad": 1100.4e6},
+    "c2": {"forward": 556.9e6, "weight_grad": 775.6e6, "input_grad": 1100.4e6},
 }
 
 # GPU kernels behind each pass (one C-ABI call)
 PASS_KERNELS = {
     "forward": "fwd_lane32_kernel",
-    "weight_grad": "wgrad_rows32_kernel",
+    "weight_grad": "wgrad_resident_kernel",
     "input_grad": "igrad_permute_weights_kernel + igrad_tile_kernel + igrad_reduce_kernel",
 }
 
