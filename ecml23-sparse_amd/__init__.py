@@ -22,7 +22,11 @@ from .fixed_fan_in_ops import (  # noqa: E402
     fan_in_sparse_matmul_bf16,
     fan_in_sparse_topk_bf16,
     topk_scores,
+    fan_in_sparse_matmul_bias,
+    fan_in_sparse_matmul_tp_bias,
 )
+from . import custom_layer  # noqa: E402
+from .custom_layer import StratifiedRewireLayerV2, FixedFractionSelector, FixedMagnitudeSelector  # noqa: E402
 
 __all__ = [
     "fan_in_sparse_matmul",
@@ -34,4 +38,9 @@ __all__ = [
     "fan_in_sparse_matmul_bf16",
     "fan_in_sparse_topk_bf16",
     "topk_scores",
+    "fan_in_sparse_matmul_bias",
+    "fan_in_sparse_matmul_tp_bias",
+    "StratifiedRewireLayerV2",
+    "FixedFractionSelector",
+    "FixedMagnitudeSelector",
 ]

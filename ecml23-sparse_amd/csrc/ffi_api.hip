@@ -126,7 +126,16 @@ int ffi_forward_f32(const float* features, const int32_t* lookup, const float* w
     if (!features || !lookup || !weights || !result) return FFI_ERR_NULL_POINTER;
     Dims d;
     FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
-    return launch_forward(features, lookup, weights, result, d, (hipStream_t)stream);
+    return launch_forward(features, lookup, weights, nullptr, result, d, (hipStream_t)stream);
+}
+
+int ffi_forward_bias_f32(const float* features, const int32_t* lookup, const float* weights, const float* bias,
+                         float* result, int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in,
+                         int transposed, ffi_stream_t stream) {
+    if (!features || !lookup || !weights || !bias || !result) return FFI_ERR_NULL_POINTER;
+    Dims d;
+    FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
+    return launch_forward(features, lookup, weights, bias, result, d, (hipStream_t)stream);
 }
 
 int ffi_weight_grad_f32(const float* features, const int32_t* lookup, const float* out_grad,
@@ -135,7 +144,7 @@ int ffi_weight_grad_f32(const float* features, const int32_t* lookup, const floa
     if (!features || !lookup || !out_grad || !weight_grad) return FFI_ERR_NULL_POINTER;
     Dims d;
     FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
-    return launch_weight_grad(features, lookup, out_grad, weight_grad, d, (hipStream_t)stream);
+    return launch_weight_grad(features, lookup, out_grad, weight_grad, nullptr, d, (hipStream_t)stream);
 }
 
 int ffi_input_grad_f32(const int32_t* lookup, const float* weights, const float* out_grad,
@@ -160,6 +169,21 @@ int ffi_backward_f32(const float* features, const int32_t* lookup, const float* 
     if (weight_grad)
         FFI_TRY(ffi_weight_grad_f32(features, lookup, out_grad, weight_grad, batch, num_features, num_units, fan_in,
                                     transposed, stream));
+    if (feature_grad)
+        FFI_TRY(ffi_input_grad_f32(lookup, weights, out_grad, feature_grad, batch, num_features, num_units, fan_in,
+                                   transposed, stream));
+    return FFI_OK;
+}
+
+int ffi_backward_bias_f32(const float* features, const int32_t* lookup, const float* weights,
+                          const float* out_grad, float* feature_grad, float* weight_grad, float* bias_grad,
+                          int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in, int transposed,
+                          ffi_stream_t stream) {
+    if (!features || !lookup || !weights || !out_grad || !weight_grad || !bias_grad) return FFI_ERR_NULL_POINTER;
+    Dims d;
+    FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
+    // the bias gradient (column sums of out_grad) is a by-product of the weight-gradient kernel
+    FFI_TRY(launch_weight_grad(features, lookup, out_grad, weight_grad, bias_grad, d, (hipStream_t)stream));
     if (feature_grad)
         FFI_TRY(ffi_input_grad_f32(lookup, weights, out_grad, feature_grad, batch, num_features, num_units, fan_in,
                                    transposed, stream));

@@ -36,6 +36,7 @@ template <bool VEC4>
 __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* __restrict__ xT,
                                                                   const int32_t* __restrict__ idx,
                                                                   const float* __restrict__ w,
+                                                                  const float* __restrict__ bias,
                                                                   float* __restrict__ out, int B, int N,
                                                                   int L, int K, int nbt, int labels_per_stream) {
     extern __shared__ __align__(16) float xs[];
@@ -103,6 +104,11 @@ __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* _
             }
         }
         xor_permute_groups(acc, lane & 7);                 // back to natural batch order
+        if (bias != nullptr) {                             // added after the sum, as a separate bias_add would
+            const float bj = bias[jj];
+#pragma unroll
+            for (int i = 0; i < 32; ++i) acc[i] += bj;
+        }
         if (valid) {
             const unsigned lane_off = (unsigned)j * 4u;
             const unsigned stride = (unsigned)L * 4u;
@@ -115,7 +121,7 @@ __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* _
 
 }  // namespace
 
-int launch_forward(const float* x, const int32_t* idx, const float* w, float* out, const Dims& d,
+int launch_forward(const float* x, const int32_t* idx, const float* w, const float* bias, float* out, const Dims& d,
                    hipStream_t s) {
     // (the kernel reaches the 32 rows of out of a batch tile through 32-bit byte offsets)
     if (tile_path_fits(d.N) && d.L < (1 << 25)) {
@@ -136,15 +142,15 @@ int launch_forward(const float* x, const int32_t* idx, const float* w, float* ou
         const int blocks = streams * nbt;
         if (vec4) {
             FFI_HIP_TRY(hipFuncSetAttribute((const void*)fwd_lane32_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-            hipLaunchKernelGGL(fwd_lane32_kernel<true>, dim3(blocks), dim3(kTileThreads), lds, s, xT, idx, w, out, d.B, d.N, d.L, d.K, nbt, per_stream);
+            hipLaunchKernelGGL(fwd_lane32_kernel<true>, dim3(blocks), dim3(kTileThreads), lds, s, xT, idx, w, bias, out, d.B, d.N, d.L, d.K, nbt, per_stream);
         } else {
             FFI_HIP_TRY(hipFuncSetAttribute((const void*)fwd_lane32_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-            hipLaunchKernelGGL(fwd_lane32_kernel<false>, dim3(blocks), dim3(kTileThreads), lds, s, xT, idx, w, out, d.B, d.N, d.L, d.K, nbt, per_stream);
+            hipLaunchKernelGGL(fwd_lane32_kernel<false>, dim3(blocks), dim3(kTileThreads), lds, s, xT, idx, w, bias, out, d.B, d.N, d.L, d.K, nbt, per_stream);
         }
         FFI_HIP_TRY(hipGetLastError());
         return FFI_OK;
     }
-    return launch_forward_wide(x, idx, w, out, d, s);
+    return launch_forward_wide(x, idx, w, bias, out, d, s);
 }
 
 }  // namespace ffi

@@ -53,13 +53,16 @@ int launch_topk_f32(const float* scores, int B, int L, int k, float* values, int
 int launch_transpose(const float* src, float* dst, int rows, int cols, hipStream_t s);
 
 // ---- launchers (each validates nothing; callers pass validated Dims) ---------------------------
-int launch_forward(const float* x, const int32_t* idx, const float* w, float* out, const Dims& d,
+// bias ([L], added to every row of out) and bias_grad ([L], column sums of g) may be null
+int launch_forward(const float* x, const int32_t* idx, const float* w, const float* bias, float* out, const Dims& d,
                    hipStream_t s);
-int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float* gw, const Dims& d,
+int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float* gw, float* bias_grad, const Dims& d,
                        hipStream_t s);
 // any shape (the tile kernels cover narrow inputs only)
-int launch_forward_wide(const float* x, const int32_t* idx, const float* w, float* out, const Dims& d, hipStream_t s);
-int launch_weight_grad_wide(const float* x, const int32_t* idx, const float* g, float* gw, const Dims& d, hipStream_t s);
+int launch_forward_wide(const float* x, const int32_t* idx, const float* w, const float* bias, float* out, const Dims& d,
+                        hipStream_t s);
+int launch_weight_grad_wide(const float* x, const int32_t* idx, const float* g, float* gw, float* bias_grad, const Dims& d,
+                            hipStream_t s);
 
 }  // namespace ffi
 

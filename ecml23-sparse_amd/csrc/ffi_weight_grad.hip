@@ -54,7 +54,8 @@ template <bool VEC4>
 __global__ __launch_bounds__(kResThreads) void wgrad_resident_kernel(const float* __restrict__ xT,
                                                                      const int32_t* __restrict__ idx,
                                                                      const float* __restrict__ g,
-                                                                     float* __restrict__ gw, int B, int N,
+                                                                     float* __restrict__ gw,
+                                                                     float* __restrict__ bias_grad, int B, int N,
                                                                      int L, int K, int nchunks, int n1, int upb1,
                                                                      int upb2) {
     extern __shared__ __align__(16) float xs[];
@@ -71,6 +72,9 @@ __global__ __launch_bounds__(kResThreads) void wgrad_resident_kernel(const float
     for (int q = 0; q < kResUnits; ++q)
 #pragma unroll
         for (int k = 0; k < kWgChunk; ++k) res[q][k] = 0.f;
+    float gsum[kResUnits];                                 // column sums of out_grad (the bias gradient)
+#pragma unroll
+    for (int q = 0; q < kResUnits; ++q) gsum[q] = 0.f;
 
     for (int bt = 0; bt < nbt; ++bt) {
         const int b0 = bt * kTileBatch;
@@ -90,6 +94,12 @@ __global__ __launch_bounds__(kResThreads) void wgrad_resident_kernel(const float
                 // out_grad of this label for the tile's 32 batch rows: coalesced across lanes
                 float gb[32];
                 load_rows32(g, L, b0, B, (unsigned)j, gb);
+                if (bias_grad != nullptr) {
+                    float t = gsum[q];
+#pragma unroll
+                    for (int b = 0; b < 32; ++b) t += gb[b];
+                    gsum[q] = t;
+                }
                 // column ids of the unit, two 16-bit ids per register (ids < 2^16 on this path)
                 unsigned idp[kWgChunk / 2];
                 if (VEC4 && k0 + kWgChunk <= K) {
@@ -127,6 +137,7 @@ __global__ __launch_bounds__(kResThreads) void wgrad_resident_kernel(const float
             const int j = (int)(u / nchunks);
             const int k0 = (int)(u - (long long)j * nchunks) * kWgChunk;
             float* grow = gw + (size_t)j * K + k0;
+            if (bias_grad != nullptr && k0 == 0) bias_grad[j] = gsum[q];
             if (VEC4 && k0 + kWgChunk <= K) {
 #pragma unroll
                 for (int t = 0; t < kWgChunk / 4; ++t)
@@ -142,7 +153,7 @@ __global__ __launch_bounds__(kResThreads) void wgrad_resident_kernel(const float
 
 }  // namespace
 
-int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float* gw, const Dims& d,
+int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float* gw, float* bias_grad, const Dims& d,
                        hipStream_t s) {
     // (32 rows of out_grad must be reachable through 32-bit byte offsets)
     if (tile_path_fits(d.N) && d.L < (1 << 25)) {
@@ -174,15 +185,15 @@ int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float
         const bool vec4 = (d.K % 4 == 0) && (((uintptr_t)gw | (uintptr_t)idx) % 16 == 0);
         if (vec4) {
             FFI_HIP_TRY(hipFuncSetAttribute((const void*)wgrad_resident_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-            hipLaunchKernelGGL(wgrad_resident_kernel<true>, dim3(blocks), dim3(kResThreads), lds, s, xT, idx, g, gw, d.B, d.N, d.L, d.K, nchunks, n1, upb, upb2);
+            hipLaunchKernelGGL(wgrad_resident_kernel<true>, dim3(blocks), dim3(kResThreads), lds, s, xT, idx, g, gw, bias_grad, d.B, d.N, d.L, d.K, nchunks, n1, upb, upb2);
         } else {
             FFI_HIP_TRY(hipFuncSetAttribute((const void*)wgrad_resident_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-            hipLaunchKernelGGL(wgrad_resident_kernel<false>, dim3(blocks), dim3(kResThreads), lds, s, xT, idx, g, gw, d.B, d.N, d.L, d.K, nchunks, n1, upb, upb2);
+            hipLaunchKernelGGL(wgrad_resident_kernel<false>, dim3(blocks), dim3(kResThreads), lds, s, xT, idx, g, gw, bias_grad, d.B, d.N, d.L, d.K, nchunks, n1, upb, upb2);
         }
         FFI_HIP_TRY(hipGetLastError());
         return FFI_OK;
     }
-    return launch_weight_grad_wide(x, idx, g, gw, d, s);
+    return launch_weight_grad_wide(x, idx, g, gw, bias_grad, d, s);
 }
 
 }  // namespace ffi

@@ -32,7 +32,8 @@ __device__ __forceinline__ float wave_sum(float v) {
 // Results go through LDS so that out is written in 256-byte rows.
 __global__ __launch_bounds__(kWideThreads) void fwd_wide_kernel(const float* __restrict__ xT,
                                                                 const int32_t* __restrict__ idx,
-                                                                const float* __restrict__ w, float* __restrict__ out,
+                                                                const float* __restrict__ w,
+                                                                const float* __restrict__ bias, float* __restrict__ out,
                                                                 int B, int N, int L, int K) {
     __shared__ float tile[kWideLabels * kWideStride];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -81,9 +82,12 @@ __global__ __launch_bounds__(kWideThreads) void fwd_wide_kernel(const float* __r
     // out[b, j0 .. j0+63]: one wavefront writes one 256-byte row per step
     const int jl = threadIdx.x & 63;
     if (j0 + jl < L) {
+        const bool has_bias = bias != nullptr;
+        const float bj = has_bias ? bias[j0 + jl] : 0.f;
         for (int bb = threadIdx.x >> 6; bb < kWideBatch; bb += kWideThreads / 64) {
             const int b = bc0 + bb;
-            if (b < B) out[(size_t)b * L + j0 + jl] = tile[jl * kWideStride + bb];
+            const float v = tile[jl * kWideStride + bb];
+            if (b < B) out[(size_t)b * L + j0 + jl] = has_bias ? v + bj : v;
         }
     }
 }
@@ -96,10 +100,13 @@ __global__ __launch_bounds__(kWideThreads) void fwd_wide_kernel(const float* __r
 __global__ __launch_bounds__(kWideThreads) void wgrad_wide_kernel(const float* __restrict__ xT,
                                                                   const int32_t* __restrict__ idx,
                                                                   const float* __restrict__ g, float* __restrict__ gw,
-                                                                  int B, int N, int L, int K) {
+                                                                  float* __restrict__ bias_grad, int B, int N, int L,
+                                                                  int K) {
     extern __shared__ float smem[];
     float* gt = smem;                                   // [64 labels][129]
     float* res = smem + kWideLabels * kWideStride;      // [64 labels][K]
+    float* bres = res + kWideLabels * K;                // [64 labels] column sums of out_grad
+    if (threadIdx.x < kWideLabels) bres[threadIdx.x] = 0.f;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j0 = blockIdx.x * kWideLabels;
     const buffer_rsrc xr = make_rsrc(xT, (size_t)N * (size_t)B * sizeof(float));
@@ -125,6 +132,10 @@ __global__ __launch_bounds__(kWideThreads) void wgrad_wide_kernel(const float* _
             const int j = j0 + jl;
             if (j >= L) break;                                  // wave-uniform
             const float g0 = gt[jl * kWideStride + lane], g1 = gt[jl * kWideStride + 64 + lane];
+            if (bias_grad != nullptr) {                         // wave-uniform
+                const float gs = wave_sum(g0 + g1);
+                if (lane == 0) bres[jl] += gs;
+            }
             const int32_t* irow = idx + (size_t)j * K;
             for (int k0 = 0; k0 < K; k0 += 64) {
                 const int kn = min(64, K - k0);
@@ -162,6 +173,7 @@ __global__ __launch_bounds__(kWideThreads) void wgrad_wide_kernel(const float* _
         const int jl = t / K;
         if (j0 + jl < L) gw[(size_t)j0 * K + t] = res[t];
     }
+    if (bias_grad != nullptr && threadIdx.x < kWideLabels && j0 + (int)threadIdx.x < L) bias_grad[j0 + threadIdx.x] = bres[threadIdx.x];
 }
 
 // ---- input gradient -----------------------------------------------------------------------------
@@ -232,7 +244,8 @@ void magic_divisor(unsigned d, unsigned* mul, unsigned* shift) {
 
 bool wide_offsets_fit(long long rows, long long B) { return rows * B * 4 < (1ll << 32); }
 
-int launch_forward_wide(const float* x, const int32_t* idx, const float* w, float* out, const Dims& d, hipStream_t s) {
+int launch_forward_wide(const float* x, const int32_t* idx, const float* w, const float* bias, float* out, const Dims& d,
+                        hipStream_t s) {
     if (!wide_offsets_fit(d.N, d.B)) return FFI_ERR_TOO_LARGE;
     const float* xT = x;
     if (!d.tp) {
@@ -243,14 +256,15 @@ int launch_forward_wide(const float* x, const int32_t* idx, const float* w, floa
     }
     dim3 grid((d.L + kWideLabels - 1) / kWideLabels, (d.B + kWideBatch - 1) / kWideBatch);
     if (grid.y > 65535u) return FFI_ERR_TOO_LARGE;
-    hipLaunchKernelGGL(fwd_wide_kernel, grid, dim3(kWideThreads), 0, s, xT, idx, w, out, d.B, d.N, d.L, d.K);
+    hipLaunchKernelGGL(fwd_wide_kernel, grid, dim3(kWideThreads), 0, s, xT, idx, w, bias, out, d.B, d.N, d.L, d.K);
     FFI_HIP_TRY(hipGetLastError());
     return FFI_OK;
 }
 
-int launch_weight_grad_wide(const float* x, const int32_t* idx, const float* g, float* gw, const Dims& d, hipStream_t s) {
+int launch_weight_grad_wide(const float* x, const int32_t* idx, const float* g, float* gw, float* bias_grad, const Dims& d,
+                            hipStream_t s) {
     if (!wide_offsets_fit(d.N, d.B)) return FFI_ERR_TOO_LARGE;
-    const size_t lds = ((size_t)kWideLabels * kWideStride + (size_t)kWideLabels * d.K) * sizeof(float);
+    const size_t lds = ((size_t)kWideLabels * kWideStride + (size_t)kWideLabels * d.K + kWideLabels) * sizeof(float);
     if (lds > 150 * 1024) return FFI_ERR_TOO_LARGE;               // fan-in beyond ~450
     const float* xT = x;
     if (!d.tp) {
@@ -261,7 +275,7 @@ int launch_weight_grad_wide(const float* x, const int32_t* idx, const float* g, 
     }
     FFI_HIP_TRY(hipFuncSetAttribute((const void*)wgrad_wide_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     hipLaunchKernelGGL(wgrad_wide_kernel, dim3((d.L + kWideLabels - 1) / kWideLabels), dim3(kWideThreads), lds, s, xT, idx,
-                       g, gw, d.B, d.N, d.L, d.K);
+                       g, gw, bias_grad, d.B, d.N, d.L, d.K);
     FFI_HIP_TRY(hipGetLastError());
     return FFI_OK;
 }

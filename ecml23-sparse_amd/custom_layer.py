@@ -1,0 +1,124 @@
+"""The caller of the fixed-fan-in ops: a torch module shaped like the reference's layer.
+
+Mirrors ``StratifiedRewireLayerV2`` (sparse/custom_layer.py:6-50) on top of ``RewireLayerBase``
+(sparse/layer.py:106-249): flat variables of ``connections`` entries, viewed as
+``[units, connections // units]`` at call time; column ids drawn uniformly with replacement; the
+call is the transposed op followed by a bias add (here one fused kernel); rewiring replaces the
+sources of the selected connections in place and clears the matching entries of optimizer state.
+Everything on the call path runs in libffi_hip.so; torch holds the variables.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import fixed_fan_in_ops as ops
+
+
+class FixedMagnitudeSelector:
+    """Rewire all weights below a fixed magnitude (sparse/layer.py:45-57)."""
+
+    def __init__(self, threshold: float):
+        self.threshold = float(threshold)
+
+    def select(self, weight_values: torch.Tensor) -> torch.Tensor:
+        return weight_values.abs() < self.threshold
+
+
+class FixedFractionSelector:
+    """Rewire a fixed fraction of the connections, those of lowest magnitude (sparse/layer.py:60-84).
+
+    As in the reference the threshold is the ``round(fraction * n)``-th smallest magnitude and the
+    comparison is strict, so the connection that defines the threshold (and its ties) stays.
+    """
+
+    def __init__(self, fraction: float):
+        if not 0.0 <= fraction <= 1.0:
+            raise ValueError(f"Received an invalid value {fraction} for `fraction`, expected 0.0 <=  fraction <= 1.0")
+        self.fraction = float(fraction)
+
+    def select(self, weight_values: torch.Tensor) -> torch.Tensor:
+        flat = weight_values.reshape(-1).abs()
+        num_selected = int(round(self.fraction * flat.numel()))
+        if num_selected <= 0:
+            return torch.zeros_like(flat, dtype=torch.bool)
+        threshold = torch.kthvalue(flat, num_selected).values
+        return flat < threshold
+
+
+class StratifiedRewireLayerV2(torch.nn.Module):
+    """Fixed-fan-in sparse layer: ``units`` outputs, each fed by ``connections // units`` inputs."""
+
+    def __init__(self, units: int, input_dim: int, *, connections: int | None = None, sparsity: float | None = None,
+                 use_bias: bool = True, rewire_selector=None, device="cuda", generator: torch.Generator | None = None):
+        super().__init__()
+        if int(units) != units or units < 0:
+            raise ValueError(f"Received an invalid value for `units`, expected a positive integer, got {units}.")
+        if sparsity is not None and connections is not None:
+            raise ValueError("The `sparsity` and `connections` arguments are mutually exclusive")
+        if sparsity is None and connections is None:
+            raise ValueError("one of `sparsity` and `connections` is needed")
+        if sparsity is not None and not 0.0 <= sparsity <= 1.0:
+            raise ValueError(f"Received an invalid value {sparsity} for `sparsity`, expected 0.0 <=  sparsity <= 1.0")
+        self.units = int(units)
+        self.input_dim = int(input_dim)
+        # sparse/layer.py:173-177
+        self.connections = int(connections) if connections is not None else int((self.units * self.input_dim) * (1.0 - sparsity))
+        if self.connections < self.units or self.connections % self.units != 0:
+            raise ValueError("connections must be a positive multiple of units (the op views them as [units, fan_in])")
+        self.use_bias = bool(use_bias)
+        self.rewire_selector = rewire_selector if rewire_selector is not None else FixedFractionSelector(0.01)
+        self._generator = generator
+        # one weight per connection, Keras' default 'glorot_uniform' on a rank-1 shape: fan_in = fan_out = connections
+        limit = math.sqrt(6.0 / (2.0 * self.connections))
+        w = (torch.rand(self.connections, device=device, generator=generator) * 2.0 - 1.0) * limit
+        self.kernel_weights = torch.nn.Parameter(w)
+        # sources drawn uniformly, with replacement (sparse/custom_layer.py:12-15); the reference stores
+        # them as uint32, the same bits as the int32 kept here
+        self.register_buffer("kernel_indices", self._random_sources(self.connections, device))
+        self.bias = torch.nn.Parameter(torch.zeros(self.units, device=device)) if self.use_bias else None
+
+    @property
+    def fan_in(self) -> int:
+        return self.connections // self.units
+
+    def _random_sources(self, count: int, device) -> torch.Tensor:
+        return torch.randint(0, self.input_dim, (count,), device=device, generator=self._generator, dtype=torch.int64).to(torch.int32)
+
+    # sparse/custom_layer.py:45-50 followed by the bias add of sparse/layer.py:245-247
+    def _sparse_matmul(self, inputs: torch.Tensor) -> torch.Tensor:
+        indices = self.kernel_indices.view(-1, self.fan_in)
+        weights = self.kernel_weights.view(-1, self.fan_in)
+        tp_in = inputs.t().contiguous()
+        return ops.fan_in_sparse_matmul_tp(tp_in, indices, weights)
+
+    def forward(self, inputs: torch.Tensor) -> torch.Tensor:
+        if inputs.dim() != 2 or inputs.shape[1] != self.input_dim:
+            raise ValueError(f"inputs must have shape [batch, {self.input_dim}], got {tuple(inputs.shape)}")
+        if inputs.dtype != torch.float32:
+            inputs = inputs.float()
+        if not self.use_bias:
+            return self._sparse_matmul(inputs)
+        # same result as _sparse_matmul(inputs) + bias; the [B,N] entry point transposes inside the library
+        indices = self.kernel_indices.view(-1, self.fan_in)
+        weights = self.kernel_weights.view(-1, self.fan_in)
+        return ops.fan_in_sparse_matmul_bias(inputs, indices, weights, self.bias)
+
+    # sparse/layer.py:215-219, 236-237 and sparse/custom_layer.py:20-43
+    @torch.no_grad()
+    def rewire(self, other_vars=None):
+        """Gives the selected connections new random sources (weights keep their values) and
+        returns ``other_vars`` (e.g. Adam moments, sparse/optimizer.py:14-23) with the entries at
+        the rewired locations set to zero.  The index buffer is edited in place; the library
+        notices through the lookup fingerprint and rebuilds its plan on the next backward call."""
+        other_vars = [] if other_vars is None else list(other_vars)
+        locations = torch.nonzero(self.rewire_selector.select(self.kernel_weights.detach())).reshape(-1)
+        if locations.numel():
+            self.kernel_indices[locations] = self._random_sources(locations.numel(), self.kernel_indices.device)
+        outputs = []
+        for other in other_vars:
+            new_v = other.clone()
+            new_v.reshape(-1)[locations] = 0
+            outputs.append(new_v)
+        return outputs

@@ -191,3 +191,84 @@ def topk_scores(scores, k=5):
         _lib.check(_lib.lib().ffi_topk_f32(scores.data_ptr(), batch, num_units, int(k), values.data_ptr(),
                                            labels.data_ptr(), _stream_handle(scores.device)))
     return values, labels
+
+
+# ------------------------------------------------------------------------------------------------
+# The op followed by tf.nn.bias_add, as the reference's layer applies it (sparse/layer.py:239-249),
+# fused into the kernels: the forward adds bias[j] before it stores a score, the backward returns the
+# bias gradient (column sums of out_grad) from the weight-gradient kernel.
+# ------------------------------------------------------------------------------------------------
+def _check_bias(bias, weights, num_units):
+    if bias.dim() != 1 or bias.shape[0] != num_units:
+        raise ValueError(f"bias must have shape ({num_units},), got {tuple(bias.shape)}")
+    if bias.dtype != torch.float32 or bias.device != weights.device:
+        raise TypeError("bias must be float32 on the weights' device")
+
+
+def _forward_bias(features, lookup, weights, bias, transposed):
+    batch, num_features, num_units, fan_in = _check_inputs(features, lookup, weights, transposed)
+    _check_bias(bias, weights, num_units)
+    features, lookup, weights, bias = features.contiguous(), lookup.contiguous(), weights.contiguous(), bias.contiguous()
+    with torch.cuda.device(features.device):
+        result = torch.empty((batch, num_units), dtype=torch.float32, device=features.device)
+        _lib.check(_lib.lib().ffi_forward_bias_f32(
+            features.data_ptr(), lookup.data_ptr(), weights.data_ptr(), bias.data_ptr(), result.data_ptr(),
+            batch, num_features, num_units, fan_in, int(transposed), _stream_handle(features.device)))
+    return result
+
+
+def _backward_bias(features, lookup, weights, out_grad, transposed, need_feature_grad=True):
+    batch, num_features, num_units, fan_in = _check_inputs(features, lookup, weights, transposed, out_grad)
+    features, lookup, weights, out_grad = features.contiguous(), lookup.contiguous(), weights.contiguous(), out_grad.contiguous()
+    with torch.cuda.device(features.device):
+        feature_grad = torch.empty_like(features) if need_feature_grad else None
+        weight_grad = torch.empty_like(weights)
+        bias_grad = torch.empty((num_units,), dtype=torch.float32, device=features.device)
+        _lib.check(_lib.lib().ffi_backward_bias_f32(
+            features.data_ptr(), lookup.data_ptr(), weights.data_ptr(), out_grad.data_ptr(),
+            feature_grad.data_ptr() if need_feature_grad else None, weight_grad.data_ptr(), bias_grad.data_ptr(),
+            batch, num_features, num_units, fan_in, int(transposed), _stream_handle(features.device)))
+    return feature_grad, weight_grad, bias_grad
+
+
+class FanInSparseMatmulBiasTp(torch.autograd.Function):
+    """``fan_in_sparse_matmul_tp`` + ``bias_add`` as one differentiable op; gradients
+    ``[feature_grad, None, weight_grad, bias_grad]``."""
+
+    @staticmethod
+    def forward(ctx, features, lookup, weights, bias):
+        ctx.save_for_backward(features, lookup, weights)
+        return _forward_bias(features, lookup, weights, bias, True)
+
+    @staticmethod
+    def backward(ctx, grad):
+        features, lookup, weights = ctx.saved_tensors
+        feature_grad, weight_grad, bias_grad = _backward_bias(features, lookup, weights, grad, True,
+                                                              need_feature_grad=ctx.needs_input_grad[0])
+        return feature_grad, None, weight_grad, bias_grad
+
+
+class FanInSparseMatmulBias(torch.autograd.Function):
+    """As above with features given as ``[B,N]``."""
+
+    @staticmethod
+    def forward(ctx, features, lookup, weights, bias):
+        ctx.save_for_backward(features, lookup, weights)
+        return _forward_bias(features, lookup, weights, bias, False)
+
+    @staticmethod
+    def backward(ctx, grad):
+        features, lookup, weights = ctx.saved_tensors
+        feature_grad, weight_grad, bias_grad = _backward_bias(features, lookup, weights, grad, False,
+                                                              need_feature_grad=ctx.needs_input_grad[0])
+        return feature_grad, None, weight_grad, bias_grad
+
+
+def fan_in_sparse_matmul_bias(features, lookup, weights, bias):
+    """``fan_in_sparse_matmul(features, lookup, weights) + bias`` in one kernel."""
+    return FanInSparseMatmulBias.apply(features, lookup, weights, bias)
+
+
+def fan_in_sparse_matmul_tp_bias(features, lookup, weights, bias):
+    """``fan_in_sparse_matmul_tp(features, lookup, weights) + bias`` in one kernel."""
+    return FanInSparseMatmulBiasTp.apply(features, lookup, weights, bias)

@@ -119,6 +119,22 @@ int ffi_check_lookup(const int32_t* lookup, int64_t num_units, int64_t fan_in, i
                      ffi_stream_t stream);
 
 /*
+ * The layer as its caller uses it: the op followed by tf.nn.bias_add (sparse/layer.py:239-249,
+ * sparse/custom_layer.py:45-50), fused.  result[b,j] = (sum_k ...) + bias[j]; bias is [num_units].
+ * The backward variant also returns bias_grad[j] = sum_b out_grad[b,j] (the gradient TensorFlow
+ * registers for bias_add), computed by the weight-gradient kernel from the out_grad values it
+ * loads anyway; weight_grad and bias_grad must both be given, feature_grad may be NULL.
+ */
+int ffi_forward_bias_f32(const float* features, const int32_t* lookup, const float* weights, const float* bias,
+                         float* result,
+                         int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in,
+                         int transposed, ffi_stream_t stream);
+int ffi_backward_bias_f32(const float* features, const int32_t* lookup, const float* weights,
+                          const float* out_grad, float* feature_grad, float* weight_grad, float* bias_grad,
+                          int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in,
+                          int transposed, ffi_stream_t stream);
+
+/*
  * Inference variant (no counterpart in the reference, whose ops are registered for float only,
  * tfsparse/cc/kernels/register.cpp:79-109): features and weights are bfloat16 (raw 16-bit
  * patterns, same layouts as above), products are accumulated in fp32, result is fp32.

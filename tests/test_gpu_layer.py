@@ -1,0 +1,161 @@
+"""The layer-level caller (sparse/custom_layer.py:45-50 + the bias add of sparse/layer.py:245-247):
+fused-bias entry points through the C ABI, and the torch module built on them, against the oracle.
+
+Expected values: oracle forward (forward.cpp:9-44 restated) plus a numpy bias add; the bias
+gradient is the float64 column sum of out_grad (the gradient of tf.nn.bias_add).
+Gates as for the ops: forward 1e-5, gradients 1e-4, relative to the largest reference magnitude.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from conftest import load_package, rel_err
+
+pytestmark = pytest.mark.gpu
+
+FWD_RTOL = 1e-5
+GRAD_RTOL = 1e-4
+
+#          B    N     L     K  transposed      (narrow: tile kernels; wide: N beyond the LDS tile)
+SHAPES = [(128, 768, 5000, 32, True),
+          (37, 300, 1001, 7, False),
+          (64, 512, 2100, 64, True),
+          (200, 96, 700, 40, False),
+          (33, 3000, 333, 12, True),
+          (130, 2048, 260, 72, False)]
+
+
+@pytest.fixture(scope="module")
+def ffi():
+    pkg = load_package()
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    return pkg
+
+
+def make_case(shape, seed):
+    B, N, L, K, tp = shape
+    rng = np.random.default_rng(seed)
+    x = np.maximum(rng.standard_normal((B, N)), 0).astype(np.float32)
+    lookup = rng.integers(0, N, size=(L, K)).astype(np.int32)          # with replacement, as the layer draws them
+    w = (rng.standard_normal((L, K)) / np.sqrt(K)).astype(np.float32)
+    bias = rng.standard_normal(L).astype(np.float32)
+    g = (rng.standard_normal((B, L)) * 0.1).astype(np.float32)
+    if tp:
+        x = np.ascontiguousarray(x.T)
+    return x, lookup, w, bias, g
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "B%d_N%d_L%d_K%d_%s" % (s[0], s[1], s[2], s[3], "tp" if s[4] else "nt"))
+def test_fused_bias_entry_points(ffi, shape):
+    B, N, L, K, tp = shape
+    x, lookup, w, bias, g = make_case(shape, 3)
+    dx, dl, dw, db, dg = dev(x), dev(lookup), dev(w), dev(bias), dev(g)
+    lib, st = ffi._lib.lib(), torch.cuda.current_stream().cuda_stream
+    out = torch.full((B, L), float("nan"), device="cuda")
+    ffi._lib.check(lib.ffi_forward_bias_f32(dx.data_ptr(), dl.data_ptr(), dw.data_ptr(), db.data_ptr(), out.data_ptr(),
+                                            B, N, L, K, int(tp), st))
+    gx = torch.full(tuple(x.shape), float("nan"), device="cuda")
+    gw = torch.full((L, K), float("nan"), device="cuda")
+    gb = torch.full((L,), float("nan"), device="cuda")
+    ffi._lib.check(lib.ffi_backward_bias_f32(dx.data_ptr(), dl.data_ptr(), dw.data_ptr(), dg.data_ptr(), gx.data_ptr(),
+                                             gw.data_ptr(), gb.data_ptr(), B, N, L, K, int(tp), st))
+    torch.cuda.synchronize()
+    want = oracle.forward(x, lookup, w, transposed=tp) + bias[None, :]
+    assert rel_err(out.cpu().numpy(), want) <= FWD_RTOL
+    want_gx, want_gw = oracle.backward(x, lookup, w, g, transposed=tp)
+    assert rel_err(gx.cpu().numpy(), want_gx) <= GRAD_RTOL
+    assert rel_err(gw.cpu().numpy(), want_gw) <= GRAD_RTOL
+    assert rel_err(gb.cpu().numpy(), g.astype(np.float64).sum(axis=0)) <= GRAD_RTOL
+    # the fused weight gradient is the plain entry point's, bit for bit
+    gw2 = torch.empty((L, K), device="cuda")
+    ffi._lib.check(lib.ffi_weight_grad_f32(dx.data_ptr(), dl.data_ptr(), dg.data_ptr(), gw2.data_ptr(), B, N, L, K, int(tp), st))
+    torch.cuda.synchronize()
+    assert torch.equal(gw, gw2)
+
+
+def test_fused_bias_null_arguments(ffi):
+    lib = ffi._lib.lib()
+    t = torch.zeros(8, device="cuda")
+    assert lib.ffi_forward_bias_f32(t.data_ptr(), t.data_ptr(), t.data_ptr(), None, t.data_ptr(), 1, 1, 1, 1, 0, None) == -1
+    assert lib.ffi_backward_bias_f32(t.data_ptr(), t.data_ptr(), t.data_ptr(), t.data_ptr(), None, t.data_ptr(), None,
+                                     1, 1, 1, 1, 0, None) == -1
+
+
+@pytest.mark.parametrize("use_bias", [True, False])
+def test_layer_forward_backward(ffi, use_bias):
+    layer_mod = ffi.custom_layer
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(7)
+    B, N, units, K = 48, 640, 3000, 32
+    layer = layer_mod.StratifiedRewireLayerV2(units, N, connections=units * K, use_bias=use_bias, generator=gen)
+    assert layer.fan_in == K and layer.kernel_indices.dtype == torch.int32 and layer.kernel_weights.shape == (units * K,)
+    if use_bias:
+        with torch.no_grad():
+            layer.bias.copy_(torch.randn(units, device="cuda", generator=gen))
+    x = torch.relu(torch.randn(B, N, device="cuda", generator=gen)).requires_grad_(True)
+    g = torch.randn(B, units, device="cuda", generator=gen) * 0.1
+    out = layer(x)
+    out.backward(g)
+    torch.cuda.synchronize()
+    xn, gn = x.detach().cpu().numpy(), g.cpu().numpy()
+    lookup = layer.kernel_indices.view(-1, K).cpu().numpy()
+    w = layer.kernel_weights.detach().view(-1, K).cpu().numpy()
+    want = oracle.forward(xn, lookup, w)
+    if use_bias:
+        want = want + layer.bias.detach().cpu().numpy()[None, :]
+    assert rel_err(out.detach().cpu().numpy(), want) <= FWD_RTOL
+    want_gx, want_gw = oracle.backward(xn, lookup, w, gn)
+    assert rel_err(x.grad.cpu().numpy(), want_gx) <= GRAD_RTOL
+    assert rel_err(layer.kernel_weights.grad.view(-1, K).cpu().numpy(), want_gw) <= GRAD_RTOL
+    if use_bias:
+        assert rel_err(layer.bias.grad.cpu().numpy(), gn.astype(np.float64).sum(axis=0)) <= GRAD_RTOL
+
+
+def test_layer_rewire(ffi):
+    layer_mod = ffi.custom_layer
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(11)
+    B, N, units, K = 40, 256, 1500, 16
+    layer = layer_mod.StratifiedRewireLayerV2(units, N, connections=units * K, rewire_selector=layer_mod.FixedFractionSelector(0.05),
+                                              generator=gen)
+    x = torch.relu(torch.randn(B, N, device="cuda", generator=gen)).requires_grad_(True)
+    g = torch.randn(B, units, device="cuda", generator=gen) * 0.1
+    layer(x).backward(g)                      # builds and caches the plan for the current indices
+    before_idx = layer.kernel_indices.clone()
+    before_w = layer.kernel_weights.detach().clone()
+    m = torch.ones(units * K, device="cuda")
+    v = torch.full((units * K,), 2.0, device="cuda")
+    selected = layer.rewire_selector.select(before_w)
+    new_m, new_v = layer.rewire([m, v])
+    n_sel = int(selected.sum())
+    assert 0 < n_sel <= round(0.05 * units * K)
+    assert torch.equal(layer.kernel_weights.detach(), before_w)                      # weights keep their values
+    assert torch.equal(layer.kernel_indices[~selected], before_idx[~selected])        # only selected sources change
+    assert int((layer.kernel_indices != before_idx).sum()) > 0
+    assert float(new_m[selected].abs().sum()) == 0 and float(new_v[selected].abs().sum()) == 0
+    assert torch.equal(new_m[~selected], m[~selected]) and torch.equal(new_v[~selected], v[~selected])
+    assert float(m.min()) == 1.0                                                      # inputs are not modified
+    # gradients after the in-place edit follow the new indices (the cached plan is rebuilt)
+    x.grad = None
+    layer.kernel_weights.grad = None
+    layer(x).backward(g)
+    torch.cuda.synchronize()
+    lookup = layer.kernel_indices.view(-1, K).cpu().numpy()
+    w = layer.kernel_weights.detach().view(-1, K).cpu().numpy()
+    want_gx, want_gw = oracle.backward(x.detach().cpu().numpy(), lookup, w, g.cpu().numpy())
+    assert rel_err(x.grad.cpu().numpy(), want_gx) <= GRAD_RTOL
+    assert rel_err(layer.kernel_weights.grad.view(-1, K).cpu().numpy(), want_gw) <= GRAD_RTOL
+
+
+def test_selectors(ffi):
+    layer_mod = ffi.custom_layer
+    w = torch.tensor([0.5, -0.1, 0.3, -0.05, 0.2, 0.05, -0.7, 0.0], device="cuda")
+    assert layer_mod.FixedMagnitudeSelector(0.1).select(w).tolist() == [False, False, False, True, False, True, False, True]
+    # fraction 0.5 of 8 -> the 4th smallest magnitude (0.1) is the threshold, strictly smaller ones are selected
+    assert layer_mod.FixedFractionSelector(0.5).select(w).tolist() == [False, False, False, True, False, True, False, True]
+    assert layer_mod.FixedFractionSelector(0.0).select(w).sum().item() == 0

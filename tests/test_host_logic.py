@@ -76,3 +76,26 @@ def test_synthetic_inputs_shapes_and_bytes():
     assert b["forward"] == b["input_grad"] == b["weight_grad"] == 515_023_104
     c3 = synth.make_inputs(synth.CONFIGS["c3"], num_units=10)["features"]
     assert torch.allclose(c3.norm(dim=1), torch.ones(256), atol=1e-5) and float(c3.min()) >= 0
+
+
+def test_layer_constructor_arithmetic():
+    """connections from sparsity (sparse/layer.py:173-177), fan-in = connections // units
+    (sparse/custom_layer.py:46), argument errors; no kernel runs."""
+    pkg = load_package()
+    L = pkg.custom_layer.StratifiedRewireLayerV2
+    layer = L(100, 64, sparsity=0.75, device="cpu")
+    assert layer.connections == int(100 * 64 * 0.25) == 1600 and layer.fan_in == 16
+    assert layer.kernel_weights.shape == (1600,) and layer.kernel_indices.shape == (1600,)
+    assert int(layer.kernel_indices.min()) >= 0 and int(layer.kernel_indices.max()) < 64
+    limit = (6.0 / (2 * 1600)) ** 0.5
+    assert float(layer.kernel_weights.detach().abs().max()) <= limit
+    assert layer.bias.shape == (100,) and float(layer.bias.detach().abs().sum()) == 0.0
+    assert L(10, 8, connections=40, use_bias=False, device="cpu").bias is None
+    with pytest.raises(ValueError):
+        L(10, 8, connections=40, sparsity=0.5, device="cpu")
+    with pytest.raises(ValueError):
+        L(10, 8, connections=45, device="cpu")
+    with pytest.raises(ValueError):
+        L(10, 8, sparsity=1.5, device="cpu")
+    with pytest.raises(RuntimeError):          # the product path needs the GPU: no CPU fallback
+        layer(torch.zeros(2, 64))
