@@ -20,27 +20,30 @@ namespace {
 // wp[slot] = w at the connection stored in that slot (0 in padding slots): brings the weights into
 // the plan's slot order so that the main kernel reads them coalesced.  One workgroup per label
 // tile, one thread per column.  The tile's weights pass through LDS in pieces of kPermChunk floats
-// (read from HBM fully coalesced); a column's slots hold ascending positions, so each thread just
-// advances a cursor through its slots while their positions fall inside the staged piece.
-constexpr int kPermChunk = 16384;     // 64 KB of LDS: two workgroups fit on a CU and overlap each other
+// (read from HBM fully coalesced).  The wavefront walks the slice's rows together (every load is
+// one coalesced 256-byte row), eight rows per step; a lane stores the slots whose position lies in
+// the staged piece.  A column's positions ascend inside each label parity and the two parities
+// alternate, so nothing of a later piece sits before the first step in which some lane met a
+// position beyond the current piece: the next piece resumes there.
+constexpr int kPermChunk = 16384;     // 64 KB of LDS per piece: two workgroups fit on a CU and overlap each other
+constexpr int kPermChunkBig = 32768;  // 128 KB: a whole tile of 1024 labels x 32 connections in one piece
 __global__ __launch_bounds__(1024) void igrad_permute_weights_kernel(
-    const unsigned* __restrict__ ent, const unsigned* __restrict__ slice_off, const unsigned short* __restrict__ col_len,
-    const float* __restrict__ w, float* __restrict__ wp, int L, int K, int tile_labels) {
-    __shared__ __align__(16) float ws[kPermChunk];
+    const unsigned* __restrict__ ent, const unsigned* __restrict__ slice_off, const float* __restrict__ w,
+    float* __restrict__ wp, int L, int K, int tile_labels, int chunk) {
+    extern __shared__ __align__(16) float ws[];
     const int t = blockIdx.x, nthreads = blockDim.x;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const size_t sl = (size_t)t * (nthreads >> 6) + wave;
     const unsigned row0 = slice_off[sl], rows = slice_off[sl + 1] - row0;
-    const unsigned len = col_len[(size_t)t * nthreads + threadIdx.x];
     const int nl = min(tile_labels, L - t * tile_labels);
     const unsigned npos = (unsigned)nl * (unsigned)K;
     const float* wt = w + (size_t)t * tile_labels * K;
     const bool vec = ((((uintptr_t)wt) & 15) == 0);
     const unsigned* ep = ent + (size_t)row0 * 64 + lane;
     float* op = wp + (size_t)row0 * 64 + lane;
-    unsigned lo = 0;                 // wave-uniform: rows below lo are finished in every column of the slice
-    for (unsigned c0 = 0; c0 < npos; c0 += kPermChunk) {
-        const unsigned n = min((unsigned)kPermChunk, npos - c0);
+    unsigned lo = 0;                 // wave-uniform: rows below lo hold nothing of this or a later piece
+    for (unsigned c0 = 0; c0 < npos; c0 += (unsigned)chunk) {
+        const unsigned n = min((unsigned)chunk, npos - c0);
         __syncthreads();
         if (vec) {
             // all of a thread's loads go out before its first LDS write: one round trip per piece
@@ -61,33 +64,24 @@ __global__ __launch_bounds__(1024) void igrad_permute_weights_kernel(
         }
         __syncthreads();
         const unsigned hi = c0 + n;
-        // The wavefront walks the slice's rows together (every load is one coalesced 256-byte
-        // row), eight rows per step; a lane stores the slots whose position lies in the staged
-        // piece.  Positions ascend inside a column, so the walk of this piece stops at the first
-        // step in which no lane found one, and the next piece resumes at the first step in which
-        // some lane met a position beyond this piece.
         unsigned resume = 0xffffffffu;
         for (unsigned i = lo; i < rows; i += 8) {
             unsigned e8[8];
 #pragma unroll
             for (int q = 0; q < 8; ++q) e8[q] = ep[(size_t)min(i + q, rows - 1) * 64];
-            bool any_here = false, any_later = false;
+            bool any_later = false;
 #pragma unroll
             for (int q = 0; q < 8; ++q) {
                 const unsigned pos = e8[q] >> kEntLabelBits;
-                const bool valid = i + q < len;
-                if (valid && pos >= c0 && pos < hi) {
-                    op[(size_t)(i + q) * 64] = ws[pos - c0];
-                    any_here = true;
-                }
-                any_later |= valid && pos >= hi;
+                const bool real = i + q < rows && (e8[q] & kEntLabelMask) < (unsigned)tile_labels;
+                if (real && pos >= c0 && pos < hi) op[(size_t)(i + q) * 64] = ws[pos - c0];
+                if (c0 == 0 && i + q < rows && !real) op[(size_t)(i + q) * 64] = 0.f;     // padding slots
+                any_later |= real && pos >= hi;
             }
             if (resume == 0xffffffffu && __any(any_later)) resume = i;
-            if (!__any(any_here) && resume != 0xffffffffu) break;
         }
         lo = (resume == 0xffffffffu) ? rows : resume;
     }
-    for (unsigned r = len; r < rows; ++r) op[(size_t)r * 64] = 0.f;     // padding slots
 }
 
 // The eight 16-byte reads of one row (chunk order skewed by the lane id) ...
@@ -118,7 +112,7 @@ __device__ __forceinline__ void igrad_fmas(const float4 (&v)[8], float wv, float
 // LPT: labels of a tile staged per thread (tile_labels <= LPT * blockDim.x).
 template <int MAXT, int LPT>
 __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned* __restrict__ ent, const float* __restrict__ wp,
-                                  const unsigned* __restrict__ slice_off, const unsigned short* __restrict__ col_len,
+                                  const unsigned* __restrict__ slice_off,
                                   const float* __restrict__ g, float* __restrict__ partial, int B, int L,
                                   int tile_labels, int tiles, int tiles_per_stream, int nbt) {
     extern __shared__ __align__(16) float gs[];
@@ -147,8 +141,8 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned* __rest
             if (jl < nl) load_rows32(g, L, b0, B, (unsigned)(j0 + jl), gbn[p]);
         }
         __syncthreads();                       // the previous tile is no longer being read
-        // row `tile_labels` is all zero: the target of padding slots
-        if (t == t_begin && threadIdx.x < 32) gs[tile_labels * kTileBatch + threadIdx.x] = 0.f;
+        // rows `tile_labels` (even) and `tile_labels + 1` (odd) are all zero: the targets of padding slots
+        if (t == t_begin && threadIdx.x < 64) gs[tile_labels * kTileBatch + threadIdx.x] = 0.f;
         // gs[jl][c] = g[b0+c][j0+jl]: the rows were loaded coalesced along labels; 16-byte LDS writes
         // whose chunk order is skewed by the label id (no bank conflicts)
 #pragma unroll
@@ -192,6 +186,9 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned* __rest
                 en[q] = ep[(size_t)r * 64];
                 wn[q] = wpp[(size_t)r * 64];
             }
+            // keep these loads here, a whole group of rows ahead of their use (left alone, the
+            // scheduler sinks them below the multiply-adds and every group waits a full round trip)
+            __builtin_amdgcn_sched_barrier(0);
             // branch-free: padding slots carry weight 0 and point at the all-zero LDS row, rows past
             // the end of the slice are redirected there too
 #pragma unroll
@@ -239,15 +236,18 @@ int launch_tiled(const ffi_plan* p, const float* w, const float* g, float* gx, i
     float* partial = nullptr;
     FFI_TRY(workspace_get(s, kWsFeaturesT, std::max<size_t>(slots, 1) * sizeof(float), (void**)&wp));
     FFI_TRY(workspace_get(s, kWsPartials, (size_t)streams * p->threads * bpad * sizeof(float), (void**)&partial));
-    hipLaunchKernelGGL(igrad_permute_weights_kernel, dim3(p->tiles), dim3(p->threads), 0, s, p->ent, p->slice_off,
-                       p->col_len, w, wp, p->L, p->K, p->tile_labels);
-    const size_t lds = tile_lds_bytes(p->tile_labels + 1);      // + the all-zero row
+    // a tile's weights in one piece when they fit (one walk over the slots instead of one per piece)
+    const int chunk = ((long long)p->tile_labels * p->K <= kPermChunkBig) ? kPermChunkBig : kPermChunk;
+    FFI_HIP_TRY(hipFuncSetAttribute((const void*)igrad_permute_weights_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, chunk * 4));
+    hipLaunchKernelGGL(igrad_permute_weights_kernel, dim3(p->tiles), dim3(p->threads), chunk * sizeof(float), s, p->ent,
+                       p->slice_off, w, wp, p->L, p->K, p->tile_labels, chunk);
+    const size_t lds = tile_lds_bytes(p->tile_labels + 2);      // + the two all-zero rows
     const dim3 grid(streams * nbt), block(p->threads);
 #define FFI_LAUNCH_TILE(MAXT, LPT)                                                                                      \
     do {                                                                                                                \
         FFI_HIP_TRY(hipFuncSetAttribute((const void*)igrad_tile_kernel<MAXT, LPT>,                                      \
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));                        \
-        hipLaunchKernelGGL((igrad_tile_kernel<MAXT, LPT>), grid, block, lds, s, p->ent, wp, p->slice_off, p->col_len, g, \
+        hipLaunchKernelGGL((igrad_tile_kernel<MAXT, LPT>), grid, block, lds, s, p->ent, wp, p->slice_off, g, \
                            partial, B, p->L, p->tile_labels, p->tiles, tps, nbt);                                       \
     } while (0)
     // the plan sizes its tiles so that one of these fits: tile_labels <= LPT * threads

@@ -72,8 +72,10 @@ int launch_weight_grad_wide(const float* x, const int32_t* idx, const float* g, 
 // connections are grouped by column, and the columns into slices of 64 (one per wavefront).  A
 // slice is stored slot-major: row i of the slice holds the i-th connection of each of its 64
 // columns (so a wavefront reads 256 contiguous bytes per step), padded to the longest column of
-// the slice.  Inside a column the connections are in ascending flat position, the order the
-// reference's CPU kernel accumulates in (tfsparse/cc/kernels/backward.cpp:64-72).
+// the slice.  Inside a column the slots alternate between even and odd labels (which parity comes
+// first depends on the lane, see ffi_plan.hip), positions ascend inside each parity, and holes are
+// padding slots: a fixed order, but not the ascending-position order in which the reference's CPU
+// kernel accumulates (tfsparse/cc/kernels/backward.cpp:64-72).
 //
 // tiled == false (any shape): a CSC per block of `block_labels` labels.  perm[e] = flat position of
 // the e-th connection in (label block, column, position) order;
@@ -91,9 +93,8 @@ struct ffi_plan {
     int tiles = 0;            // ceil(L / tile_labels)
     long long total_rows = 0; // rows of 64 entries over all slices
     unsigned* slice_off = nullptr;       // [tiles*slices + 1] first row of each slice
-    unsigned short* col_len = nullptr;   // [tiles][threads] connections of each column in each tile
     unsigned* ent = nullptr;             // [total_rows*64]  (position in tile << 11) | label in tile;
-                                         // padding slots hold label == tile_labels (an all-zero row)
+                                         // padding slots hold label == tile_labels + parity (all-zero rows)
     // blocked global form
     int block_labels = 0;     // labels per block (bounds the part of out_grad that is live at a time)
     int nblocks = 0;

@@ -92,6 +92,13 @@ __device__ __forceinline__ void load_rows32(const float* __restrict__ m, int ld,
 // the bank group depends on the chunk number only, and any eight consecutive lanes hit eight
 // different bank groups (4.3x faster than the unskewed order, 1.4x faster than padded rows).
 // Consequence: register group c of lane l holds batch entries 4*(c ^ (l&7)) .. +3.
+// A 128-byte row covers half of the 64 banks (even rows one half, odd rows the other).  The LDS
+// serves a ds_read_b128 at 16 lanes per clock (256 bytes) only when eight of those lanes read each
+// half; measured with this access pattern: 4 clocks per wavefront read when the lanes with bit 3 of
+// their id clear read even rows and the others odd rows, 8 clocks when row parities are random or
+// all equal.  Kernels whose row order is theirs to choose (the input gradient, through its plan)
+// arrange that; the forward pass and the weight gradient take rows in the order of the lookup
+// matrix and run at the 8-clock rate.
 
 __device__ __forceinline__ void cond_swap(bool p, float& a, float& b) {
     const float t = p ? b : a;

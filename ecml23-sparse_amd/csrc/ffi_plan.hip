@@ -69,10 +69,6 @@ __global__ __launch_bounds__(kBlock) void fingerprint_kernel(const int32_t* __re
     }
 }
 
-__global__ __launch_bounds__(kBlock) void fill_u32_kernel(unsigned* p, size_t n, unsigned value) {
-    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) p[i] = value;
-}
-
 __global__ __launch_bounds__(kBlock) void zero_u64_kernel(unsigned long long* p, int n) {
     const int i = blockIdx.x * kBlock + threadIdx.x;
     if (i < n) p[i] = 0;
@@ -80,22 +76,37 @@ __global__ __launch_bounds__(kBlock) void zero_u64_kernel(unsigned long long* p,
 
 // ---- tiled form ---------------------------------------------------------------------------------
 
+// Order of a column's slots inside a tile.  The kernel that walks the plan reads, per slot, the
+// 128-byte LDS row of the slot's label; rows of even labels sit in one half of the LDS banks, rows
+// of odd labels in the other, and the LDS serves 16 lanes per clock only if 8 of them read each
+// half.  So the lanes whose id has bit 3 clear walk their column as even, odd, even, ... labels
+// and the lanes with bit 3 set as odd, even, odd, ...: slot 2t holds the t-th label of the lane's
+// first parity, slot 2t+1 the t-th label of the other parity, holes are padding slots that point
+// at an all-zero row of the right parity.  Inside a parity class positions ascend.
+__device__ __forceinline__ unsigned parity_first(unsigned thread) { return (thread >> 3) & 1u; }       // parity walked at even slots
+__device__ __forceinline__ unsigned column_slots(unsigned thread, unsigned even, unsigned odd) {
+    const unsigned first = parity_first(thread) ? odd : even, second = parity_first(thread) ? even : odd;
+    return max(first ? 2u * first - 1u : 0u, 2u * second);
+}
+
 // One workgroup per label tile, one thread per column.  Counts the tile's connections per column
-// (integer LDS atomics: order-independent), stores them, and the longest column of each slice.
+// and label parity (integer LDS atomics: order-independent), stores the slot count of the longest
+// column of each slice.
 __global__ void tile_count_kernel(const int32_t* __restrict__ idx, int L, int K, int tile_labels,
-                                  unsigned short* __restrict__ col_len, unsigned* __restrict__ slice_len) {
-    extern __shared__ unsigned cnt[];
+                                  unsigned* __restrict__ slice_len) {
+    extern __shared__ unsigned cnt[];          // [2][threads]: even labels, odd labels
     const int t = blockIdx.x, nthreads = blockDim.x;
     cnt[threadIdx.x] = 0;
+    cnt[nthreads + threadIdx.x] = 0;
     __syncthreads();
     const int j0 = t * tile_labels;
     const int nl = min(tile_labels, L - j0);
     const int* src = idx + (size_t)j0 * K;
     const int total = nl * K;
-    for (int e = threadIdx.x; e < total; e += nthreads) atomicAdd(&cnt[(unsigned)src[e]], 1u);
+    for (int e = threadIdx.x; e < total; e += nthreads) atomicAdd(&cnt[((e / K) & 1) * nthreads + (unsigned)src[e]], 1u);
     __syncthreads();
-    unsigned c = cnt[threadIdx.x];
-    col_len[(size_t)t * nthreads + threadIdx.x] = (unsigned short)c;
+    const unsigned even = cnt[threadIdx.x], odd = cnt[nthreads + threadIdx.x];
+    unsigned c = column_slots(threadIdx.x, even, odd);
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) c = max(c, (unsigned)__shfl_xor((int)c, off));
     if ((threadIdx.x & 63) == 0) slice_len[(size_t)t * (nthreads >> 6) + (threadIdx.x >> 6)] = c;
@@ -123,9 +134,10 @@ __global__ __launch_bounds__(1024) void slice_scan_kernel(const unsigned* __rest
 }
 
 // One workgroup per label tile, one thread per column n.  The tile's column ids pass through LDS
-// in chunks; every thread scans them in flat-position order and appends the ones equal to its
-// column, so the connections of a column end up in ascending position: deterministic and stable
-// without any sort.  ent = (position inside the tile << 11) | label inside the tile.
+// in chunks; every thread scans them in flat-position order and places the ones equal to its
+// column (see column_slots for the order), so the result is deterministic without any sort.
+// ent = (position inside the tile << 11) | label inside the tile; the slots a column leaves empty
+// up to the slice's length become padding: position 0, label tile_labels + parity (all-zero rows).
 constexpr int kFillChunk = 8192;
 __global__ void tile_fill_kernel(const int32_t* __restrict__ idx, int L, int K, int tile_labels,
                                  const unsigned* __restrict__ slice_off, unsigned* __restrict__ ent) {
@@ -136,10 +148,15 @@ __global__ void tile_fill_kernel(const int32_t* __restrict__ idx, int L, int K, 
     const int* src = idx + (size_t)j0 * K;
     const int total = nl * K;
     const int mine = threadIdx.x;
-    const size_t row0 = slice_off[(size_t)t * (nthreads >> 6) + (threadIdx.x >> 6)];
+    const size_t sl = (size_t)t * (nthreads >> 6) + (threadIdx.x >> 6);
+    const size_t row0 = slice_off[sl];
+    const unsigned rows = slice_off[sl + 1] - slice_off[sl];
     unsigned* dst = ent + row0 * 64 + (threadIdx.x & 63);
-    unsigned count = 0;
-    int label = 0, kk = 0;       // label and connection slot of the entry under the cursor
+    const unsigned first = parity_first(threadIdx.x);
+    // padding everywhere first; the thread's own slots are then overwritten (same thread: ordered)
+    for (unsigned r = 0; r < rows; ++r) dst[(size_t)r * 64] = (unsigned)tile_labels + ((r & 1u) ^ first);
+    unsigned seen[2] = {0u, 0u};  // labels of each parity placed so far
+    int label = 0, kk = 0;        // label and connection slot of the entry under the cursor
     for (int c0 = 0; c0 < total; c0 += kFillChunk) {
         const int n = min(kFillChunk, total - c0);
         __syncthreads();
@@ -147,8 +164,10 @@ __global__ void tile_fill_kernel(const int32_t* __restrict__ idx, int L, int K, 
         __syncthreads();
         for (int e = 0; e < n; ++e) {
             if (keys[e] == mine) {
-                dst[(size_t)count * 64] = ((unsigned)(c0 + e) << kEntLabelBits) | (unsigned)label;
-                ++count;
+                const unsigned par = (unsigned)label & 1u;
+                const unsigned t2 = par ? seen[1]++ : seen[0]++;
+                const unsigned slot = 2u * t2 + (par ^ first);
+                dst[(size_t)slot * 64] = ((unsigned)(c0 + e) << kEntLabelBits) | (unsigned)label;
             }
             if (++kk == K) { kk = 0; ++label; }
         }
@@ -180,9 +199,8 @@ void free_arrays(ffi_plan* p) {
     if (p->perm) (void)hipFree(p->perm);
     if (p->col_ptr) (void)hipFree(p->col_ptr);
     if (p->slice_off) (void)hipFree(p->slice_off);
-    if (p->col_len) (void)hipFree(p->col_len);
     if (p->ent) (void)hipFree(p->ent);
-    p->perm = nullptr; p->col_ptr = nullptr; p->slice_off = nullptr; p->col_len = nullptr; p->ent = nullptr;
+    p->perm = nullptr; p->col_ptr = nullptr; p->slice_off = nullptr; p->ent = nullptr;
     p->tiled = false; p->total_rows = 0; p->bytes = 0;
 }
 
@@ -203,18 +221,18 @@ int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     const int threads = ((p->N + 63) / 64) * 64;
     // every thread of the kernel that walks the plan stages at most two labels of a tile (one when
     // the workgroup is larger than 768 threads and registers are scarcer)
-    const int TL = std::min(std::min(kPlanTileLabels, p->L), threads > 768 ? threads : 2 * threads);
+    // (even, so that label parity inside a tile is the parity of the LDS row)
+    const int TL = (std::min(std::min(kPlanTileLabels, p->L), threads > 768 ? threads : 2 * threads) + 1) & ~1;
     const int slices = threads / 64;
     const int tiles = (p->L + TL - 1) / TL;
     const size_t nslices = (size_t)tiles * slices;
     unsigned* slice_len = nullptr;
-    if (!dev_alloc(&p->slice_off, nslices + 1) || !dev_alloc(&p->col_len, (size_t)tiles * threads) ||
-        !dev_alloc(&slice_len, nslices)) {
+    if (!dev_alloc(&p->slice_off, nslices + 1) || !dev_alloc(&slice_len, nslices)) {
         if (slice_len) (void)hipFree(slice_len);
         return FFI_ERR_OUT_OF_MEMORY;
     }
-    hipLaunchKernelGGL(tile_count_kernel, dim3(tiles), dim3(threads), threads * sizeof(unsigned), s, lookup, p->L, p->K,
-                       TL, p->col_len, slice_len);
+    hipLaunchKernelGGL(tile_count_kernel, dim3(tiles), dim3(threads), 2 * threads * sizeof(unsigned), s, lookup, p->L, p->K,
+                       TL, slice_len);
     hipLaunchKernelGGL(slice_scan_kernel, dim3(1), dim3(1024), 0, s, slice_len, p->slice_off, (int)nslices,
                        p->d_scratch + 2);
     hipError_t e = hipGetLastError();
@@ -226,8 +244,6 @@ int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     const unsigned long long connections = (unsigned long long)p->L * p->K;
     if (rows * 64ull > 3ull * connections + 64ull * nslices || rows >= 0xffffffffull) return FFI_OK;   // too skewed
     if (!dev_alloc(&p->ent, (size_t)rows * 64)) return FFI_ERR_OUT_OF_MEMORY;
-    // every slot starts as padding: position 0, label TL (the all-zero row of the walking kernel)
-    hipLaunchKernelGGL(fill_u32_kernel, dim3(1024), dim3(kBlock), 0, s, p->ent, (size_t)rows * 64, (unsigned)TL);
     hipLaunchKernelGGL(tile_fill_kernel, dim3(tiles), dim3(threads), 0, s, lookup, p->L, p->K, TL, p->slice_off, p->ent);
     e = hipGetLastError();
     if (e == hipSuccess) e = hipStreamSynchronize(s);
@@ -235,7 +251,7 @@ int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     p->tiled = true;
     p->tile_labels = TL; p->threads = threads; p->slices = slices; p->tiles = tiles;
     p->total_rows = (long long)rows;
-    p->bytes = (size_t)rows * 64 * sizeof(unsigned) + (nslices + 1) * sizeof(unsigned) + (size_t)tiles * threads * sizeof(unsigned short);
+    p->bytes = (size_t)rows * 64 * sizeof(unsigned) + (nslices + 1) * sizeof(unsigned);
     return FFI_OK;
 }
 
