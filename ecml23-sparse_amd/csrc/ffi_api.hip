@@ -38,10 +38,7 @@ int plan_alloc(int L, int K, int N, ffi_plan** out) {
     if (hipGetDevice(&p->device) != hipSuccess) { delete p; return FFI_ERR_NO_DEVICE; }
     p->L = L; p->K = K; p->N = N;
     // the plan arrays themselves are sized and allocated by plan_build
-    bool ok = hipMalloc(&p->d_scratch, 8 * sizeof(unsigned long long)) == hipSuccess &&
-              hipHostMalloc(&p->h_scratch, 8 * sizeof(unsigned long long)) == hipSuccess;
-    if (!ok) {
-        (void)hipGetLastError();
+    if (plan_scratch_alloc(p) != FFI_OK) {
         plan_free(p);
         delete p;
         return FFI_ERR_OUT_OF_MEMORY;
@@ -50,29 +47,22 @@ int plan_alloc(int L, int K, int N, ffi_plan** out) {
     return FFI_OK;
 }
 
-// Finds or builds the cached plan for `lookup`; re-checks the content fingerprint on every call.
+// The cached plan for `lookup`, if there is one (moved to the most-recently-used end).
 // Caller holds g_cache_mutex.
-int cached_plan(const int32_t* lookup, const Dims& d, hipStream_t s, ffi_plan** out) {
-    int dev = -1;
-    if (hipGetDevice(&dev) != hipSuccess) return FFI_ERR_NO_DEVICE;
-    ffi_plan* hit = nullptr;
+ffi_plan* find_cached_plan(const int32_t* lookup, const Dims& d, int dev) {
     for (size_t i = 0; i < g_cache.size(); ++i) {
         ffi_plan* p = g_cache[i];
         if (p->device == dev && p->lookup == lookup && p->L == d.L && p->K == d.K && p->N == d.N) {
-            hit = p;
-            g_cache.erase(g_cache.begin() + i);   // move to the back (most recently used)
+            g_cache.erase(g_cache.begin() + i);
             g_cache.push_back(p);
-            break;
+            return p;
         }
     }
-    if (hit) {
-        unsigned long long fp = 0, bad = 0;
-        FFI_TRY(plan_fingerprint(hit, lookup, s, &fp, &bad));
-        if (bad) return FFI_ERR_BAD_LOOKUP;
-        if (fp != hit->fingerprint) FFI_TRY(plan_build(hit, lookup, s));
-        *out = hit;
-        return FFI_OK;
-    }
+    return nullptr;
+}
+
+// Builds a plan for a lookup that has none and adds it to the cache.  Caller holds g_cache_mutex.
+int create_cached_plan(const int32_t* lookup, const Dims& d, int dev, hipStream_t s, ffi_plan** out) {
     if (g_cache.size() >= kMaxCachedPlans) {
         // evict the least recently used plan of this device; its stream work must have drained
         for (size_t i = 0; i < g_cache.size(); ++i) {
@@ -92,6 +82,33 @@ int cached_plan(const int32_t* lookup, const Dims& d, hipStream_t s, ffi_plan** 
     g_cache.push_back(p);
     *out = p;
     return FFI_OK;
+}
+
+// Input gradient through the plan cache.  The lookup's content fingerprint is re-checked on every
+// call: its kernel goes first, then `between` (the weight-gradient launch, or nothing) is enqueued,
+// and the host waits for the fingerprint kernel alone, so that it learns the result, and enqueues
+// the input-gradient kernels, while the weight gradient is still running.
+template <class Between>
+int input_grad_cached(const int32_t* lookup, const float* weights, const float* out_grad, float* feature_grad,
+                      const Dims& d, hipStream_t s, Between between) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) return FFI_ERR_NO_DEVICE;
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    ffi_plan* p = find_cached_plan(lookup, d, dev);
+    if (p) FFI_TRY(plan_fingerprint_begin(p, lookup, s));
+    const int st_between = between();
+    if (p) {
+        unsigned long long fp = 0, bad = 0;
+        const int st_fp = plan_fingerprint_end(p, &fp, &bad);
+        if (st_between != FFI_OK) return st_between;
+        if (st_fp != FFI_OK) return st_fp;
+        if (bad) return FFI_ERR_BAD_LOOKUP;
+        if (fp != p->fingerprint) FFI_TRY(plan_build(p, lookup, s));
+    } else {
+        if (st_between != FFI_OK) return st_between;
+        FFI_TRY(create_cached_plan(lookup, d, dev, s, &p));
+    }
+    return launch_input_grad(p, weights, out_grad, feature_grad, d.B, d.tp, s);
 }
 
 }  // namespace
@@ -153,10 +170,7 @@ int ffi_input_grad_f32(const int32_t* lookup, const float* weights, const float*
     if (!lookup || !weights || !out_grad || !feature_grad) return FFI_ERR_NULL_POINTER;
     Dims d;
     FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
-    std::lock_guard<std::mutex> lock(g_cache_mutex);
-    ffi_plan* p = nullptr;
-    FFI_TRY(cached_plan(lookup, d, (hipStream_t)stream, &p));
-    return launch_input_grad(p, weights, out_grad, feature_grad, d.B, d.tp, (hipStream_t)stream);
+    return input_grad_cached(lookup, weights, out_grad, feature_grad, d, (hipStream_t)stream, [] { return (int)FFI_OK; });
 }
 
 int ffi_backward_f32(const float* features, const int32_t* lookup, const float* weights,
@@ -165,14 +179,13 @@ int ffi_backward_f32(const float* features, const int32_t* lookup, const float* 
                      ffi_stream_t stream) {
     if (!features || !lookup || !weights || !out_grad) return FFI_ERR_NULL_POINTER;
     if (!feature_grad && !weight_grad) return FFI_ERR_NULL_POINTER;
+    Dims d;
+    FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
+    hipStream_t s = (hipStream_t)stream;
     // weight gradient first, then input gradient, as backward.cpp:95-107 orders them
-    if (weight_grad)
-        FFI_TRY(ffi_weight_grad_f32(features, lookup, out_grad, weight_grad, batch, num_features, num_units, fan_in,
-                                    transposed, stream));
-    if (feature_grad)
-        FFI_TRY(ffi_input_grad_f32(lookup, weights, out_grad, feature_grad, batch, num_features, num_units, fan_in,
-                                   transposed, stream));
-    return FFI_OK;
+    auto wgrad = [&] { return weight_grad ? launch_weight_grad(features, lookup, out_grad, weight_grad, nullptr, d, s) : (int)FFI_OK; };
+    if (!feature_grad) return wgrad();
+    return input_grad_cached(lookup, weights, out_grad, feature_grad, d, s, wgrad);
 }
 
 int ffi_backward_bias_f32(const float* features, const int32_t* lookup, const float* weights,
@@ -182,12 +195,11 @@ int ffi_backward_bias_f32(const float* features, const int32_t* lookup, const fl
     if (!features || !lookup || !weights || !out_grad || !weight_grad || !bias_grad) return FFI_ERR_NULL_POINTER;
     Dims d;
     FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
+    hipStream_t s = (hipStream_t)stream;
     // the bias gradient (column sums of out_grad) is a by-product of the weight-gradient kernel
-    FFI_TRY(launch_weight_grad(features, lookup, out_grad, weight_grad, bias_grad, d, (hipStream_t)stream));
-    if (feature_grad)
-        FFI_TRY(ffi_input_grad_f32(lookup, weights, out_grad, feature_grad, batch, num_features, num_units, fan_in,
-                                   transposed, stream));
-    return FFI_OK;
+    auto wgrad = [&] { return launch_weight_grad(features, lookup, out_grad, weight_grad, bias_grad, d, s); };
+    if (!feature_grad) return wgrad();
+    return input_grad_cached(lookup, weights, out_grad, feature_grad, d, s, wgrad);
 }
 
 int ffi_forward_bf16_f32(const uint16_t* features, const int32_t* lookup, const uint16_t* weights, float* result,
@@ -291,9 +303,7 @@ int ffi_check_lookup(const int32_t* lookup, int64_t num_units, int64_t fan_in, i
     FFI_TRY(check_dims(1, num_features, num_units, fan_in, 0, &d));
     ffi_plan tmp;
     tmp.L = d.L; tmp.K = d.K; tmp.N = d.N;
-    if (hipMalloc(&tmp.d_scratch, 8 * sizeof(unsigned long long)) != hipSuccess ||
-        hipHostMalloc(&tmp.h_scratch, 8 * sizeof(unsigned long long)) != hipSuccess) {
-        (void)hipGetLastError();
+    if (plan_scratch_alloc(&tmp) != FFI_OK) {
         plan_free(&tmp);
         return FFI_ERR_OUT_OF_MEMORY;
     }

@@ -102,6 +102,8 @@ struct ffi_plan {
     int32_t* col_ptr = nullptr;
     unsigned long long* d_scratch = nullptr;  // fingerprint / counters (device)
     unsigned long long* h_scratch = nullptr;  // pinned mirror
+    hipEvent_t fp_done = nullptr;             // recorded behind the fingerprint kernel and its copy to h_scratch
+    int fp_slot = 0;                          // which pair of d_scratch words the next fingerprint adds into (0: [0,1], 1: [4,5])
     size_t bytes = 0;
 };
 
@@ -110,8 +112,14 @@ constexpr int kPlanTileLabels = 1024;     // a [1024+1][32] fp32 tile fits LDS
 constexpr int kEntLabelBits = 11;         // label-in-tile field of a plan slot (values 0..1024)
 constexpr unsigned kEntLabelMask = (1u << kEntLabelBits) - 1;
 int plan_build(ffi_plan* p, const int32_t* lookup, hipStream_t s);
+// Content fingerprint of `lookup` (and the count of ids outside [0,N)).  _begin enqueues the kernel
+// on `s` and returns; _end waits for that kernel only, not for what the caller enqueued on `s`
+// after it, so the host learns the result while later kernels are still running.
+int plan_fingerprint_begin(ffi_plan* p, const int32_t* lookup, hipStream_t s);
+int plan_fingerprint_end(ffi_plan* p, unsigned long long* out, unsigned long long* bad_ids);
 int plan_fingerprint(ffi_plan* p, const int32_t* lookup, hipStream_t s, unsigned long long* out,
                      unsigned long long* bad_ids);
+int plan_scratch_alloc(ffi_plan* p);
 void plan_free(ffi_plan* p);
 int launch_input_grad(const ffi_plan* p, const float* w, const float* g, float* gx, int B, bool tp,
                       hipStream_t s);

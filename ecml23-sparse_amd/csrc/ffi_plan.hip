@@ -28,7 +28,8 @@ __device__ __forceinline__ unsigned mix32(unsigned v) {
 // of the atomics.  Four ids per load when the array allows it.
 __global__ __launch_bounds__(kBlock) void fingerprint_kernel(const int32_t* __restrict__ idx,
                                                               size_t total, unsigned N,
-                                                              unsigned long long* __restrict__ out) {
+                                                              unsigned long long* __restrict__ out,
+                                                              unsigned long long* __restrict__ out_next) {
     unsigned long long h = 0;
     unsigned bad = 0;
     const size_t stride = (size_t)gridDim.x * kBlock;
@@ -66,12 +67,9 @@ __global__ __launch_bounds__(kBlock) void fingerprint_kernel(const int32_t* __re
         for (int i = 0; i < kBlock / 64; ++i) { hs += part[0][i]; bs += part[1][i]; }
         atomicAdd(&out[0], hs);
         if (bs) atomicAdd(&out[1], bs);
+        // the words the next call will add into (calls alternate between two pairs) start from zero
+        if (blockIdx.x == 0) { out_next[0] = 0; out_next[1] = 0; }
     }
-}
-
-__global__ __launch_bounds__(kBlock) void zero_u64_kernel(unsigned long long* p, int n) {
-    const int i = blockIdx.x * kBlock + threadIdx.x;
-    if (i < n) p[i] = 0;
 }
 
 // ---- tiled form ---------------------------------------------------------------------------------
@@ -312,18 +310,43 @@ int build_global(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
 
 }  // namespace
 
-int plan_fingerprint(ffi_plan* p, const int32_t* lookup, hipStream_t s, unsigned long long* out,
-                     unsigned long long* bad_ids) {
+// device/pinned scratch words and the fingerprint event of a plan
+int plan_scratch_alloc(ffi_plan* p) {
+    const bool ok = hipMalloc(&p->d_scratch, 8 * sizeof(unsigned long long)) == hipSuccess &&
+                    hipHostMalloc(&p->h_scratch, 8 * sizeof(unsigned long long)) == hipSuccess &&
+                    hipEventCreateWithFlags(&p->fp_done, hipEventDisableTiming) == hipSuccess &&
+                    hipMemset(p->d_scratch, 0, 8 * sizeof(unsigned long long)) == hipSuccess;
+    if (!ok) {
+        (void)hipGetLastError();
+        return FFI_ERR_OUT_OF_MEMORY;
+    }
+    return FFI_OK;
+}
+
+int plan_fingerprint_begin(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     const size_t total = (size_t)p->L * p->K;
-    hipLaunchKernelGGL(zero_u64_kernel, dim3(1), dim3(kBlock), 0, s, p->d_scratch, 2);
     const unsigned blocks = (unsigned)std::min<size_t>((total / 4 + kBlock - 1) / kBlock + 1, 2048);
-    hipLaunchKernelGGL(fingerprint_kernel, dim3(blocks), dim3(kBlock), 0, s, lookup, total, (unsigned)p->N, p->d_scratch);
+    unsigned long long* cur = p->d_scratch + (p->fp_slot ? 4 : 0);
+    unsigned long long* next = p->d_scratch + (p->fp_slot ? 0 : 4);
+    p->fp_slot ^= 1;
+    hipLaunchKernelGGL(fingerprint_kernel, dim3(blocks), dim3(kBlock), 0, s, lookup, total, (unsigned)p->N, cur, next);
     FFI_HIP_TRY(hipGetLastError());
-    FFI_HIP_TRY(hipMemcpyAsync(p->h_scratch, p->d_scratch, 2 * sizeof(unsigned long long), hipMemcpyDeviceToHost, s));
-    FFI_HIP_TRY(hipStreamSynchronize(s));
+    FFI_HIP_TRY(hipMemcpyAsync(p->h_scratch, cur, 2 * sizeof(unsigned long long), hipMemcpyDeviceToHost, s));
+    FFI_HIP_TRY(hipEventRecord(p->fp_done, s));
+    return FFI_OK;
+}
+
+int plan_fingerprint_end(ffi_plan* p, unsigned long long* out, unsigned long long* bad_ids) {
+    FFI_HIP_TRY(hipEventSynchronize(p->fp_done));
     *out = p->h_scratch[0];
     *bad_ids = p->h_scratch[1];
     return FFI_OK;
+}
+
+int plan_fingerprint(ffi_plan* p, const int32_t* lookup, hipStream_t s, unsigned long long* out,
+                     unsigned long long* bad_ids) {
+    FFI_TRY(plan_fingerprint_begin(p, lookup, s));
+    return plan_fingerprint_end(p, out, bad_ids);
 }
 
 int plan_build(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
@@ -354,7 +377,8 @@ void plan_free(ffi_plan* p) {
     free_arrays(p);
     if (p->d_scratch) (void)hipFree(p->d_scratch);
     if (p->h_scratch) (void)hipHostFree(p->h_scratch);
-    p->d_scratch = nullptr; p->h_scratch = nullptr;
+    if (p->fp_done) (void)hipEventDestroy(p->fp_done);
+    p->d_scratch = nullptr; p->h_scratch = nullptr; p->fp_done = nullptr;
 }
 
 }  // namespace ffi
