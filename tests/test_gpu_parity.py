@@ -161,6 +161,22 @@ def test_code_paths(ffi, shape, transposed):
     assert rel_err(gx, o_gx) <= GRAD_RTOL
 
 
+def test_columns_fed_by_one_label_parity(ffi):
+    # even labels connect to the lower half of the columns only, odd labels to the upper half: every
+    # column's connections come from labels of one parity, the worst case for the plan's
+    # alternating slot order (every second slot of a column is padding)
+    B, N, L, K = 70, 256, 5001, 16
+    x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=31)
+    half = N // 2
+    lookup = (lookup % half + (np.arange(L)[:, None] % 2) * half).astype(np.int32)
+    for transposed in (False, True):
+        xin = np.ascontiguousarray(x.T) if transposed else x
+        gx, gw = hip_backward(ffi, xin, lookup, w, g, transposed)
+        o_gx, o_gw = oracle.backward(xin, lookup, w, g, transposed=transposed)
+        assert rel_err(gx, o_gx) <= GRAD_RTOL
+        assert rel_err(gw, o_gw) <= GRAD_RTOL
+
+
 def test_skewed_lookup_uses_the_global_plan(ffi):
     # every connection points at one of two columns: the padded tiled plan would explode, the
     # library must fall back to the global column order and still be exact to tolerance
