@@ -19,7 +19,8 @@
  *   - every function returns FFI_OK (0) or a negative ffi_status instead of aborting, where the
  *     reference fail-fasts through gsl_Expects (forward.cu:19-28, backward.cu:27-40):
  *     null pointers, any dimension <= 0 or > INT32_MAX, num_units*fan_in > INT32_MAX.
- *   - the library is thread-safe; calls that share a plan or the internal plan cache serialise.
+ *   - the library is thread-safe; calls that share a plan or the internal plan cache serialise.  Calls that
+ *     use the same stream share that stream's internal workspaces: issue them from one thread at a time.
  */
 #ifndef FFI_HIP_H
 #define FFI_HIP_H
