@@ -84,10 +84,14 @@ int create_cached_plan(const int32_t* lookup, const Dims& d, int dev, hipStream_
     return FFI_OK;
 }
 
-// Input gradient through the plan cache.  The lookup's content fingerprint is re-checked on every
-// call: its kernel goes first, then `between` (the weight-gradient launch, or nothing) is enqueued,
-// and the host waits for the fingerprint kernel alone, so that it learns the result, and enqueues
-// the input-gradient kernels, while the weight gradient is still running.
+// Input gradient through the plan cache, with `between(plan)` (the weight-gradient launch, or
+// nothing) enqueued ahead of it.  The lookup's content fingerprint is re-checked on every call: its
+// kernel goes first, then `between` is enqueued with the cached plan, and the host waits for the
+// fingerprint kernel alone, so that it learns the result, and enqueues the input-gradient kernels,
+// while the weight gradient is still running.  If the lookup did change (a rewire), the plan is
+// rebuilt and `between` is enqueued again: it overwrites, in stream order, what the first launch
+// computed from the plan's outdated copy of the column ids (plan-driven kernels read the plan,
+// never the lookup, so that first launch is safe whatever the lookup holds now).
 template <class Between>
 int input_grad_cached(const int32_t* lookup, const float* weights, const float* out_grad, float* feature_grad,
                       const Dims& d, hipStream_t s, Between between) {
@@ -95,18 +99,21 @@ int input_grad_cached(const int32_t* lookup, const float* weights, const float* 
     if (hipGetDevice(&dev) != hipSuccess) return FFI_ERR_NO_DEVICE;
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     ffi_plan* p = find_cached_plan(lookup, d, dev);
-    if (p) FFI_TRY(plan_fingerprint_begin(p, lookup, s));
-    const int st_between = between();
     if (p) {
+        FFI_TRY(plan_fingerprint_begin(p, lookup, s));
+        const int st_between = between(p);
         unsigned long long fp = 0, bad = 0;
         const int st_fp = plan_fingerprint_end(p, &fp, &bad);
         if (st_between != FFI_OK) return st_between;
         if (st_fp != FFI_OK) return st_fp;
         if (bad) return FFI_ERR_BAD_LOOKUP;
-        if (fp != p->fingerprint) FFI_TRY(plan_build(p, lookup, s));
+        if (fp != p->fingerprint) {
+            FFI_TRY(plan_build(p, lookup, s));
+            FFI_TRY(between(p));
+        }
     } else {
-        if (st_between != FFI_OK) return st_between;
         FFI_TRY(create_cached_plan(lookup, d, dev, s, &p));
+        FFI_TRY(between(p));
     }
     return launch_input_grad(p, weights, out_grad, feature_grad, d.B, d.tp, s);
 }
@@ -170,7 +177,7 @@ int ffi_input_grad_f32(const int32_t* lookup, const float* weights, const float*
     if (!lookup || !weights || !out_grad || !feature_grad) return FFI_ERR_NULL_POINTER;
     Dims d;
     FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
-    return input_grad_cached(lookup, weights, out_grad, feature_grad, d, (hipStream_t)stream, [] { return (int)FFI_OK; });
+    return input_grad_cached(lookup, weights, out_grad, feature_grad, d, (hipStream_t)stream, [](const ffi_plan*) { return (int)FFI_OK; });
 }
 
 int ffi_backward_f32(const float* features, const int32_t* lookup, const float* weights,
@@ -183,8 +190,10 @@ int ffi_backward_f32(const float* features, const int32_t* lookup, const float* 
     FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
     hipStream_t s = (hipStream_t)stream;
     // weight gradient first, then input gradient, as backward.cpp:95-107 orders them
-    auto wgrad = [&] { return weight_grad ? launch_weight_grad(features, lookup, out_grad, weight_grad, nullptr, d, s) : (int)FFI_OK; };
-    if (!feature_grad) return wgrad();
+    auto wgrad = [&](const ffi_plan* plan) {
+        return weight_grad ? launch_weight_grad(features, lookup, out_grad, weight_grad, nullptr, d, s, plan) : (int)FFI_OK;
+    };
+    if (!feature_grad) return wgrad(nullptr);
     return input_grad_cached(lookup, weights, out_grad, feature_grad, d, s, wgrad);
 }
 
@@ -197,8 +206,8 @@ int ffi_backward_bias_f32(const float* features, const int32_t* lookup, const fl
     FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
     hipStream_t s = (hipStream_t)stream;
     // the bias gradient (column sums of out_grad) is a by-product of the weight-gradient kernel
-    auto wgrad = [&] { return launch_weight_grad(features, lookup, out_grad, weight_grad, bias_grad, d, s); };
-    if (!feature_grad) return wgrad();
+    auto wgrad = [&](const ffi_plan* plan) { return launch_weight_grad(features, lookup, out_grad, weight_grad, bias_grad, d, s, plan); };
+    if (!feature_grad) return wgrad(nullptr);
     return input_grad_cached(lookup, weights, out_grad, feature_grad, d, s, wgrad);
 }
 

@@ -8,6 +8,8 @@
 
 #include "ffi_hip.h"
 
+struct ffi_plan;
+
 namespace ffi {
 
 // Shape bundle, validated on the host before any launch.
@@ -56,8 +58,9 @@ int launch_transpose(const float* src, float* dst, int rows, int cols, hipStream
 // bias ([L], added to every row of out) and bias_grad ([L], column sums of g) may be null
 int launch_forward(const float* x, const int32_t* idx, const float* w, const float* bias, float* out, const Dims& d,
                    hipStream_t s);
+// `plan` (may be null): a plan of the same lookup whose arranged copy of the column ids the kernel may use
 int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float* gw, float* bias_grad, const Dims& d,
-                       hipStream_t s);
+                       hipStream_t s, const ffi_plan* plan = nullptr);
 // any shape (the tile kernels cover narrow inputs only)
 int launch_forward_wide(const float* x, const int32_t* idx, const float* w, const float* bias, float* out, const Dims& d,
                         hipStream_t s);
@@ -95,6 +98,10 @@ struct ffi_plan {
     unsigned* slice_off = nullptr;       // [tiles*slices + 1] first row of each slice
     unsigned* ent = nullptr;             // [total_rows*64]  (position in tile << 11) | label in tile;
                                          // padding slots hold label == tile_labels + parity (all-zero rows)
+    // arranged copy of the column ids for the weight gradient (narrow inputs only, else null):
+    // [chunks of 32 connections][L][32] entries of (connection inside the chunk << 11) | column id, each
+    // label's connections reordered so that even and odd columns alternate (see ffi_plan.hip)
+    unsigned short* idx16 = nullptr;
     // blocked global form
     int block_labels = 0;     // labels per block (bounds the part of out_grad that is live at a time)
     int nblocks = 0;
@@ -111,6 +118,7 @@ namespace ffi {
 constexpr int kPlanTileLabels = 1024;     // a [1024+1][32] fp32 tile fits LDS
 constexpr int kEntLabelBits = 11;         // label-in-tile field of a plan slot (values 0..1024)
 constexpr unsigned kEntLabelMask = (1u << kEntLabelBits) - 1;
+constexpr int kArrIdBits = 11;            // column-id field of an arranged entry (narrow inputs: ids < 1216)
 int plan_build(ffi_plan* p, const int32_t* lookup, hipStream_t s);
 // Content fingerprint of `lookup` (and the count of ids outside [0,N)).  _begin enqueues the kernel
 // on `s` and returns; _end waits for that kernel only, not for what the caller enqueued on `s`

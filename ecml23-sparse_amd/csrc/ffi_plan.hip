@@ -4,6 +4,7 @@
 // lookup[j,k] == n.  The plan lists those connections column by column so that they can be walked
 // sequentially, without atomics, in an order that never changes from run to run.
 #include "ffi_internal.h"
+#include "ffi_lds_tile.h"
 
 #include <algorithm>
 #include <cstring>
@@ -198,7 +199,8 @@ void free_arrays(ffi_plan* p) {
     if (p->col_ptr) (void)hipFree(p->col_ptr);
     if (p->slice_off) (void)hipFree(p->slice_off);
     if (p->ent) (void)hipFree(p->ent);
-    p->perm = nullptr; p->col_ptr = nullptr; p->slice_off = nullptr; p->ent = nullptr;
+    if (p->idx16) (void)hipFree(p->idx16);
+    p->perm = nullptr; p->col_ptr = nullptr; p->slice_off = nullptr; p->ent = nullptr; p->idx16 = nullptr;
     p->tiled = false; p->total_rows = 0; p->bytes = 0;
 }
 
@@ -310,6 +312,50 @@ int build_global(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
 
 }  // namespace
 
+// ---- arranged column ids for the weight gradient ------------------------------------------------
+// The weight-gradient kernel reads, per connection, the 128-byte LDS row of the connection's
+// column: even columns sit in one half of the LDS banks, odd columns in the other, and the LDS
+// serves 16 lanes per clock only if 8 of them read each half.  Lanes l and l+8 work on labels j and
+// j+8, so if the labels with bit 3 clear take their connections as even, odd, even, ... columns and
+// the others as odd, even, odd, ..., the two lanes always read opposite halves (as far as a label's
+// even and odd columns pair up; what is left over comes last).  One thread per (label, chunk of 32
+// connections); entry i of a unit = (connection inside the chunk << 11) | column id; units are
+// stored chunk-major ([chunk][label][32]) so that consecutive lanes work on consecutive labels.
+__global__ __launch_bounds__(kBlock) void arrange_units_kernel(const int32_t* __restrict__ idx, int L, int K, int nchunks,
+                                                                unsigned short* __restrict__ out) {
+    const long long u = (long long)blockIdx.x * kBlock + threadIdx.x;
+    if (u >= (long long)L * nchunks) return;
+    const int c = (int)(u / L), j = (int)(u - (long long)c * L);
+    const int k0 = c * 32, kn = min(32, K - k0);
+    const int32_t* row = idx + (size_t)j * K + k0;
+    const unsigned role = ((unsigned)j >> 3) & 1u;        // parity taken at even positions
+    unsigned nfirst = 0;
+    for (int k = 0; k < kn; ++k) nfirst += (((unsigned)row[k] & 1u) == role) ? 1u : 0u;
+    const unsigned m = min(nfirst, (unsigned)kn - nfirst);
+    unsigned short* dst = out + (size_t)u * 32;
+    unsigned tf = 0, ts = 0;
+    for (int k = 0; k < kn; ++k) {
+        const unsigned id = (unsigned)row[k];
+        const bool first = (id & 1u) == role;
+        const unsigned t = first ? tf++ : ts++;
+        const unsigned pos = t < m ? 2u * t + (first ? 0u : 1u) : 2u * m + (t - m);
+        dst[pos] = (unsigned short)(((unsigned)k << kArrIdBits) | id);
+    }
+    // a chunk the fan-in does not fill: the rest points at connection 31, which such a chunk never stores
+    for (int k = kn; k < 32; ++k) dst[k] = (unsigned short)(31u << kArrIdBits);
+}
+
+int build_arranged(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
+    const int nchunks = (p->K + 31) / 32;
+    const long long units = (long long)p->L * nchunks;
+    if (!dev_alloc(&p->idx16, (size_t)units * 32)) return FFI_ERR_OUT_OF_MEMORY;
+    hipLaunchKernelGGL(arrange_units_kernel, dim3((unsigned)((units + kBlock - 1) / kBlock)), dim3(kBlock), 0, s, lookup,
+                       p->L, p->K, nchunks, p->idx16);
+    FFI_HIP_TRY(hipGetLastError());
+    p->bytes += (size_t)units * 32 * sizeof(unsigned short);
+    return FFI_OK;
+}
+
 // device/pinned scratch words and the fingerprint event of a plan
 int plan_scratch_alloc(ffi_plan* p) {
     const bool ok = hipMalloc(&p->d_scratch, 8 * sizeof(unsigned long long)) == hipSuccess &&
@@ -365,6 +411,11 @@ int plan_build(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     if (!p->tiled) {
         free_arrays(p);
         int st = build_global(p, lookup, s);
+        if (st != FFI_OK) { free_arrays(p); return st; }
+    }
+    // (ids < 2^11 and an [N][32] fp32 tile in LDS: the shapes the narrow weight-gradient kernel takes)
+    if (tile_path_fits(p->N) && p->N < (1 << kArrIdBits)) {
+        int st = build_arranged(p, lookup, s);
         if (st != FFI_OK) { free_arrays(p); return st; }
     }
     p->lookup = lookup;

@@ -151,10 +151,114 @@ __global__ __launch_bounds__(kResThreads) void wgrad_resident_kernel(const float
     }
 }
 
+
+// ------------------------------------------------------------------------------------------------
+// The same kernel fed by a plan's arranged copy of the column ids (ffi_plan.hip): entry i of a unit
+// is (connection inside the chunk << 11) | column id, in an order in which lanes l and l+8 read
+// opposite halves of the LDS banks, and units are numbered chunk-major (u = chunk * L + label) so
+// that consecutive lanes work on consecutive labels.  Half the id traffic (16-bit entries), and the
+// LDS reads mostly free of bank conflicts.  Partial sum i of a unit belongs to connection
+// (entry i >> 11); the sums are put back in connection order through a thread-private 128-byte LDS
+// slot before they are stored.
+// ------------------------------------------------------------------------------------------------
+constexpr unsigned kArrIdMask = (1u << kArrIdBits) - 1;
+
+__global__ __launch_bounds__(kResThreads) void wgrad_arranged_kernel(const float* __restrict__ xT,
+                                                                     const unsigned short* __restrict__ idx16,
+                                                                     const float* __restrict__ g,
+                                                                     float* __restrict__ gw,
+                                                                     float* __restrict__ bias_grad, int B, int N,
+                                                                     int L, int K, int nchunks, int n1, int upb1,
+                                                                     int upb2) {
+    extern __shared__ __align__(16) float xs[];
+    const char* xs_bytes = reinterpret_cast<const char*>(xs);
+    const int lane = threadIdx.x & 63;
+    const int blk = blockIdx.x;
+    const long long total_units = (long long)L * nchunks;
+    const long long u_begin = blk < n1 ? (long long)blk * upb1 : (long long)n1 * upb1 + (long long)(blk - n1) * upb2;
+    const long long u_end = min(u_begin + (blk < n1 ? upb1 : upb2), total_units);
+    const int nbt = (B + kTileBatch - 1) / kTileBatch;
+
+    float res[kResUnits][kWgChunk];
+#pragma unroll
+    for (int q = 0; q < kResUnits; ++q)
+#pragma unroll
+        for (int k = 0; k < kWgChunk; ++k) res[q][k] = 0.f;
+    float gsum[kResUnits];                                 // column sums of out_grad (the bias gradient)
+#pragma unroll
+    for (int q = 0; q < kResUnits; ++q) gsum[q] = 0.f;
+
+    for (int bt = 0; bt < nbt; ++bt) {
+        const int b0 = bt * kTileBatch;
+        __syncthreads();                                   // everyone is done with the previous tile
+        stage_rows32<kResThreads, 8>(xs, xT, N, B, b0);
+        __syncthreads();
+        unsigned skew = (unsigned)(lane & 7) * 16u;
+        asm volatile("" : "+v"(skew));                     // keep the LDS addresses out of loop-invariant hoisting
+#pragma unroll
+        for (int q = 0; q < kResUnits; ++q) {
+            const long long ubase = u_begin + (long long)q * kResThreads;
+            if (ubase + (long long)(threadIdx.x & ~63u) < u_end) {          // the wavefront has units in this round
+                const long long u = min(ubase + (long long)threadIdx.x, u_end - 1);   // clamped: loads stay in bounds
+                const int j = (int)(u % L);
+                float gb[32];
+                load_rows32(g, L, b0, B, (unsigned)j, gb);
+                if (bias_grad != nullptr) {
+                    float t = gsum[q];
+#pragma unroll
+                    for (int b = 0; b < 32; ++b) t += gb[b];
+                    gsum[q] = t;
+                }
+                unsigned idp[kWgChunk / 2];                // two 16-bit entries per register
+                const uint4* erow = reinterpret_cast<const uint4*>(idx16 + (size_t)u * kWgChunk);
+#pragma unroll
+                for (int t = 0; t < kWgChunk / 8; ++t) {
+                    const uint4 v = erow[t];
+                    idp[4 * t] = v.x; idp[4 * t + 1] = v.y; idp[4 * t + 2] = v.z; idp[4 * t + 3] = v.w;
+                }
+                xor_permute_groups(gb, lane & 7);          // match the skewed chunk order of the gathers
+#pragma unroll
+                for (int k = 0; k < kWgChunk; ++k) {
+                    const unsigned e = (k & 1) ? (idp[k >> 1] >> 16) : idp[k >> 1];
+                    float4 xv[8];
+                    wgrad_reads(xs_bytes, ((e & kArrIdMask) << 7) | skew, xv);
+                    __builtin_amdgcn_sched_barrier(0);
+                    res[q][k] = wgrad_dot(xv, gb, res[q][k]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+    }
+    __syncthreads();                                       // xs is free: its first 64 KB become per-thread slots
+    float* slot = xs + (size_t)threadIdx.x * kWgChunk;
+    const bool vec4 = (K % 4 == 0) && (((uintptr_t)gw & 15) == 0);
+#pragma unroll
+    for (int q = 0; q < kResUnits; ++q) {
+        const long long u = u_begin + (long long)q * kResThreads + threadIdx.x;
+        if (u < u_end) {
+            const int c = (int)(u / L), j = (int)(u - (long long)c * L);
+            const int k0 = c * kWgChunk;
+            if (bias_grad != nullptr && c == 0) bias_grad[j] = gsum[q];
+            const unsigned short* erow = idx16 + (size_t)u * kWgChunk;
+#pragma unroll
+            for (int i = 0; i < kWgChunk; ++i) slot[erow[i] >> kArrIdBits] = res[q][i];
+            float* grow = gw + (size_t)j * K + k0;
+            if (vec4 && k0 + kWgChunk <= K) {
+#pragma unroll
+                for (int t = 0; t < kWgChunk / 4; ++t)
+                    *reinterpret_cast<float4*>(grow + 4 * t) = *reinterpret_cast<const float4*>(slot + 4 * t);
+            } else {
+                for (int k = 0; k < kWgChunk; ++k)
+                    if (k0 + k < K) grow[k] = slot[k];
+            }
+        }
+    }
+}
+
 }  // namespace
 
 int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float* gw, float* bias_grad, const Dims& d,
-                       hipStream_t s) {
+                       hipStream_t s, const ffi_plan* plan) {
     // (32 rows of out_grad must be reachable through 32-bit byte offsets)
     if (tile_path_fits(d.N) && d.L < (1 << 25)) {
         const float* xT = x;
@@ -181,6 +285,14 @@ int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float
         }
         const unsigned blocks = (unsigned)(n1 + n2);
         const int upb = (int)cap;
+        if (plan != nullptr && plan->idx16 != nullptr) {
+            // the unit slots of the final reordering need 128 bytes per thread
+            const size_t lds = std::max(tile_lds_bytes(d.N), (size_t)kResThreads * kWgChunk * sizeof(float));
+            FFI_HIP_TRY(hipFuncSetAttribute((const void*)wgrad_arranged_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+            hipLaunchKernelGGL(wgrad_arranged_kernel, dim3(blocks), dim3(kResThreads), lds, s, xT, plan->idx16, g, gw, bias_grad, d.B, d.N, d.L, d.K, nchunks, n1, upb, upb2);
+            FFI_HIP_TRY(hipGetLastError());
+            return FFI_OK;
+        }
         const size_t lds = tile_lds_bytes(d.N);
         const bool vec4 = (d.K % 4 == 0) && (((uintptr_t)gw | (uintptr_t)idx) % 16 == 0);
         if (vec4) {
