@@ -31,7 +31,7 @@ MEASURED_TRAFFIC_BYTES = {
 # GPU kernels behind each pass (one C-ABI call)
 PASS_KERNELS = {
     "forward": "fwd_lane32_kernel",
-    "weight_grad": "wgrad_resident_kernel",
+    "weight_grad": "wgrad_arranged_kernel",
     "input_grad": "igrad_permute_weights_kernel + igrad_tile_kernel + igrad_reduce_kernel",
 }
 
@@ -157,7 +157,7 @@ def main():
     iters = max(3, min(args.steps, 20))
     kernels = {
         "forward": lambda: check(lib.ffi_forward_f32(ptr(x), ptr(lookup), ptr(w), ptr(out), B, N, L, K, int(tp), sh)),
-        "weight_grad": lambda: check(lib.ffi_weight_grad_f32(ptr(x), ptr(lookup), ptr(g), ptr(gw), B, N, L, K, int(tp), sh)),
+        "weight_grad": lambda: check(lib.ffi_weight_grad_planned_f32(plan, ptr(x), ptr(lookup), ptr(g), ptr(gw), B, int(tp), sh)),
         "input_grad": lambda: check(lib.ffi_input_grad_planned_f32(plan, ptr(w), ptr(g), ptr(gx), B, int(tp), sh)),
     }
     kernel_ms = {name: time_kernel(fn, stream, iters) for name, fn in kernels.items()}

@@ -277,6 +277,18 @@ int ffi_input_grad_planned_f32(const ffi_plan* plan, const float* weights, const
     return launch_input_grad(plan, weights, out_grad, feature_grad, (int)batch, transposed != 0, (hipStream_t)stream);
 }
 
+int ffi_weight_grad_planned_f32(const ffi_plan* plan, const float* features, const int32_t* lookup,
+                                const float* out_grad, float* weight_grad, int64_t batch, int transposed,
+                                ffi_stream_t stream) {
+    if (!plan || !features || !lookup || !out_grad || !weight_grad) return FFI_ERR_NULL_POINTER;
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) return FFI_ERR_NO_DEVICE;
+    if (dev != plan->device) return FFI_ERR_BAD_ARGUMENT;
+    Dims d;
+    FFI_TRY(check_dims(batch, plan->N, plan->L, plan->K, transposed, &d));
+    return launch_weight_grad(features, lookup, out_grad, weight_grad, nullptr, d, (hipStream_t)stream, plan);
+}
+
 int ffi_cache_clear(void) {
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     int dev = -1;

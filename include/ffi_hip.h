@@ -106,6 +106,16 @@ int ffi_plan_destroy(ffi_plan* plan);
 int ffi_input_grad_planned_f32(const ffi_plan* plan, const float* weights, const float* out_grad,
                                float* feature_grad, int64_t batch, int transposed, ffi_stream_t stream);
 
+/*
+ * Weight gradient with an explicit plan of the same lookup matrix: for narrow inputs the kernel then
+ * reads the plan's 16-bit copy of the column ids, reordered per label so that its LDS reads are free
+ * of bank conflicts (ffi_backward_f32 does the same through its cached plan).  `lookup` is still
+ * needed for shapes the plan holds no such copy for.  No counterpart in the reference.
+ */
+int ffi_weight_grad_planned_f32(const ffi_plan* plan, const float* features, const int32_t* lookup,
+                                const float* out_grad, float* weight_grad, int64_t batch, int transposed,
+                                ffi_stream_t stream);
+
 /* Drops every cached plan and workspace of the calling thread's current device. */
 int ffi_cache_clear(void);
 /* Device bytes currently held by the library (plans + workspaces) on the current device. */

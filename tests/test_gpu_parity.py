@@ -161,6 +161,28 @@ def test_code_paths(ffi, shape, transposed):
     assert rel_err(gx, o_gx) <= GRAD_RTOL
 
 
+@pytest.mark.parametrize("shape", [(300, 700, 5000, 32), (33, 96, 9, 5), (128, 512, 4100, 100), (40, 1216, 2500, 36), (64, 1100, 3000, 12),
+                                   (48, 1300, 2000, 20)])
+def test_planned_weight_grad_code_paths(ffi, shape):
+    B, N, L, K = shape
+    x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=B + K)
+    dl, dg = dev(lookup), dev(g)
+    lib = ffi._lib.lib()
+    plan = ctypes.c_void_p()
+    ffi._lib.check(lib.ffi_plan_create(dl.data_ptr(), L, K, N, B, stream(), ctypes.byref(plan)))
+    try:
+        for transposed in (0, 1):
+            xin = np.ascontiguousarray(x.T) if transposed else x
+            dx = dev(xin)
+            gw = torch.full((L, K), float("nan"), device="cuda")
+            ffi._lib.check(lib.ffi_weight_grad_planned_f32(plan, dx.data_ptr(), dl.data_ptr(), dg.data_ptr(), gw.data_ptr(), B,
+                                                           transposed, stream()))
+            torch.cuda.synchronize()
+            assert rel_err(gw.cpu().numpy(), oracle.weight_grad(xin, lookup, w, g, transposed=bool(transposed))) <= GRAD_RTOL
+    finally:
+        ffi._lib.check(lib.ffi_plan_destroy(plan))
+
+
 def test_columns_fed_by_one_label_parity(ffi):
     # even labels connect to the lower half of the columns only, odd labels to the upper half: every
     # column's connections come from labels of one parity, the worst case for the plan's
@@ -295,8 +317,16 @@ def test_explicit_plan_matches_cached_path(ffi):
             ffi._lib.check(lib.ffi_input_grad_planned_f32(plan, dw.data_ptr(), dg.data_ptr(), gx.data_ptr(), B,
                                                           transposed, stream()))
             torch.cuda.synchronize()
-            ref = oracle.input_grad(x.T.copy() if transposed else x, lookup, w, g, transposed=bool(transposed))
+            xin = np.ascontiguousarray(x.T) if transposed else x
+            ref = oracle.input_grad(xin, lookup, w, g, transposed=bool(transposed))
             assert rel_err(gx.cpu().numpy(), ref) <= GRAD_RTOL
+            # the weight gradient fed by the plan's arranged copy of the column ids
+            gw = torch.full((L, K), float("nan"), device="cuda")
+            dx = dev(xin)
+            ffi._lib.check(lib.ffi_weight_grad_planned_f32(plan, dx.data_ptr(), dl.data_ptr(), dg.data_ptr(), gw.data_ptr(), B,
+                                                           transposed, stream()))
+            torch.cuda.synchronize()
+            assert rel_err(gw.cpu().numpy(), oracle.weight_grad(xin, lookup, w, g, transposed=bool(transposed))) <= GRAD_RTOL
     finally:
         ffi._lib.check(lib.ffi_plan_destroy(plan))
 
