@@ -45,6 +45,8 @@ def parse_args():
     ap.add_argument("--layout", default="nb", choices=["nb", "bn"],
                     help="features as [N,B] (the production 'Tp' op) or [B,N]")
     ap.add_argument("--seed", type=int, default=42)
+    ap.add_argument("--arranged", action="store_true",
+                    help="reorder every label's connections with ffi_arrange_connections_f32 first (same connection sets)")
     ap.add_argument("--cpu-labels", type=int, default=0, help="labels in the CPU-baseline sample (0 = auto)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-bytes", type=int, default=0,
@@ -119,6 +121,8 @@ def main():
     t = synth.make_inputs(cfg, seed=args.seed, device="cuda", transposed=tp)
     x, lookup, w, g = t["features"], t["lookup"], t["weights"], t["out_grad"]
     B, N, L, K = cfg.batch, cfg.num_features, cfg.num_units, cfg.fan_in
+    if args.arranged:
+        pkg.arrange_connections(lookup, w)
     out = torch.empty((B, L), device="cuda")
     gx = torch.empty_like(x)
     gw = torch.empty_like(w)
@@ -193,7 +197,8 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": f"{cfg.name}: FFI layer fwd+input-grad+weight-grad, batch {B}, {N} inputs, "
-                               f"{L} labels, fan-in {K}, features [{'N,B' if tp else 'B,N'}]",
+                               f"{L} labels, fan-in {K}, features [{'N,B' if tp else 'B,N'}]"
+                               + (", connections of each label reordered by ffi_arrange_connections_f32" if args.arranged else ""),
                    "label_samples_per_s": round(B * L / (ms_per_step * 1e-3), 1)},
         "roofline": roofline,
     }

@@ -24,6 +24,7 @@ from .fixed_fan_in_ops import (  # noqa: E402
     topk_scores,
     fan_in_sparse_matmul_bias,
     fan_in_sparse_matmul_tp_bias,
+    arrange_connections,
 )
 from . import custom_layer  # noqa: E402
 from .custom_layer import StratifiedRewireLayerV2, FixedFractionSelector, FixedMagnitudeSelector  # noqa: E402
@@ -40,6 +41,7 @@ __all__ = [
     "topk_scores",
     "fan_in_sparse_matmul_bias",
     "fan_in_sparse_matmul_tp_bias",
+    "arrange_connections",
     "StratifiedRewireLayerV2",
     "FixedFractionSelector",
     "FixedMagnitudeSelector",

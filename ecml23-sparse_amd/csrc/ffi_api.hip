@@ -289,6 +289,17 @@ int ffi_weight_grad_planned_f32(const ffi_plan* plan, const float* features, con
     return launch_weight_grad(features, lookup, out_grad, weight_grad, nullptr, d, (hipStream_t)stream, plan);
 }
 
+int ffi_arrange_connections_f32(int32_t* lookup, float* const* arrays, int n_arrays, int64_t num_units, int64_t fan_in,
+                                ffi_stream_t stream) {
+    if (!lookup || (n_arrays > 0 && !arrays)) return FFI_ERR_NULL_POINTER;
+    if (n_arrays < 0 || n_arrays > 4) return FFI_ERR_BAD_ARGUMENT;
+    for (int i = 0; i < n_arrays; ++i)
+        if (!arrays[i]) return FFI_ERR_NULL_POINTER;
+    Dims d;
+    FFI_TRY(check_dims(1, 1, num_units, fan_in, 0, &d));
+    return launch_arrange_in_place(lookup, arrays, n_arrays, d.L, d.K, (hipStream_t)stream);
+}
+
 int ffi_cache_clear(void) {
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     int dev = -1;

@@ -120,6 +120,7 @@ constexpr int kEntLabelBits = 11;         // label-in-tile field of a plan slot 
 constexpr unsigned kEntLabelMask = (1u << kEntLabelBits) - 1;
 constexpr int kArrIdBits = 11;            // column-id field of an arranged entry (narrow inputs: ids < 1216)
 int plan_build(ffi_plan* p, const int32_t* lookup, hipStream_t s);
+int launch_arrange_in_place(int32_t* lookup, float* const* arrays, int n_arrays, int L, int K, hipStream_t s);
 // Content fingerprint of `lookup` (and the count of ids outside [0,N)).  _begin enqueues the kernel
 // on `s` and returns; _end waits for that kernel only, not for what the caller enqueued on `s`
 // after it, so the host learns the result while later kernels are still running.

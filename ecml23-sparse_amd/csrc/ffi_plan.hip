@@ -310,8 +310,6 @@ int build_global(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     return FFI_OK;
 }
 
-}  // namespace
-
 // ---- arranged column ids for the weight gradient ------------------------------------------------
 // The weight-gradient kernel reads, per connection, the 128-byte LDS row of the connection's
 // column: even columns sit in one half of the LDS banks, odd columns in the other, and the LDS
@@ -345,6 +343,53 @@ __global__ __launch_bounds__(kBlock) void arrange_units_kernel(const int32_t* __
     for (int k = kn; k < 32; ++k) dst[k] = (unsigned short)(31u << kArrIdBits);
 }
 
+// The same reordering applied in place to the lookup matrix itself and to up to four float
+// matrices of its shape (weights, optimizer state): one thread per (label, chunk of 32).
+struct ArrangeArrays { float* a[4]; };
+__global__ __launch_bounds__(kBlock) void arrange_in_place_kernel(int32_t* __restrict__ idx, ArrangeArrays arr, int L, int K,
+                                                                   int nchunks) {
+    const long long u = (long long)blockIdx.x * kBlock + threadIdx.x;
+    if (u >= (long long)L * nchunks) return;
+    const int c = (int)(u / L), j = (int)(u - (long long)c * L);
+    const int k0 = c * 32, kn = min(32, K - k0);
+    int32_t* row = idx + (size_t)j * K + k0;
+    const unsigned role = ((unsigned)j >> 3) & 1u;
+    int32_t ids[32];
+    unsigned char pos[32];
+    unsigned nfirst = 0;
+    for (int k = 0; k < kn; ++k) { ids[k] = row[k]; nfirst += (((unsigned)ids[k] & 1u) == role) ? 1u : 0u; }
+    const unsigned m = min(nfirst, (unsigned)kn - nfirst);
+    unsigned tf = 0, ts = 0;
+    for (int k = 0; k < kn; ++k) {
+        const bool first = ((unsigned)ids[k] & 1u) == role;
+        const unsigned t = first ? tf++ : ts++;
+        pos[k] = (unsigned char)(t < m ? 2u * t + (first ? 0u : 1u) : 2u * m + (t - m));
+    }
+    for (int k = 0; k < kn; ++k) row[pos[k]] = ids[k];
+    for (int a = 0; a < 4; ++a) {
+        if (arr.a[a] == nullptr) continue;
+        float* frow = arr.a[a] + (size_t)j * K + k0;
+        float v[32];
+        for (int k = 0; k < kn; ++k) v[k] = frow[k];
+        for (int k = 0; k < kn; ++k) frow[pos[k]] = v[k];
+    }
+}
+
+}  // namespace
+
+int launch_arrange_in_place(int32_t* lookup, float* const* arrays, int n_arrays, int L, int K, hipStream_t s) {
+    ArrangeArrays arr{{nullptr, nullptr, nullptr, nullptr}};
+    for (int i = 0; i < n_arrays && i < 4; ++i) arr.a[i] = arrays[i];
+    const int nchunks = (K + 31) / 32;
+    const long long units = (long long)L * nchunks;
+    hipLaunchKernelGGL(arrange_in_place_kernel, dim3((unsigned)((units + kBlock - 1) / kBlock)), dim3(kBlock), 0, s, lookup, arr,
+                       L, K, nchunks);
+    FFI_HIP_TRY(hipGetLastError());
+    return FFI_OK;
+}
+
+namespace {
+
 int build_arranged(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     const int nchunks = (p->K + 31) / 32;
     const long long units = (long long)p->L * nchunks;
@@ -355,6 +400,8 @@ int build_arranged(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     p->bytes += (size_t)units * 32 * sizeof(unsigned short);
     return FFI_OK;
 }
+
+}  // namespace
 
 // device/pinned scratch words and the fingerprint event of a plan
 int plan_scratch_alloc(ffi_plan* p) {

@@ -51,7 +51,8 @@ class StratifiedRewireLayerV2(torch.nn.Module):
     """Fixed-fan-in sparse layer: ``units`` outputs, each fed by ``connections // units`` inputs."""
 
     def __init__(self, units: int, input_dim: int, *, connections: int | None = None, sparsity: float | None = None,
-                 use_bias: bool = True, rewire_selector=None, device="cuda", generator: torch.Generator | None = None):
+                 use_bias: bool = True, rewire_selector=None, arrange: bool = True, device="cuda",
+                 generator: torch.Generator | None = None):
         super().__init__()
         if int(units) != units or units < 0:
             raise ValueError(f"Received an invalid value for `units`, expected a positive integer, got {units}.")
@@ -78,6 +79,17 @@ class StratifiedRewireLayerV2(torch.nn.Module):
         # them as uint32, the same bits as the int32 kept here
         self.register_buffer("kernel_indices", self._random_sources(self.connections, device))
         self.bias = torch.nn.Parameter(torch.zeros(self.units, device=device)) if self.use_bias else None
+        # keep every label's connections in the order the kernels read fastest (see arrange_connections);
+        # no counterpart in the reference, where the order inside a row is arbitrary as well
+        self.arrange = bool(arrange) and torch.device(device).type == "cuda"
+        if self.arrange:
+            self.arrange_connections()
+
+    @torch.no_grad()
+    def arrange_connections(self, other_vars=None):
+        """Reorders each label's connections (indices, weights and ``other_vars`` together) in place."""
+        others = [] if other_vars is None else [o.view(-1, self.fan_in) for o in other_vars]
+        ops.arrange_connections(self.kernel_indices.view(-1, self.fan_in), self.kernel_weights.data.view(-1, self.fan_in), *others)
 
     @property
     def fan_in(self) -> int:
@@ -121,4 +133,6 @@ class StratifiedRewireLayerV2(torch.nn.Module):
             new_v = other.clone()
             new_v.reshape(-1)[locations] = 0
             outputs.append(new_v)
+        if self.arrange:
+            self.arrange_connections(outputs)
         return outputs

@@ -272,3 +272,27 @@ def fan_in_sparse_matmul_bias(features, lookup, weights, bias):
 def fan_in_sparse_matmul_tp_bias(features, lookup, weights, bias):
     """``fan_in_sparse_matmul_tp(features, lookup, weights) + bias`` in one kernel."""
     return FanInSparseMatmulBiasTp.apply(features, lookup, weights, bias)
+
+
+def arrange_connections(lookup, *arrays):
+    """Reorders, in place, the connections inside every row of ``lookup`` ([L,K] int32/uint32) so that
+    even and odd column ids alternate (which the kernels read faster), and applies the same
+    permutation to every float32 ``[L,K]`` tensor in ``arrays`` (weights, optimizer moments).
+
+    The order of a label's connections carries no meaning, so all results stay the same up to
+    summation order.  Idempotent.  Up to four arrays per call.
+    """
+    import ctypes
+
+    if lookup.dim() != 2 or lookup.dtype not in _INDEX_DTYPES or not lookup.is_cuda or not lookup.is_contiguous():
+        raise TypeError("lookup must be a contiguous int32/uint32 [L,K] device tensor")
+    if len(arrays) > 4:
+        raise ValueError("at most four arrays per call")
+    for a in arrays:
+        if a.dtype != torch.float32 or tuple(a.shape) != tuple(lookup.shape) or a.device != lookup.device or not a.is_contiguous():
+            raise TypeError("arrays must be contiguous float32 tensors of lookup's shape on lookup's device")
+    num_units, fan_in = lookup.shape
+    ptrs = (ctypes.c_void_p * max(len(arrays), 1))(*[a.data_ptr() for a in arrays])
+    with torch.cuda.device(lookup.device):
+        _lib.check(_lib.lib().ffi_arrange_connections_f32(lookup.data_ptr(), ptrs, len(arrays), num_units, fan_in,
+                                                          _stream_handle(lookup.device)))

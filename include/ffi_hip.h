@@ -116,6 +116,20 @@ int ffi_weight_grad_planned_f32(const ffi_plan* plan, const float* features, con
                                 const float* out_grad, float* weight_grad, int64_t batch, int transposed,
                                 ffi_stream_t stream);
 
+/*
+ * Optional layout help for the caller (no counterpart in the reference).  The order of a label's
+ * connections inside its row of lookup / weights carries no meaning, and the kernels run faster when
+ * even and odd column ids alternate along a row, starting with an even id in labels whose index has
+ * bit 3 clear and with an odd id in the others (the forward pass and the weight gradient then read
+ * both halves of the LDS banks in every clock).  This reorders every row of `lookup` that way, in
+ * place, per chunk of 32 connections, and applies the same permutation to up to four float matrices
+ * of the same shape (weights, optimizer moments, ...; `arrays` is a HOST array of `n_arrays` device
+ * pointers).  Results of all entry points are unchanged up to summation order; the call is
+ * idempotent.  A caller that rewires (sparse/custom_layer.py:32-43) may call it again afterwards.
+ */
+int ffi_arrange_connections_f32(int32_t* lookup, float* const* arrays, int n_arrays,
+                                int64_t num_units, int64_t fan_in, ffi_stream_t stream);
+
 /* Drops every cached plan and workspace of the calling thread's current device. */
 int ffi_cache_clear(void);
 /* Device bytes currently held by the library (plans + workspaces) on the current device. */

@@ -127,7 +127,7 @@ def test_layer_rewire(ffi):
     gen.manual_seed(11)
     B, N, units, K = 40, 256, 1500, 16
     layer = layer_mod.StratifiedRewireLayerV2(units, N, connections=units * K, rewire_selector=layer_mod.FixedFractionSelector(0.05),
-                                              generator=gen)
+                                              arrange=False, generator=gen)
     x = torch.relu(torch.randn(B, N, device="cuda", generator=gen)).requires_grad_(True)
     g = torch.randn(B, units, device="cuda", generator=gen) * 0.1
     layer(x).backward(g)                      # builds and caches the plan for the current indices
@@ -164,3 +164,71 @@ def test_selectors(ffi):
     # fraction 0.5 of 8 -> the 4th smallest magnitude (0.1) is the threshold, strictly smaller ones are selected
     assert layer_mod.FixedFractionSelector(0.5).select(w).tolist() == [False, False, False, True, False, True, False, True]
     assert layer_mod.FixedFractionSelector(0.0).select(w).sum().item() == 0
+
+
+def test_arrange_connections(ffi):
+    """Rows are permuted (indices, weights and extra arrays together), even and odd ids alternate as far
+    as they pair up, the call is idempotent, and the layer's results do not change beyond rounding."""
+    ops = ffi.fixed_fan_in_ops
+    rng = np.random.default_rng(3)
+    B, N, L, K = 40, 300, 1003, 40                      # two chunks per label, the second one partly filled
+    lookup = rng.integers(0, N, size=(L, K)).astype(np.int32)
+    w = rng.standard_normal((L, K)).astype(np.float32)
+    m = rng.standard_normal((L, K)).astype(np.float32)
+    x = np.maximum(rng.standard_normal((B, N)), 0).astype(np.float32)
+    g = (rng.standard_normal((B, L)) * 0.1).astype(np.float32)
+    dl, dw, dm = dev(lookup), dev(w), dev(m)
+    ops.arrange_connections(dl, dw, dm)
+    torch.cuda.synchronize()
+    al, aw, am = dl.cpu().numpy(), dw.cpu().numpy(), dm.cpu().numpy()
+    for lo, hi in ((0, 32), (32, 40)):                  # permutation inside each chunk, the three arrays together
+        before = np.stack([lookup[:, lo:hi], w[:, lo:hi].view(np.int32), m[:, lo:hi].view(np.int32)], axis=-1)
+        after = np.stack([al[:, lo:hi], aw[:, lo:hi].view(np.int32), am[:, lo:hi].view(np.int32)], axis=-1)
+        key = lambda a: np.sort(a.astype(np.int64)[..., 0] * (1 << 40) + (a.astype(np.int64)[..., 1] & 0xffffffff), axis=1)
+        np.testing.assert_array_equal(key(before), key(after))
+        # alternation: position i holds parity (i + role) & 1 for i < 2 * min(#even, #odd)
+        par = al[:, lo:hi] & 1
+        role = ((np.arange(L) >> 3) & 1)[:, None]
+        n_first = (par == role).sum(1, keepdims=True)
+        paired = 2 * np.minimum(n_first, (hi - lo) - n_first)
+        pos = np.arange(hi - lo)[None, :]
+        assert (((par ^ role ^ (pos & 1)) == 0) | (pos >= paired)).all()
+    dl2, dw2, dm2 = dl.clone(), dw.clone(), dm.clone()
+    ops.arrange_connections(dl2, dw2, dm2)              # idempotent
+    assert torch.equal(dl, dl2) and torch.equal(dw, dw2) and torch.equal(dm, dm2)
+    out_a = ops.fan_in_sparse_matmul(dev(x), dl, dw)
+    torch.cuda.synchronize()
+    assert rel_err(out_a.cpu().numpy(), oracle.forward(x, lookup, w)) <= FWD_RTOL
+    gx_a, gw_a = ops.fan_in_sparse_matmul_grad(dev(x), dl, dw, dev(g))
+    torch.cuda.synchronize()
+    want_gx, want_gw = oracle.backward(x, al, aw, g)
+    assert rel_err(gx_a.cpu().numpy(), want_gx) <= GRAD_RTOL and rel_err(gw_a.cpu().numpy(), want_gw) <= GRAD_RTOL
+    assert rel_err(want_gx, oracle.input_grad(x, lookup, w, g)) <= 1e-5     # same operator, rows reordered
+
+
+def test_layer_keeps_connections_arranged(ffi):
+    layer_mod = ffi.custom_layer
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(5)
+    units, N, K = 700, 128, 32
+    layer = layer_mod.StratifiedRewireLayerV2(units, N, connections=units * K, rewire_selector=layer_mod.FixedFractionSelector(0.1),
+                                              generator=gen)
+    def alternates(idx):
+        par = idx.view(-1, K).cpu().numpy() & 1
+        role = ((np.arange(units) >> 3) & 1)[:, None]
+        n_first = (par == role).sum(1, keepdims=True)
+        paired = 2 * np.minimum(n_first, K - n_first)
+        pos = np.arange(K)[None, :]
+        return bool((((par ^ role ^ (pos & 1)) == 0) | (pos >= paired)).all())
+    assert alternates(layer.kernel_indices)
+    w_before = layer.kernel_weights.detach().clone()
+    mom = torch.arange(units * K, device="cuda", dtype=torch.float32)
+    selected = layer.rewire_selector.select(w_before)
+    (new_mom,) = layer.rewire([mom])
+    assert alternates(layer.kernel_indices)
+    # per label: the same weights as before (reordered), and the moment entries travel with their weights
+    wb, wa = w_before.view(units, K).cpu().numpy(), layer.kernel_weights.detach().view(units, K).cpu().numpy()
+    np.testing.assert_array_equal(np.sort(wb, 1), np.sort(wa, 1))
+    want_mom = torch.where(selected, torch.zeros_like(mom), mom).view(units, K).cpu().numpy()
+    order_b, order_a = np.argsort(wb, 1, kind="stable"), np.argsort(wa, 1, kind="stable")
+    np.testing.assert_array_equal(np.take_along_axis(want_mom, order_b, 1), np.take_along_axis(new_mom.view(units, K).cpu().numpy(), order_a, 1))
