@@ -21,14 +21,15 @@ namespace {
 // the plan's slot order so that the main kernel reads them coalesced.  One workgroup per label
 // tile, one thread per column.  The tile's weights pass through LDS in pieces of kPermChunk floats
 // (read from HBM fully coalesced).  The wavefront walks the slice's rows together (every load is
-// one coalesced 256-byte row), eight rows per step; a lane stores the slots whose position lies in
+// one coalesced 128-byte row), kPermRows rows per step; a lane stores the slots whose position lies in
 // the staged piece.  A column's positions ascend inside each label parity and the two parities
 // alternate, so nothing of a later piece sits before the first step in which some lane met a
 // position beyond the current piece: the next piece resumes there.
 constexpr int kPermChunk = 16384;     // 64 KB of LDS per piece: two workgroups fit on a CU and overlap each other
+constexpr int kPermRows = 24;          // slot rows a wavefront handles per step
 constexpr int kPermChunkBig = 32768;  // 128 KB: a whole tile of 1024 labels x 32 connections in one piece
 __global__ __launch_bounds__(1024) void igrad_permute_weights_kernel(
-    const unsigned* __restrict__ ent, const unsigned* __restrict__ slice_off, const float* __restrict__ w,
+    const unsigned short* __restrict__ pos16, const unsigned* __restrict__ slice_off, const float* __restrict__ w,
     float* __restrict__ wp, int L, int K, int tile_labels, int chunk) {
     extern __shared__ __align__(16) float ws[];
     const int t = blockIdx.x, nthreads = blockDim.x;
@@ -39,7 +40,7 @@ __global__ __launch_bounds__(1024) void igrad_permute_weights_kernel(
     const unsigned npos = (unsigned)nl * (unsigned)K;
     const float* wt = w + (size_t)t * tile_labels * K;
     const bool vec = ((((uintptr_t)wt) & 15) == 0);
-    const unsigned* ep = ent + (size_t)row0 * 64 + lane;
+    const unsigned short* ep = pos16 + (size_t)row0 * 64 + lane;
     float* op = wp + (size_t)row0 * 64 + lane;
     unsigned lo = 0;                 // wave-uniform: rows below lo hold nothing of this or a later piece
     for (unsigned c0 = 0; c0 < npos; c0 += (unsigned)chunk) {
@@ -65,15 +66,16 @@ __global__ __launch_bounds__(1024) void igrad_permute_weights_kernel(
         __syncthreads();
         const unsigned hi = c0 + n;
         unsigned resume = 0xffffffffu;
-        for (unsigned i = lo; i < rows; i += 8) {
-            unsigned e8[8];
+        // kPermRows rows per step: all of a step's slot loads are in flight together
+        for (unsigned i = lo; i < rows; i += kPermRows) {
+            unsigned e[kPermRows];
 #pragma unroll
-            for (int q = 0; q < 8; ++q) e8[q] = ep[(size_t)min(i + q, rows - 1) * 64];
+            for (int q = 0; q < kPermRows; ++q) e[q] = ep[(size_t)min(i + q, rows - 1) * 64];
             bool any_later = false;
 #pragma unroll
-            for (int q = 0; q < 8; ++q) {
-                const unsigned pos = e8[q] >> kEntLabelBits;
-                const bool real = i + q < rows && (e8[q] & kEntLabelMask) < (unsigned)tile_labels;
+            for (int q = 0; q < kPermRows; ++q) {
+                const unsigned pos = e[q];
+                const bool real = i + q < rows && pos != kPadPos;
                 if (real && pos >= c0 && pos < hi) op[(size_t)(i + q) * 64] = ws[pos - c0];
                 if (c0 == 0 && i + q < rows && !real) op[(size_t)(i + q) * 64] = 0.f;     // padding slots
                 any_later |= real && pos >= hi;
@@ -86,7 +88,7 @@ __global__ __launch_bounds__(1024) void igrad_permute_weights_kernel(
 
 // The eight 16-byte reads of one row (chunk order skewed by the lane id) ...
 __device__ __forceinline__ void igrad_reads(const char* __restrict__ gs_bytes, unsigned e, unsigned skew, float4 (&v)[8]) {
-    const unsigned base = ((e & kEntLabelMask) << 7) | skew;
+    const unsigned base = (e << 7) | skew;
     v[0] = *reinterpret_cast<const float4*>(gs_bytes + skew_addr<0>(base));
     v[1] = *reinterpret_cast<const float4*>(gs_bytes + skew_addr<1>(base));
     v[2] = *reinterpret_cast<const float4*>(gs_bytes + skew_addr<2>(base));
@@ -111,7 +113,7 @@ __device__ __forceinline__ void igrad_fmas(const float4 (&v)[8], float wv, float
 // MAXT: largest workgroup the instantiation is launched with (sets the register budget);
 // LPT: labels of a tile staged per thread (tile_labels <= LPT * blockDim.x).
 template <int MAXT, int LPT>
-__global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned* __restrict__ ent, const float* __restrict__ wp,
+__global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* __restrict__ lab16, const float* __restrict__ wp,
                                   const unsigned* __restrict__ slice_off,
                                   const float* __restrict__ g, float* __restrict__ partial, int B, int L,
                                   int tile_labels, int tiles, int tiles_per_stream, int nbt) {
@@ -162,7 +164,7 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned* __rest
         const size_t sl = (size_t)t * (nthreads >> 6) + wave;
         const unsigned row0 = __builtin_amdgcn_readfirstlane(slice_off[sl]);
         const unsigned rows = __builtin_amdgcn_readfirstlane(slice_off[sl + 1]) - row0;
-        const unsigned* ep = ent + (size_t)row0 * 64 + lane;
+        const unsigned short* ep = lab16 + (size_t)row0 * 64 + lane;
         const float* wpp = wp + (size_t)row0 * 64 + lane;
         if (rows == 0) continue;               // wave-uniform: no column of this slice is used in the tile
         // Slots are fetched from memory kAhead rows ahead of the multiply-adds that use them (row
@@ -239,7 +241,7 @@ int launch_tiled(const ffi_plan* p, const float* w, const float* g, float* gx, i
     // a tile's weights in one piece when they fit (one walk over the slots instead of one per piece)
     const int chunk = ((long long)p->tile_labels * p->K <= kPermChunkBig) ? kPermChunkBig : kPermChunk;
     FFI_HIP_TRY(hipFuncSetAttribute((const void*)igrad_permute_weights_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, chunk * 4));
-    hipLaunchKernelGGL(igrad_permute_weights_kernel, dim3(p->tiles), dim3(p->threads), chunk * sizeof(float), s, p->ent,
+    hipLaunchKernelGGL(igrad_permute_weights_kernel, dim3(p->tiles), dim3(p->threads), chunk * sizeof(float), s, p->pos16,
                        p->slice_off, w, wp, p->L, p->K, p->tile_labels, chunk);
     const size_t lds = tile_lds_bytes(p->tile_labels + 2);      // + the two all-zero rows
     const dim3 grid(streams * nbt), block(p->threads);
@@ -247,7 +249,7 @@ int launch_tiled(const ffi_plan* p, const float* w, const float* g, float* gx, i
     do {                                                                                                                \
         FFI_HIP_TRY(hipFuncSetAttribute((const void*)igrad_tile_kernel<MAXT, LPT>,                                      \
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));                        \
-        hipLaunchKernelGGL((igrad_tile_kernel<MAXT, LPT>), grid, block, lds, s, p->ent, wp, p->slice_off, g, \
+        hipLaunchKernelGGL((igrad_tile_kernel<MAXT, LPT>), grid, block, lds, s, p->lab16, wp, p->slice_off, g, \
                            partial, B, p->L, p->tile_labels, p->tiles, tps, nbt);                                       \
     } while (0)
     // the plan sizes its tiles so that one of these fits: tile_labels <= LPT * threads

@@ -73,7 +73,7 @@ int launch_weight_grad_wide(const float* x, const int32_t* idx, const float* g, 
 //
 // tiled == true (narrow inputs): labels are cut into tiles of `tile_labels`; inside a tile the
 // connections are grouped by column, and the columns into slices of 64 (one per wavefront).  A
-// slice is stored slot-major: row i of the slice holds the i-th connection of each of its 64
+// slice is stored slot-major (two 16-bit arrays): row i of the slice holds the i-th connection of each of its 64
 // columns (so a wavefront reads 256 contiguous bytes per step), padded to the longest column of
 // the slice.  Inside a column the slots alternate between even and odd labels (which parity comes
 // first depends on the lane, see ffi_plan.hip), positions ascend inside each parity, and holes are
@@ -96,8 +96,10 @@ struct ffi_plan {
     int tiles = 0;            // ceil(L / tile_labels)
     long long total_rows = 0; // rows of 64 entries over all slices
     unsigned* slice_off = nullptr;       // [tiles*slices + 1] first row of each slice
-    unsigned* ent = nullptr;             // [total_rows*64]  (position in tile << 11) | label in tile;
-                                         // padding slots hold label == tile_labels + parity (all-zero rows)
+    unsigned short* lab16 = nullptr;     // [total_rows*64] label (inside the tile) of each slot; padding slots hold
+                                         // tile_labels + parity (two all-zero rows of the walking kernel)
+    unsigned short* pos16 = nullptr;     // [total_rows*64] position (inside the tile's rows of lookup) of each slot;
+                                         // kPadPos in padding slots
     // arranged copy of the column ids for the weight gradient (narrow inputs only, else null):
     // [chunks of 32 connections][L][32] entries of (connection inside the chunk << 11) | column id, each
     // label's connections reordered so that even and odd columns alternate (see ffi_plan.hip)
@@ -116,8 +118,7 @@ struct ffi_plan {
 
 namespace ffi {
 constexpr int kPlanTileLabels = 1024;     // a [1024+1][32] fp32 tile fits LDS
-constexpr int kEntLabelBits = 11;         // label-in-tile field of a plan slot (values 0..1024)
-constexpr unsigned kEntLabelMask = (1u << kEntLabelBits) - 1;
+constexpr unsigned kPadPos = 0xffffu;      // pos16 of a padding slot; real positions are below it (tile_labels * K <= 0xffff)
 constexpr int kArrIdBits = 11;            // column-id field of an arranged entry (narrow inputs: ids < 1216)
 int plan_build(ffi_plan* p, const int32_t* lookup, hipStream_t s);
 int launch_arrange_in_place(int32_t* lookup, float* const* arrays, int n_arrays, int L, int K, hipStream_t s);

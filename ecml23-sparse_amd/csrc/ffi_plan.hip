@@ -135,11 +135,13 @@ __global__ __launch_bounds__(1024) void slice_scan_kernel(const unsigned* __rest
 // One workgroup per label tile, one thread per column n.  The tile's column ids pass through LDS
 // in chunks; every thread scans them in flat-position order and places the ones equal to its
 // column (see column_slots for the order), so the result is deterministic without any sort.
-// ent = (position inside the tile << 11) | label inside the tile; the slots a column leaves empty
-// up to the slice's length become padding: position 0, label tile_labels + parity (all-zero rows).
+// Per slot: lab16 = label inside the tile, pos16 = position inside the tile's rows of lookup; the
+// slots a column leaves empty up to the slice's length become padding: pos16 = kPadPos, lab16 =
+// tile_labels + parity (all-zero rows).
 constexpr int kFillChunk = 8192;
 __global__ void tile_fill_kernel(const int32_t* __restrict__ idx, int L, int K, int tile_labels,
-                                 const unsigned* __restrict__ slice_off, unsigned* __restrict__ ent) {
+                                 const unsigned* __restrict__ slice_off, unsigned short* __restrict__ lab16,
+                                 unsigned short* __restrict__ pos16) {
     __shared__ __align__(16) int keys[kFillChunk];
     const int t = blockIdx.x, nthreads = blockDim.x;
     const int j0 = t * tile_labels;
@@ -150,10 +152,14 @@ __global__ void tile_fill_kernel(const int32_t* __restrict__ idx, int L, int K, 
     const size_t sl = (size_t)t * (nthreads >> 6) + (threadIdx.x >> 6);
     const size_t row0 = slice_off[sl];
     const unsigned rows = slice_off[sl + 1] - slice_off[sl];
-    unsigned* dst = ent + row0 * 64 + (threadIdx.x & 63);
+    unsigned short* dlab = lab16 + row0 * 64 + (threadIdx.x & 63);
+    unsigned short* dpos = pos16 + row0 * 64 + (threadIdx.x & 63);
     const unsigned first = parity_first(threadIdx.x);
     // padding everywhere first; the thread's own slots are then overwritten (same thread: ordered)
-    for (unsigned r = 0; r < rows; ++r) dst[(size_t)r * 64] = (unsigned)tile_labels + ((r & 1u) ^ first);
+    for (unsigned r = 0; r < rows; ++r) {
+        dlab[(size_t)r * 64] = (unsigned short)((unsigned)tile_labels + ((r & 1u) ^ first));
+        dpos[(size_t)r * 64] = (unsigned short)kPadPos;
+    }
     unsigned seen[2] = {0u, 0u};  // labels of each parity placed so far
     int label = 0, kk = 0;        // label and connection slot of the entry under the cursor
     for (int c0 = 0; c0 < total; c0 += kFillChunk) {
@@ -166,7 +172,8 @@ __global__ void tile_fill_kernel(const int32_t* __restrict__ idx, int L, int K, 
                 const unsigned par = (unsigned)label & 1u;
                 const unsigned t2 = par ? seen[1]++ : seen[0]++;
                 const unsigned slot = 2u * t2 + (par ^ first);
-                dst[(size_t)slot * 64] = ((unsigned)(c0 + e) << kEntLabelBits) | (unsigned)label;
+                dlab[(size_t)slot * 64] = (unsigned short)label;
+                dpos[(size_t)slot * 64] = (unsigned short)(c0 + e);
             }
             if (++kk == K) { kk = 0; ++label; }
         }
@@ -198,9 +205,10 @@ void free_arrays(ffi_plan* p) {
     if (p->perm) (void)hipFree(p->perm);
     if (p->col_ptr) (void)hipFree(p->col_ptr);
     if (p->slice_off) (void)hipFree(p->slice_off);
-    if (p->ent) (void)hipFree(p->ent);
+    if (p->lab16) (void)hipFree(p->lab16);
+    if (p->pos16) (void)hipFree(p->pos16);
     if (p->idx16) (void)hipFree(p->idx16);
-    p->perm = nullptr; p->col_ptr = nullptr; p->slice_off = nullptr; p->ent = nullptr; p->idx16 = nullptr;
+    p->perm = nullptr; p->col_ptr = nullptr; p->slice_off = nullptr; p->lab16 = nullptr; p->pos16 = nullptr; p->idx16 = nullptr;
     p->tiled = false; p->total_rows = 0; p->bytes = 0;
 }
 
@@ -222,7 +230,9 @@ int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     // every thread of the kernel that walks the plan stages at most two labels of a tile (one when
     // the workgroup is larger than 768 threads and registers are scarcer)
     // (even, so that label parity inside a tile is the parity of the LDS row)
-    const int TL = (std::min(std::min(kPlanTileLabels, p->L), threads > 768 ? threads : 2 * threads) + 1) & ~1;
+    // and small enough for the positions inside a tile to fit 16 bits
+    const int TL = std::min((std::min(std::min(kPlanTileLabels, p->L), threads > 768 ? threads : 2 * threads) + 1) & ~1,
+                            (int)((kPadPos - 1) / (unsigned)p->K) & ~1);
     const int slices = threads / 64;
     const int tiles = (p->L + TL - 1) / TL;
     const size_t nslices = (size_t)tiles * slices;
@@ -243,15 +253,16 @@ int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     const unsigned long long rows = p->h_scratch[2];
     const unsigned long long connections = (unsigned long long)p->L * p->K;
     if (rows * 64ull > 3ull * connections + 64ull * nslices || rows >= 0xffffffffull) return FFI_OK;   // too skewed
-    if (!dev_alloc(&p->ent, (size_t)rows * 64)) return FFI_ERR_OUT_OF_MEMORY;
-    hipLaunchKernelGGL(tile_fill_kernel, dim3(tiles), dim3(threads), 0, s, lookup, p->L, p->K, TL, p->slice_off, p->ent);
+    if (!dev_alloc(&p->lab16, (size_t)rows * 64) || !dev_alloc(&p->pos16, (size_t)rows * 64)) return FFI_ERR_OUT_OF_MEMORY;
+    hipLaunchKernelGGL(tile_fill_kernel, dim3(tiles), dim3(threads), 0, s, lookup, p->L, p->K, TL, p->slice_off, p->lab16,
+                       p->pos16);
     e = hipGetLastError();
     if (e == hipSuccess) e = hipStreamSynchronize(s);
     if (e != hipSuccess) return hip_fail(e);
     p->tiled = true;
     p->tile_labels = TL; p->threads = threads; p->slices = slices; p->tiles = tiles;
     p->total_rows = (long long)rows;
-    p->bytes = (size_t)rows * 64 * sizeof(unsigned) + (nslices + 1) * sizeof(unsigned);
+    p->bytes = (size_t)rows * 64 * 2 * sizeof(unsigned short) + (nslices + 1) * sizeof(unsigned);
     return FFI_OK;
 }
 
@@ -447,11 +458,11 @@ int plan_build(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     FFI_TRY(plan_fingerprint(p, lookup, s, &fp, &bad));
     if (bad != 0) return FFI_ERR_BAD_LOOKUP;   // also keeps the build kernels' LDS counters in range
     // a rebuild replaces the arrays: whatever still reads the old ones must have drained
-    if (p->perm || p->ent) FFI_HIP_TRY(hipDeviceSynchronize());
+    if (p->perm || p->lab16 || p->idx16) FFI_HIP_TRY(hipDeviceSynchronize());
     free_arrays(p);
-    // tiled form: one thread per column (N <= 1024) and positions inside a tile in 21 bits
+    // tiled form: one thread per column (N <= 1024), tiles of at least 62 labels with positions in 16 bits
     // (and 32 rows of out_grad within 32-bit byte offsets, as the kernels' buffer loads need)
-    if (p->N <= 1024 && (long long)kPlanTileLabels * p->K < (1ll << (32 - kEntLabelBits)) && p->L < (1 << 25)) {
+    if (p->N <= 1024 && p->K <= 1024 && p->L < (1 << 25)) {
         int st = build_tiled(p, lookup, s);
         if (st != FFI_OK) { free_arrays(p); return st; }
     }
