@@ -238,8 +238,9 @@ int launch_tiled(const ffi_plan* p, const float* w, const float* g, float* gx, i
     float* partial = nullptr;
     FFI_TRY(workspace_get(s, kWsFeaturesT, std::max<size_t>(slots, 1) * sizeof(float), (void**)&wp));
     FFI_TRY(workspace_get(s, kWsPartials, (size_t)streams * p->threads * bpad * sizeof(float), (void**)&partial));
-    // a tile's weights in one piece when they fit (one walk over the slots instead of one per piece)
-    const int chunk = ((long long)p->tile_labels * p->K <= kPermChunkBig) ? kPermChunkBig : kPermChunk;
+    // large pieces (a whole tile of 1024 labels x 32 connections in one) as soon as the small one does not hold the
+    // tile: every piece costs a walk over the tile's slots
+    const int chunk = ((long long)p->tile_labels * p->K <= kPermChunk) ? kPermChunk : kPermChunkBig;
     FFI_HIP_TRY(hipFuncSetAttribute((const void*)igrad_permute_weights_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, chunk * 4));
     hipLaunchKernelGGL(igrad_permute_weights_kernel, dim3(p->tiles), dim3(p->threads), chunk * sizeof(float), s, p->pos16,
                        p->slice_off, w, wp, p->L, p->K, p->tile_labels, chunk);
