@@ -87,16 +87,21 @@ __global__ __launch_bounds__(1024) void igrad_permute_weights_kernel(
 }
 
 // The eight 16-byte reads of one row (chunk order skewed by the lane id) ...
-__device__ __forceinline__ void igrad_reads(const char* __restrict__ gs_bytes, unsigned e, unsigned skew, float4 (&v)[8]) {
-    const unsigned base = (e << 7) | skew;
-    v[0] = *reinterpret_cast<const float4*>(gs_bytes + skew_addr<0>(base));
-    v[1] = *reinterpret_cast<const float4*>(gs_bytes + skew_addr<1>(base));
-    v[2] = *reinterpret_cast<const float4*>(gs_bytes + skew_addr<2>(base));
-    v[3] = *reinterpret_cast<const float4*>(gs_bytes + skew_addr<3>(base));
-    v[4] = *reinterpret_cast<const float4*>(gs_bytes + skew_addr<4>(base));
-    v[5] = *reinterpret_cast<const float4*>(gs_bytes + skew_addr<5>(base));
-    v[6] = *reinterpret_cast<const float4*>(gs_bytes + skew_addr<6>(base));
-    v[7] = *reinterpret_cast<const float4*>(gs_bytes + skew_addr<7>(base));
+// `skewbase` = LDS address of the tile + (lane & 7) * 16; the tile is 128-byte aligned, so the chunk
+// bits can be flipped with XOR after the row offset has been added (one add + seven XORs per row).
+typedef float lds_v4f __attribute__((ext_vector_type(4)));
+typedef const lds_v4f __attribute__((address_space(3)))* lds_v4f_ptr;
+template <int C>
+__device__ __forceinline__ float4 igrad_read_chunk(unsigned base) {
+    const lds_v4f t = *(lds_v4f_ptr)(size_t)(skew_addr<C>(base));
+    return make_float4(t.x, t.y, t.z, t.w);
+}
+__device__ __forceinline__ void igrad_reads(unsigned e, unsigned skewbase, float4 (&v)[8]) {
+    const unsigned base = (e << 7) + skewbase;
+    v[0] = igrad_read_chunk<0>(base); v[1] = igrad_read_chunk<1>(base);
+    v[2] = igrad_read_chunk<2>(base); v[3] = igrad_read_chunk<3>(base);
+    v[4] = igrad_read_chunk<4>(base); v[5] = igrad_read_chunk<5>(base);
+    v[6] = igrad_read_chunk<6>(base); v[7] = igrad_read_chunk<7>(base);
 }
 // ... and the 32 multiply-adds that consume them.
 __device__ __forceinline__ void igrad_fmas(const float4 (&v)[8], float wv, float (&acc)[32]) {
@@ -116,7 +121,7 @@ template <int MAXT, int LPT>
 __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* __restrict__ lab16, const float* __restrict__ wp,
                                   const unsigned* __restrict__ slice_off,
                                   const float* __restrict__ g, float* __restrict__ partial, int B, int L,
-                                  int tile_labels, int tiles, int tiles_per_stream, int nbt) {
+                                  int tile_labels, int tiles, int tiles_per_stream, int nbt, unsigned total_rows) {
     extern __shared__ __align__(16) float gs[];
     char* gs_bytes = reinterpret_cast<char*>(gs);
     const int nthreads = blockDim.x;
@@ -125,7 +130,13 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
     const int b0 = bt * kTileBatch;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const unsigned skew = (unsigned)(lane & 7) * 16u;
+    // LDS address of gs (a 32-bit offset inside the workgroup's LDS) plus the lane's skew
+    const unsigned skewbase = (unsigned)(size_t)(__attribute__((address_space(3))) float*)gs + skew;
     const int t_begin = stream * tiles_per_stream, t_end = min(t_begin + tiles_per_stream, tiles);
+    // plan slots and permuted weights, addressed as (scalar row offset) + (lane offset); 4-GB buffers at most
+    const buffer_rsrc lab_rsrc = make_rsrc(lab16, (size_t)total_rows * 128u);
+    const buffer_rsrc wp_rsrc = make_rsrc(wp, (size_t)total_rows * 256u);
+    const unsigned lane2 = (unsigned)lane * 2u, lane4 = (unsigned)lane * 4u;
 
     float acc[32];
 #pragma unroll
@@ -164,20 +175,23 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
         const size_t sl = (size_t)t * (nthreads >> 6) + wave;
         const unsigned row0 = __builtin_amdgcn_readfirstlane(slice_off[sl]);
         const unsigned rows = __builtin_amdgcn_readfirstlane(slice_off[sl + 1]) - row0;
-        const unsigned short* ep = lab16 + (size_t)row0 * 64 + lane;
-        const float* wpp = wp + (size_t)row0 * 64 + lane;
         if (rows == 0) continue;               // wave-uniform: no column of this slice is used in the tile
-        // Slots are fetched from memory kAhead rows ahead of the multiply-adds that use them (row
-        // indices clamped, not predicated, so the loads carry no branches).
+        // Slots are fetched from memory kAhead rows ahead of the multiply-adds that use them, through
+        // buffer loads whose row offset is a scalar (row indices clamped, not predicated, so the loads
+        // carry neither branches nor per-lane address arithmetic).
         constexpr int kAhead = 4;
         const unsigned last = rows - 1;
+        auto load_lab = [&](unsigned r) {
+            return (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(lab_rsrc, lane2, (row0 + r) * 128u, 0);
+        };
+        auto load_w = [&](unsigned r) { return buffer_load_f32(wp_rsrc, lane4, (row0 + r) * 256u); };
         unsigned e4[kAhead];
         float w4[kAhead];
 #pragma unroll
         for (int q = 0; q < kAhead; ++q) {
             const unsigned r = min((unsigned)q, last);
-            e4[q] = ep[(size_t)r * 64];
-            w4[q] = wpp[(size_t)r * 64];
+            e4[q] = load_lab(r);
+            w4[q] = load_w(r);
         }
         for (unsigned i = 0; i < rows; i += kAhead) {
             unsigned en[kAhead];
@@ -185,13 +199,13 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
 #pragma unroll
             for (int q = 0; q < kAhead; ++q) {
                 const unsigned r = min(i + kAhead + q, last);
-                en[q] = ep[(size_t)r * 64];
-                wn[q] = wpp[(size_t)r * 64];
+                en[q] = load_lab(r);
+                wn[q] = load_w(r);
             }
             // keep these loads here, a whole group of rows ahead of their use (left alone, the
             // scheduler sinks them below the multiply-adds and every group waits a full round trip)
             __builtin_amdgcn_sched_barrier(0);
-            // branch-free: padding slots carry weight 0 and point at the all-zero LDS row, rows past
+            // branch-free: padding slots carry weight 0 and point at an all-zero LDS row, rows past
             // the end of the slice are redirected there too
 #pragma unroll
             for (int q = 0; q < kAhead; ++q) {
@@ -199,7 +213,7 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
                 const unsigned e = in ? e4[q] : (unsigned)tile_labels;
                 const float wv = in ? w4[q] : 0.f;
                 float4 xv[8];
-                igrad_reads(gs_bytes, e, skew, xv);
+                igrad_reads(e, skewbase, xv);
                 igrad_fmas(xv, wv, acc);
             }
 #pragma unroll
@@ -251,7 +265,7 @@ int launch_tiled(const ffi_plan* p, const float* w, const float* g, float* gx, i
         FFI_HIP_TRY(hipFuncSetAttribute((const void*)igrad_tile_kernel<MAXT, LPT>,                                      \
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));                        \
         hipLaunchKernelGGL((igrad_tile_kernel<MAXT, LPT>), grid, block, lds, s, p->lab16, wp, p->slice_off, g, \
-                           partial, B, p->L, p->tile_labels, p->tiles, tps, nbt);                                       \
+                           partial, B, p->L, p->tile_labels, p->tiles, tps, nbt, (unsigned)p->total_rows);                                       \
     } while (0)
     // the plan sizes its tiles so that one of these fits: tile_labels <= LPT * threads
     if (p->threads <= 768) {

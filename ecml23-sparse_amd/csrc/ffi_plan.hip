@@ -252,7 +252,8 @@ int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     if (e != hipSuccess) return hip_fail(e);
     const unsigned long long rows = p->h_scratch[2];
     const unsigned long long connections = (unsigned long long)p->L * p->K;
-    if (rows * 64ull > 3ull * connections + 64ull * nslices || rows >= 0xffffffffull) return FFI_OK;   // too skewed
+    // too skewed, or beyond what the walking kernel's 32-bit buffer offsets reach (256 bytes per row)
+    if (rows * 64ull > 3ull * connections + 64ull * nslices || rows >= (1ull << 24)) return FFI_OK;
     if (!dev_alloc(&p->lab16, (size_t)rows * 64) || !dev_alloc(&p->pos16, (size_t)rows * 64)) return FFI_ERR_OUT_OF_MEMORY;
     hipLaunchKernelGGL(tile_fill_kernel, dim3(tiles), dim3(threads), 0, s, lookup, p->L, p->K, TL, p->slice_off, p->lab16,
                        p->pos16);
