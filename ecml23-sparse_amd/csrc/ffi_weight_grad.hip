@@ -28,15 +28,20 @@ constexpr int kResThreads = 512;
 constexpr int kResUnits = 4;        // units per thread
 
 // The eight 16-byte reads of one row, all issued before the first use ...
-__device__ __forceinline__ void wgrad_reads(const char* __restrict__ xs_bytes, unsigned base, float4 (&v)[8]) {
-    v[0] = *reinterpret_cast<const float4*>(xs_bytes + skew_addr<0>(base));
-    v[1] = *reinterpret_cast<const float4*>(xs_bytes + skew_addr<1>(base));
-    v[2] = *reinterpret_cast<const float4*>(xs_bytes + skew_addr<2>(base));
-    v[3] = *reinterpret_cast<const float4*>(xs_bytes + skew_addr<3>(base));
-    v[4] = *reinterpret_cast<const float4*>(xs_bytes + skew_addr<4>(base));
-    v[5] = *reinterpret_cast<const float4*>(xs_bytes + skew_addr<5>(base));
-    v[6] = *reinterpret_cast<const float4*>(xs_bytes + skew_addr<6>(base));
-    v[7] = *reinterpret_cast<const float4*>(xs_bytes + skew_addr<7>(base));
+// `base` = LDS address of the row + (lane & 7) * 16 (rows are 128-byte aligned, so the chunk bits can
+// be flipped with XOR).
+typedef float lds_v4f __attribute__((ext_vector_type(4)));
+typedef const lds_v4f __attribute__((address_space(3)))* lds_v4f_ptr;
+template <int C>
+__device__ __forceinline__ float4 wgrad_read_chunk(unsigned base) {
+    const lds_v4f t = *(lds_v4f_ptr)(size_t)(skew_addr<C>(base));
+    return make_float4(t.x, t.y, t.z, t.w);
+}
+__device__ __forceinline__ void wgrad_reads(unsigned base, float4 (&v)[8]) {
+    v[0] = wgrad_read_chunk<0>(base); v[1] = wgrad_read_chunk<1>(base);
+    v[2] = wgrad_read_chunk<2>(base); v[3] = wgrad_read_chunk<3>(base);
+    v[4] = wgrad_read_chunk<4>(base); v[5] = wgrad_read_chunk<5>(base);
+    v[6] = wgrad_read_chunk<6>(base); v[7] = wgrad_read_chunk<7>(base);
 }
 // ... and their dot product with the (equally skewed) out_grad values.
 __device__ __forceinline__ float wgrad_dot(const float4 (&v)[8], const float (&gb)[32], float acc) {
@@ -59,7 +64,6 @@ __global__ __launch_bounds__(kResThreads) void wgrad_resident_kernel(const float
                                                                      int L, int K, int nchunks, int n1, int upb1,
                                                                      int upb2) {
     extern __shared__ __align__(16) float xs[];
-    const char* xs_bytes = reinterpret_cast<const char*>(xs);
     const int lane = threadIdx.x & 63;
     const int blk = blockIdx.x;
     const long long total_units = (long long)L * nchunks;
@@ -81,7 +85,8 @@ __global__ __launch_bounds__(kResThreads) void wgrad_resident_kernel(const float
         __syncthreads();                                   // everyone is done with the previous tile
         stage_rows32<kResThreads, 8>(xs, xT, N, B, b0);
         __syncthreads();
-        unsigned skew = (unsigned)(lane & 7) * 16u;
+        // LDS address of xs plus the lane's skew
+        unsigned skew = (unsigned)(size_t)(__attribute__((address_space(3))) float*)xs + (unsigned)(lane & 7) * 16u;
         asm volatile("" : "+v"(skew));                     // keep the LDS addresses out of loop-invariant hoisting
 #pragma unroll
         for (int q = 0; q < kResUnits; ++q) {
@@ -122,7 +127,7 @@ __global__ __launch_bounds__(kResThreads) void wgrad_resident_kernel(const float
                 for (int k = 0; k < kWgChunk; ++k) {
                     const unsigned id = (k & 1) ? (idp[k >> 1] >> 16) : (idp[k >> 1] & 0xffffu);
                     float4 xv[8];
-                    wgrad_reads(xs_bytes, (id << 7) | skew, xv);
+                    wgrad_reads((id << 7) + skew, xv);
                     __builtin_amdgcn_sched_barrier(0);
                     res[q][k] = wgrad_dot(xv, gb, res[q][k]);
                     __builtin_amdgcn_sched_barrier(0);
@@ -171,7 +176,6 @@ __global__ __launch_bounds__(kResThreads) void wgrad_arranged_kernel(const float
                                                                      int L, int K, int nchunks, int n1, int upb1,
                                                                      int upb2) {
     extern __shared__ __align__(16) float xs[];
-    const char* xs_bytes = reinterpret_cast<const char*>(xs);
     const int lane = threadIdx.x & 63;
     const int blk = blockIdx.x;
     const long long total_units = (long long)L * nchunks;
@@ -193,7 +197,8 @@ __global__ __launch_bounds__(kResThreads) void wgrad_arranged_kernel(const float
         __syncthreads();                                   // everyone is done with the previous tile
         stage_rows32<kResThreads, 8>(xs, xT, N, B, b0);
         __syncthreads();
-        unsigned skew = (unsigned)(lane & 7) * 16u;
+        // LDS address of xs plus the lane's skew
+        unsigned skew = (unsigned)(size_t)(__attribute__((address_space(3))) float*)xs + (unsigned)(lane & 7) * 16u;
         asm volatile("" : "+v"(skew));                     // keep the LDS addresses out of loop-invariant hoisting
 #pragma unroll
         for (int q = 0; q < kResUnits; ++q) {
@@ -221,7 +226,7 @@ __global__ __launch_bounds__(kResThreads) void wgrad_arranged_kernel(const float
                 for (int k = 0; k < kWgChunk; ++k) {
                     const unsigned e = (k & 1) ? (idp[k >> 1] >> 16) : idp[k >> 1];
                     float4 xv[8];
-                    wgrad_reads(xs_bytes, ((e & kArrIdMask) << 7) | skew, xv);
+                    wgrad_reads(((e & kArrIdMask) << 7) + skew, xv);
                     __builtin_amdgcn_sched_barrier(0);
                     res[q][k] = wgrad_dot(xv, gb, res[q][k]);
                     __builtin_amdgcn_sched_barrier(0);
