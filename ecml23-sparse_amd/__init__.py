@@ -26,7 +26,13 @@ from .fixed_fan_in_ops import (  # noqa: E402
     fan_in_sparse_matmul_tp_bias,
     arrange_connections,
 )
-from . import custom_layer  # noqa: E402
+from . import custom_layer, metrics  # noqa: E402
+from .metrics import (  # noqa: E402
+    SparseHingeLoss,
+    SparseSquaredHingeLoss,
+    SparseBinaryCrossEntropyLoss,
+    PrecisionAtK,
+)
 from .custom_layer import StratifiedRewireLayerV2, FixedFractionSelector, FixedMagnitudeSelector  # noqa: E402
 
 __all__ = [
@@ -45,4 +51,8 @@ __all__ = [
     "StratifiedRewireLayerV2",
     "FixedFractionSelector",
     "FixedMagnitudeSelector",
+    "SparseHingeLoss",
+    "SparseSquaredHingeLoss",
+    "SparseBinaryCrossEntropyLoss",
+    "PrecisionAtK",
 ]

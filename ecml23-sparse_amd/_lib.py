@@ -10,6 +10,7 @@ LIB_PATH = os.path.join(_HERE, "libffi_hip.so")
 _vp = ctypes.c_void_p
 _i64 = ctypes.c_int64
 _int = ctypes.c_int
+_f32 = ctypes.c_float
 
 # name -> (restype, argtypes); the single source of truth for the Python side of the ABI
 SIGNATURES = {
@@ -35,6 +36,8 @@ SIGNATURES = {
     "ffi_forward_bf16_f32": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "ffi_forward_topk_bf16": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "ffi_topk_f32": (_int, [_vp, _i64, _i64, _int, _vp, _vp, _vp]),
+    "ffi_loss_grad_f32": (_int, [_vp, _vp, _vp, _i64, _int, _f32, _vp, _vp, _i64, _i64, _vp]),
+    "ffi_forward_loss_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _int, _f32, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
 }
 
 _lib = None

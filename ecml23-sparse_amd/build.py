@@ -26,6 +26,7 @@ SOURCES = [
     "ffi_util.hip",
     "ffi_wide.hip",
     "ffi_bf16.hip",
+    "ffi_loss.hip",
 ]
 
 # gfx950 only.  Packed-fp32 VALU forms are switched off for all device code.

@@ -237,6 +237,38 @@ int ffi_topk_f32(const float* scores, int64_t batch, int64_t num_units, int k, f
     return launch_topk_f32(scores, (int)batch, (int)num_units, k, topk_values, topk_indices, (hipStream_t)stream);
 }
 
+static int check_loss_args(const int64_t* label_indices, int64_t nnz, int loss_kind, int64_t batch, int64_t num_units) {
+    if (nnz < 0) return FFI_ERR_BAD_SHAPE;
+    if (nnz > 0 && !label_indices) return FFI_ERR_NULL_POINTER;
+    if (nnz >= INT32_MAX) return FFI_ERR_TOO_LARGE;
+    if (loss_kind != FFI_LOSS_HINGE && loss_kind != FFI_LOSS_SQUARED_HINGE && loss_kind != FFI_LOSS_BCE) return FFI_ERR_BAD_ARGUMENT;
+    if (batch <= 0 || num_units <= 0) return FFI_ERR_BAD_SHAPE;
+    if (batch >= INT32_MAX || num_units >= INT32_MAX) return FFI_ERR_TOO_LARGE;
+    return FFI_OK;
+}
+
+int ffi_loss_grad_f32(const float* scores, const int64_t* label_indices, const float* label_values, int64_t nnz,
+                      int loss_kind, float grad_scale, float* out_grad, float* loss_sum, int64_t batch, int64_t num_units,
+                      ffi_stream_t stream) {
+    if (!scores || !out_grad) return FFI_ERR_NULL_POINTER;
+    FFI_TRY(check_loss_args(label_indices, nnz, loss_kind, batch, num_units));
+    const LossArgs la{label_indices, label_values, (int)nnz, loss_kind, grad_scale, loss_sum};
+    return launch_loss_grad(la, scores, out_grad, (int)batch, (int)num_units, (hipStream_t)stream);
+}
+
+int ffi_forward_loss_f32(const float* features, const int32_t* lookup, const float* weights, const float* bias,
+                         const int64_t* label_indices, const float* label_values, int64_t nnz, int loss_kind,
+                         float grad_scale, float* scores, float* out_grad, float* loss_sum, int64_t batch,
+                         int64_t num_features, int64_t num_units, int64_t fan_in, int transposed, ffi_stream_t stream) {
+    if (!features || !lookup || !weights || !out_grad) return FFI_ERR_NULL_POINTER;
+    if (scores == out_grad) return FFI_ERR_BAD_ARGUMENT;
+    Dims d;
+    FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
+    FFI_TRY(check_loss_args(label_indices, nnz, loss_kind, batch, num_units));
+    const LossArgs la{label_indices, label_values, (int)nnz, loss_kind, grad_scale, loss_sum};
+    return launch_forward_loss(features, lookup, weights, bias, la, scores, out_grad, d, (hipStream_t)stream);
+}
+
 int ffi_plan_create(const int32_t* lookup, int64_t num_units, int64_t fan_in, int64_t num_features,
                     int64_t batch_hint, ffi_stream_t stream, ffi_plan** plan) {
     if (!lookup || !plan) return FFI_ERR_NULL_POINTER;

@@ -9,6 +9,7 @@
 // Other shapes go to the wide-input kernel (ffi_wide.hip).
 #include "ffi_internal.h"
 #include "ffi_lds_tile.h"
+#include "ffi_loss.h"
 
 #include <algorithm>
 
@@ -32,13 +33,28 @@ __device__ __forceinline__ void fwd_lane_step(const char* __restrict__ xs_bytes,
     acc[4 * C + 3] = fmaf(wv, v.w, acc[4 * C + 3]);
 }
 
-template <bool VEC4>
+// What the kernel does with a finished score s (after the bias):
+//   kEpiScores       out = s
+//   kEpiLossGrad     out = scale * dloss(s, 0)/ds, the loss gradient of a position that is not a listed label
+//                    (listed positions are patched afterwards), and the loss(s, 0) summed per wavefront
+//   kEpiLossGradAndScores  both: scores to `out`, gradients to `gout`
+enum FwdEpilogue { kEpiScores = 0, kEpiLossGrad = 1, kEpiLossGradAndScores = 2 };
+
+struct FwdLoss {
+    float* gout;        // [B,L] gradients (kEpiLossGradAndScores), else unused
+    double* partial;    // [gridDim.x * wavefronts per workgroup] loss sums
+    float scale;
+    int kind;
+};
+
+template <bool VEC4, int EPI>
 __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* __restrict__ xT,
                                                                   const int32_t* __restrict__ idx,
                                                                   const float* __restrict__ w,
                                                                   const float* __restrict__ bias,
                                                                   float* __restrict__ out, int B, int N,
-                                                                  int L, int K, int nbt, int labels_per_stream) {
+                                                                  int L, int K, int nbt, int labels_per_stream,
+                                                                  FwdLoss fl) {
     extern __shared__ __align__(16) float xs[];
     const char* xs_bytes = reinterpret_cast<const char*>(xs);
     const int u = xcd_contiguous_block(blockIdx.x, gridDim.x);
@@ -55,6 +71,9 @@ __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* _
     const int nrows = min(kTileBatch, B - b0);
     float* obase = out + (size_t)b0 * (size_t)L;
     const buffer_rsrc orsrc = make_rsrc(obase, (size_t)nrows * (size_t)L * sizeof(float));
+    buffer_rsrc grsrc = orsrc;
+    if (EPI == kEpiLossGradAndScores) grsrc = make_rsrc(fl.gout + (size_t)b0 * (size_t)L, (size_t)nrows * (size_t)L * sizeof(float));
+    float lsum = 0.f;
 
     for (int base = l_begin; base < l_end; base += kTileThreads) {
         if (base + (int)(threadIdx.x & ~63u) >= l_end) break;     // nothing left for this wavefront
@@ -109,14 +128,90 @@ __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* _
 #pragma unroll
             for (int i = 0; i < 32; ++i) acc[i] += bj;
         }
-        if (valid) {
-            const unsigned lane_off = (unsigned)j * 4u;
-            const unsigned stride = (unsigned)L * 4u;
+        const unsigned lane_off = (unsigned)j * 4u;
+        const unsigned stride = (unsigned)L * 4u;
+        if (EPI != kEpiLossGrad && valid) {
 #pragma unroll
             for (int b = 0; b < 32; ++b)
                 __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, acc[b]), orsrc, lane_off, (unsigned)b * stride, 0);
         }
+        if (EPI != kEpiScores) {
+            float l = 0.f;
+#pragma unroll
+            for (int b = 0; b < 32; ++b) {
+                float lb, gb;
+                cwise_loss_and_grad(fl.kind, acc[b], 0.f, lb, gb);
+                l += b < nrows ? lb : 0.f;
+                acc[b] = fl.scale * gb;
+            }
+            if (valid) {
+                lsum += l;
+#pragma unroll
+                for (int b = 0; b < 32; ++b)
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, acc[b]), EPI == kEpiLossGrad ? orsrc : grsrc, lane_off, (unsigned)b * stride, 0);
+            }
+        }
     }
+    if (EPI != kEpiScores) {
+        const double t = wave_sum((double)lsum);
+        if (lane == 0) fl.partial[(size_t)blockIdx.x * (kTileThreads / 64) + (threadIdx.x >> 6)] = t;
+    }
+}
+
+}  // namespace
+
+namespace {
+
+template <bool VEC4, int EPI>
+int launch_lane32(const float* xT, const int32_t* idx, const float* w, const float* bias, float* out, const Dims& d, int nbt,
+                  int per_stream, int blocks, size_t lds, const FwdLoss& fl, hipStream_t s) {
+    FFI_HIP_TRY(hipFuncSetAttribute((const void*)fwd_lane32_kernel<VEC4, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL((fwd_lane32_kernel<VEC4, EPI>), dim3(blocks), dim3(kTileThreads), lds, s, xT, idx, w, bias, out, d.B, d.N,
+                       d.L, d.K, nbt, per_stream, fl);
+    FFI_HIP_TRY(hipGetLastError());
+    return FFI_OK;
+}
+
+// Narrow-input forward pass with the given epilogue; `la` is needed for the loss epilogues only.
+int forward_tiles(const float* x, const int32_t* idx, const float* w, const float* bias, float* out, float* gout, int epi,
+                  const LossArgs* la, const Dims& d, hipStream_t s) {
+    const float* xT = x;
+    if (!d.tp) {
+        float* ws = nullptr;
+        FFI_TRY(workspace_get(s, kWsFeaturesT, (size_t)d.N * d.B * sizeof(float), (void**)&ws));
+        FFI_TRY(launch_transpose(x, ws, d.B, d.N, s));   // [B,N] -> [N,B]
+        xT = ws;
+    }
+    const size_t lds = tile_lds_bytes(d.N);
+    const bool vec4 = (d.K % 4 == 0) && (((uintptr_t)w | (uintptr_t)idx) % 16 == 0);
+    const int cus = device_cu_count();
+    const int nbt = (d.B + kTileBatch - 1) / kTileBatch;
+    int streams = std::max(1, cus / nbt);
+    const int per_stream = (d.L + streams - 1) / streams;
+    streams = (d.L + per_stream - 1) / per_stream;
+    const int blocks = streams * nbt;
+    FwdLoss fl{gout, nullptr, 0.f, 0};
+    if (epi == kEpiScores)
+        return vec4 ? launch_lane32<true, kEpiScores>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, s)
+                    : launch_lane32<false, kEpiScores>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, s);
+    const int npartial = blocks * (kTileThreads / 64);
+    double* corr = nullptr;
+    FFI_TRY(loss_partial_buffer(s, npartial, la->nnz, &fl.partial, &corr, nullptr));
+    fl.scale = la->scale;
+    fl.kind = la->kind;
+    if (epi == kEpiLossGrad) {
+        FFI_TRY(vec4 ? (launch_lane32<true, kEpiLossGrad>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, s))
+                     : (launch_lane32<false, kEpiLossGrad>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, s)));
+    } else {
+        FFI_TRY(vec4 ? (launch_lane32<true, kEpiLossGradAndScores>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, s))
+                     : (launch_lane32<false, kEpiLossGradAndScores>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, s)));
+    }
+    // the listed label positions: from the score matrix when it was written, else recomputed from x ([N,B] here)
+    Dims dt = d;
+    dt.tp = true;
+    float* g = epi == kEpiLossGrad ? out : gout;
+    return launch_loss_positives(*la, nullptr, epi == kEpiLossGrad ? nullptr : out, xT, idx, w, bias, g, dt, fl.partial, npartial,
+                                 corr, s);
 }
 
 }  // namespace
@@ -124,33 +219,21 @@ __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* _
 int launch_forward(const float* x, const int32_t* idx, const float* w, const float* bias, float* out, const Dims& d,
                    hipStream_t s) {
     // (the kernel reaches the 32 rows of out of a batch tile through 32-bit byte offsets)
-    if (tile_path_fits(d.N) && d.L < (1 << 25)) {
-        const float* xT = x;
-        if (!d.tp) {
-            float* ws = nullptr;
-            FFI_TRY(workspace_get(s, kWsFeaturesT, (size_t)d.N * d.B * sizeof(float), (void**)&ws));
-            FFI_TRY(launch_transpose(x, ws, d.B, d.N, s));   // [B,N] -> [N,B]
-            xT = ws;
-        }
-        const size_t lds = tile_lds_bytes(d.N);
-        const bool vec4 = (d.K % 4 == 0) && (((uintptr_t)w | (uintptr_t)idx) % 16 == 0);
-        const int cus = device_cu_count();
-        const int nbt = (d.B + kTileBatch - 1) / kTileBatch;
-        int streams = std::max(1, cus / nbt);
-        const int per_stream = (d.L + streams - 1) / streams;
-        streams = (d.L + per_stream - 1) / per_stream;
-        const int blocks = streams * nbt;
-        if (vec4) {
-            FFI_HIP_TRY(hipFuncSetAttribute((const void*)fwd_lane32_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-            hipLaunchKernelGGL(fwd_lane32_kernel<true>, dim3(blocks), dim3(kTileThreads), lds, s, xT, idx, w, bias, out, d.B, d.N, d.L, d.K, nbt, per_stream);
-        } else {
-            FFI_HIP_TRY(hipFuncSetAttribute((const void*)fwd_lane32_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-            hipLaunchKernelGGL(fwd_lane32_kernel<false>, dim3(blocks), dim3(kTileThreads), lds, s, xT, idx, w, bias, out, d.B, d.N, d.L, d.K, nbt, per_stream);
-        }
-        FFI_HIP_TRY(hipGetLastError());
-        return FFI_OK;
-    }
+    if (tile_path_fits(d.N) && d.L < (1 << 25)) return forward_tiles(x, idx, w, bias, out, nullptr, kEpiScores, nullptr, d, s);
     return launch_forward_wide(x, idx, w, bias, out, d, s);
+}
+
+int launch_forward_loss(const float* x, const int32_t* idx, const float* w, const float* bias, const LossArgs& la,
+                        float* scores, float* g, const Dims& d, hipStream_t s) {
+    if (tile_path_fits(d.N) && d.L < (1 << 25)) {
+        if (scores == nullptr) return forward_tiles(x, idx, w, bias, g, nullptr, kEpiLossGrad, &la, d, s);
+        return forward_tiles(x, idx, w, bias, scores, g, kEpiLossGradAndScores, &la, d, s);
+    }
+    // wide inputs: scores by the wide kernel (into g itself when the caller wants no scores), then the
+    // loss gradient as a pass of its own
+    float* sc = scores ? scores : g;
+    FFI_TRY(launch_forward_wide(x, idx, w, bias, sc, d, s));
+    return launch_loss_grad(la, sc, g, d.B, d.L, s);
 }
 
 }  // namespace ffi

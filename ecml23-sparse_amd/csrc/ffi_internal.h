@@ -38,7 +38,7 @@ int hip_fail(hipError_t e);
 
 // Library-owned device scratch, one buffer per (device, stream, slot), grown on demand and kept.
 // Work that uses a buffer is ordered by the stream it belongs to.
-enum WorkspaceSlot { kWsFeaturesT = 0, kWsPartials = 1, kWsSlots = 2 };
+enum WorkspaceSlot { kWsFeaturesT = 0, kWsPartials = 1, kWsSlots = 2, kWsLoss = 3 };
 int workspace_get(hipStream_t s, int slot, size_t bytes, void** out);
 void workspace_clear(int device);
 size_t workspace_bytes(int device);
@@ -66,6 +66,29 @@ int launch_forward_wide(const float* x, const int32_t* idx, const float* w, cons
                         hipStream_t s);
 int launch_weight_grad_wide(const float* x, const int32_t* idx, const float* g, float* gw, float* bias_grad, const Dims& d,
                             hipStream_t s);
+
+
+// ---- loss gradient (ffi_loss.hip) ---------------------------------------------------------------
+struct LossArgs {
+    const int64_t* indices;   // [nnz,2] (row, column) of the listed label positions
+    const float* values;      // [nnz] or null (all 1)
+    int nnz;
+    int kind;                 // ffi_loss_kind
+    float scale;              // factor on the gradient
+    float* loss_sum;          // device float or null
+};
+// partial[npartial] loss sums, corr[nnz] loss corrections and saved[nnz] scores of the listed positions
+int loss_partial_buffer(hipStream_t s, int npartial, int nnz, double** partial, double** corr, float** saved);
+// g at the listed positions, loss corrections, final loss sum; the score of a listed position comes from
+// saved[p], else scores[b,j], else from its row of idx / w (+ bias) and x
+int launch_loss_positives(const LossArgs& la, const float* saved, const float* scores, const float* x, const int32_t* idx,
+                          const float* w, const float* bias, float* g, const Dims& d, const double* partial, int npartial,
+                          double* corr, hipStream_t s);
+// g = scale * dloss/dscore for a whole score matrix (g may be the score buffer itself)
+int launch_loss_grad(const LossArgs& la, const float* scores, float* g, int B, int L, hipStream_t s);
+// forward pass whose epilogue turns the scores into loss gradients (scores may be null)
+int launch_forward_loss(const float* x, const int32_t* idx, const float* w, const float* bias, const LossArgs& la,
+                        float* scores, float* g, const Dims& d, hipStream_t s);
 
 }  // namespace ffi
 

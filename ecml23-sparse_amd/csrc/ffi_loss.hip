@@ -1,0 +1,171 @@
+// Loss gradient with respect to the scores of the layer: the producer of out_grad
+// (SparseLossBase.call, sparse/metrics.py:136-139, over dense_sparse_cwise_op, sparse/utils.py:11-17).
+//
+//   loss_dense_kernel      every (b,j) as a negative: g = scale * dloss(s, 0), loss partial sums
+//   loss_gather_kernel     saves the scores of the listed label positions (needed when out_grad
+//                          overwrites the scores in place)
+//   loss_positive_kernel   the listed label positions: g and the loss correction loss(s,y) - loss(s,0);
+//                          takes s from the saved scores or the score matrix, or recomputes it from the
+//                          label's row of lookup / weights when the scores were never written
+//   loss_finish_kernel     sums the partial sums and the corrections in a fixed order
+#include "ffi_internal.h"
+#include "ffi_loss.h"
+
+#include <algorithm>
+
+namespace ffi {
+namespace {
+
+constexpr int kLossThreads = 256;
+constexpr int kLossVecPerThread = 4;    // float4 loads in flight per thread and round
+
+__global__ __launch_bounds__(kLossThreads) void loss_dense_kernel(const float* scores, float* g, size_t total, float scale,
+                                                                  int kind, double* __restrict__ partial) {
+    // `scores` and `g` may be the same buffer: every element is read before it is written, by the same thread
+    const size_t nvec = total / 4;
+    const size_t stride = (size_t)gridDim.x * kLossThreads;
+    float lsum = 0.f;
+    for (size_t v0 = (size_t)blockIdx.x * kLossThreads + threadIdx.x; v0 < nvec; v0 += stride * kLossVecPerThread) {
+        float4 s[kLossVecPerThread];
+#pragma unroll
+        for (int i = 0; i < kLossVecPerThread; ++i) {
+            const size_t v = v0 + (size_t)i * stride;
+            s[i] = v < nvec ? reinterpret_cast<const float4*>(scores)[v] : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int i = 0; i < kLossVecPerThread; ++i) {
+            const size_t v = v0 + (size_t)i * stride;
+            if (v < nvec) {
+                float4 l, o;
+                cwise_loss_and_grad(kind, s[i].x, 0.f, l.x, o.x);
+                cwise_loss_and_grad(kind, s[i].y, 0.f, l.y, o.y);
+                cwise_loss_and_grad(kind, s[i].z, 0.f, l.z, o.z);
+                cwise_loss_and_grad(kind, s[i].w, 0.f, l.w, o.w);
+                lsum += (l.x + l.y) + (l.z + l.w);
+                o.x *= scale; o.y *= scale; o.z *= scale; o.w *= scale;
+                reinterpret_cast<float4*>(g)[v] = o;
+            }
+        }
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (total & 3)) {       // the last 1..3 elements
+        const size_t e = nvec * 4 + threadIdx.x;
+        const float sv = scores[e];
+        lsum += cwise_loss(kind, sv, 0.f);
+        g[e] = scale * cwise_loss_grad(kind, sv, 0.f);
+    }
+    const double w = wave_sum((double)lsum);
+    if ((threadIdx.x & 63) == 0) partial[blockIdx.x * (kLossThreads / 64) + (threadIdx.x >> 6)] = w;
+}
+
+__global__ __launch_bounds__(kLossThreads) void loss_gather_kernel(const int64_t* __restrict__ label_indices, int nnz,
+                                                                   const float* __restrict__ scores, int B, int L,
+                                                                   float* __restrict__ saved) {
+    const int p = blockIdx.x * kLossThreads + threadIdx.x;
+    if (p >= nnz) return;
+    const int64_t b = label_indices[2 * (size_t)p], j = label_indices[2 * (size_t)p + 1];
+    saved[p] = (b >= 0 && b < B && j >= 0 && j < L) ? scores[(size_t)b * L + j] : 0.f;
+}
+
+// One thread per listed label position.  x is addressed as x[b * xsb + n * xsn] (either layout).
+__global__ __launch_bounds__(kLossThreads) void loss_positive_kernel(
+    const int64_t* __restrict__ label_indices, const float* __restrict__ label_values, int nnz,
+    const float* __restrict__ saved, const float* __restrict__ scores, const float* __restrict__ x, size_t xsb, size_t xsn,
+    const int32_t* __restrict__ idx, const float* __restrict__ w, const float* __restrict__ bias, float* __restrict__ g,
+    float scale, int kind, int B, int N, int L, int K, double* __restrict__ corr) {
+    const int p = blockIdx.x * kLossThreads + threadIdx.x;
+    if (p >= nnz) return;
+    const int64_t b = label_indices[2 * (size_t)p], j = label_indices[2 * (size_t)p + 1];
+    double c = 0.0;
+    if (b >= 0 && b < B && j >= 0 && j < L) {
+        float s;
+        if (saved != nullptr) {
+            s = saved[p];
+        } else if (scores != nullptr) {
+            s = scores[(size_t)b * L + j];
+        } else {
+            // the same sum the forward kernel forms: ascending k, fused multiply-adds, bias last
+            s = 0.f;
+            for (int k = 0; k < K; ++k) {
+                const unsigned id = (unsigned)idx[(size_t)j * K + k];
+                s = fmaf(w[(size_t)j * K + k], x[(size_t)b * xsb + (size_t)(id < (unsigned)N ? id : 0u) * xsn], s);
+            }
+            if (bias != nullptr) s += bias[j];
+        }
+        const float y = label_values ? label_values[p] : 1.f;
+        g[(size_t)b * L + j] = scale * cwise_loss_grad(kind, s, y);
+        // minus what the bulk pass charged this position as a negative (the same arithmetic as there)
+        float l0, g0;
+        cwise_loss_and_grad<false>(kind, s, 0.f, l0, g0);
+        c = (double)cwise_loss(kind, s, y) - (double)l0;
+    }
+    corr[p] = c;
+}
+
+__global__ __launch_bounds__(kLossThreads) void loss_finish_kernel(const double* __restrict__ partial, int npartial,
+                                                                   const double* __restrict__ corr, int ncorr,
+                                                                   float* __restrict__ loss_sum) {
+    __shared__ double red[kLossThreads / 64];
+    double a = 0.0;
+    for (int i = threadIdx.x; i < npartial; i += kLossThreads) a += partial[i];
+    for (int i = threadIdx.x; i < ncorr; i += kLossThreads) a += corr[i];
+    a = wave_sum(a);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = a;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double t = 0.0;
+        for (int i = 0; i < kLossThreads / 64; ++i) t += red[i];
+        *loss_sum = (float)t;
+    }
+}
+
+}  // namespace
+
+int loss_partial_buffer(hipStream_t s, int npartial, int nnz, double** partial, double** corr, float** saved) {
+    double* buf = nullptr;
+    FFI_TRY(workspace_get(s, kWsLoss, ((size_t)npartial + 2 * (size_t)nnz + 2) * sizeof(double), (void**)&buf));
+    *partial = buf;
+    *corr = buf + npartial;
+    if (saved) *saved = reinterpret_cast<float*>(buf + npartial + nnz);
+    return FFI_OK;
+}
+
+int launch_loss_positives(const LossArgs& la, const float* saved, const float* scores, const float* x, const int32_t* idx, const float* w,
+                          const float* bias, float* g, const Dims& d, const double* partial, int npartial, double* corr,
+                          hipStream_t s) {
+    if (la.nnz > 0) {
+        const size_t xsb = d.tp ? 1 : (size_t)d.N, xsn = d.tp ? (size_t)d.B : 1;
+        hipLaunchKernelGGL(loss_positive_kernel, dim3((la.nnz + kLossThreads - 1) / kLossThreads), dim3(kLossThreads), 0, s,
+                           la.indices, la.values, la.nnz, saved, scores, x, xsb, xsn, idx, w, bias, g, la.scale, la.kind, d.B, d.N,
+                           d.L, d.K, corr);
+        FFI_HIP_TRY(hipGetLastError());
+    }
+    if (la.loss_sum != nullptr) {
+        hipLaunchKernelGGL(loss_finish_kernel, dim3(1), dim3(kLossThreads), 0, s, partial, npartial, corr, la.nnz, la.loss_sum);
+        FFI_HIP_TRY(hipGetLastError());
+    }
+    return FFI_OK;
+}
+
+int launch_loss_grad(const LossArgs& la, const float* scores, float* g, int B, int L, hipStream_t s) {
+    const size_t total = (size_t)B * (size_t)L;
+    const size_t nvec = total / 4;
+    const size_t per_block = (size_t)kLossThreads * kLossVecPerThread;
+    const int blocks = (int)std::max<size_t>(1, std::min<size_t>((nvec + per_block - 1) / per_block, (size_t)device_cu_count() * 16));
+    const int npartial = blocks * (kLossThreads / 64);
+    double *partial = nullptr, *corr = nullptr;
+    float* saved = nullptr;
+    FFI_TRY(loss_partial_buffer(s, npartial, la.nnz, &partial, &corr, &saved));
+    // when g overwrites the scores in place, the scores of the listed positions are put aside first
+    const bool in_place = scores == g;
+    if (in_place && la.nnz > 0) {
+        hipLaunchKernelGGL(loss_gather_kernel, dim3((la.nnz + kLossThreads - 1) / kLossThreads), dim3(kLossThreads), 0, s,
+                           la.indices, la.nnz, scores, B, L, saved);
+        FFI_HIP_TRY(hipGetLastError());
+    }
+    hipLaunchKernelGGL(loss_dense_kernel, dim3(blocks), dim3(kLossThreads), 0, s, scores, g, total, la.scale, la.kind, partial);
+    FFI_HIP_TRY(hipGetLastError());
+    Dims d{B, 1, L, 1, false};
+    return launch_loss_positives(la, in_place ? saved : nullptr, scores, nullptr, nullptr, nullptr, nullptr, g, d, partial, npartial, corr, s);
+}
+
+}  // namespace ffi

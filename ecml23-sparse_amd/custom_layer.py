@@ -117,6 +117,16 @@ class StratifiedRewireLayerV2(torch.nn.Module):
         weights = self.kernel_weights.view(-1, self.fan_in)
         return ops.fan_in_sparse_matmul_bias(inputs, indices, weights, self.bias)
 
+    def forward_loss(self, inputs: torch.Tensor, y_true, loss, want_scores: bool = False):
+        """``loss(y_true, self(inputs))`` with the loss gradient formed inside the forward kernel:
+        returns ``(loss value, scores or None)``; the score matrix is written only if asked for
+        (metrics).  ``loss`` is one of the objects of ``metrics`` (e.g. ``SparseSquaredHingeLoss``)."""
+        if inputs.dim() != 2 or inputs.shape[1] != self.input_dim:
+            raise ValueError(f"inputs must have shape [batch, {self.input_dim}], got {tuple(inputs.shape)}")
+        indices = self.kernel_indices.view(-1, self.fan_in)
+        weights = self.kernel_weights.view(-1, self.fan_in)
+        return loss.fused(inputs.float(), indices, weights, self.bias, y_true, transposed=False, want_scores=want_scores)
+
     # sparse/layer.py:215-219, 236-237 and sparse/custom_layer.py:20-43
     @torch.no_grad()
     def rewire(self, other_vars=None):

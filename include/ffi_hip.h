@@ -183,6 +183,42 @@ int ffi_forward_topk_bf16(const uint16_t* features, const int32_t* lookup, const
 int ffi_topk_f32(const float* scores, int64_t batch, int64_t num_units, int k,
                  float* topk_values, int32_t* topk_indices, ffi_stream_t stream);
 
+/*
+ * The loss the reference trains the layer with, and its gradient with respect to the scores: the
+ * producer of out_grad.  Restates SparseLossBase.call (sparse/metrics.py:136-139) on top of
+ * dense_sparse_cwise_op (sparse/utils.py:11-17): every (b,j) is charged loss(score, 0), except the
+ * positions listed in the sparse label matrix, which are charged loss(score, value).
+ *   label_indices  [nnz, 2] int64 (row, column) pairs, the layout of tf.sparse.SparseTensor.indices;
+ *   label_values   [nnz] float (NULL = all 1.0); nnz may be 0 (both may then be NULL).
+ * A position must not be listed twice (TensorFlow's scatter update leaves the outcome open as
+ * well); pairs outside [0,batch) x [0,num_units) are skipped, as TensorFlow's GPU gather does.
+ *   out_grad[b,j]  = grad_scale * d loss / d score  (Keras' mean over labels, then over the batch,
+ *                    is grad_scale = 1 / (batch * num_units)); may alias `scores`;
+ *   loss_sum       one float on the device: the un-scaled sum of the element losses; may be NULL.
+ * Sums are formed in a fixed order (no atomics).
+ */
+enum ffi_loss_kind {
+    FFI_LOSS_HINGE = 1,           /* SparseHingeLoss          sparse/metrics.py:147-154 */
+    FFI_LOSS_SQUARED_HINGE = 2,   /* SparseSquaredHingeLoss   sparse/metrics.py:157-164 */
+    FFI_LOSS_BCE = 3              /* SparseBinaryCrossEntropyLoss  sparse/metrics.py:167-173 */
+};
+int ffi_loss_grad_f32(const float* scores, const int64_t* label_indices, const float* label_values, int64_t nnz,
+                      int loss_kind, float grad_scale, float* out_grad, float* loss_sum,
+                      int64_t batch, int64_t num_units, ffi_stream_t stream);
+
+/*
+ * Forward pass, bias add and loss gradient in one pass (no counterpart in the reference, where they
+ * are three TensorFlow ops and the [batch, num_units] score matrix makes two more trips through
+ * memory): the forward kernel turns each finished score into its loss gradient before storing it.
+ * `bias` may be NULL; `scores` may be NULL when only the gradient and the loss are wanted (the
+ * scores of the listed label positions are then recomputed from their rows of lookup / weights).
+ */
+int ffi_forward_loss_f32(const float* features, const int32_t* lookup, const float* weights, const float* bias,
+                         const int64_t* label_indices, const float* label_values, int64_t nnz,
+                         int loss_kind, float grad_scale, float* scores, float* out_grad, float* loss_sum,
+                         int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in,
+                         int transposed, ffi_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

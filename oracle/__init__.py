@@ -204,3 +204,48 @@ def dense_backward(features, lookup, weights, out_grad, transposed=False):
     L, K = lookup.shape
     gw = dense_gw[lookup, np.arange(L)[:, None]]
     return gx, gw
+
+
+# ---- loss and its gradient with respect to the scores (numpy, float64 inside) --------------------
+LOSS_HINGE, LOSS_SQUARED_HINGE, LOSS_BCE = 1, 2, 3
+
+
+def cwise_loss(kind, score, y):
+    """Element loss, sparse/metrics.py:142-144 (hinge), :152-154, :162-164 (squared hinge), :172-173 (bce:
+    tf.nn.sigmoid_cross_entropy_with_logits = max(x,0) - x*z + log1p(exp(-|x|)))."""
+    score = np.asarray(score, dtype=np.float64)
+    y = np.asarray(y, dtype=np.float64)
+    if kind == LOSS_BCE:
+        return np.maximum(score, 0.0) - score * y + np.log1p(np.exp(-np.abs(score)))
+    r = np.maximum(1.0 - (2.0 * y - 1.0) * score, 0.0)
+    return r if kind == LOSS_HINGE else r * r
+
+
+def cwise_loss_grad(kind, score, y):
+    """d cwise_loss / d score; relu' is 0 at 0 (TensorFlow's ReluGrad passes the gradient where x > 0)."""
+    score = np.asarray(score, dtype=np.float64)
+    y = np.asarray(y, dtype=np.float64)
+    if kind == LOSS_BCE:
+        return 1.0 / (1.0 + np.exp(-score)) - y
+    sign = 2.0 * y - 1.0
+    r = np.maximum(1.0 - sign * score, 0.0)
+    if kind == LOSS_HINGE:
+        return np.where(r > 0.0, -sign, 0.0)
+    return -2.0 * sign * r
+
+
+def sparse_loss(scores, label_indices, label_values, kind):
+    """SparseLossBase.call (sparse/metrics.py:136-139) through dense_sparse_cwise_op (sparse/utils.py:11-17):
+    the dense part charges every entry loss(s, 0); the listed positions are overwritten with
+    loss(s, value).  Returns (element losses [B,L], d sum(losses) / d scores [B,L]) in float64;
+    the reference's per-sample value is ``losses.mean(axis=-1)``."""
+    s = np.asarray(scores, dtype=np.float64)
+    idx = np.asarray(label_indices, dtype=np.int64).reshape(-1, 2)
+    vals = np.ones(len(idx)) if label_values is None else np.asarray(label_values, dtype=np.float64)
+    losses = cwise_loss(kind, s, 0.0)
+    grad = cwise_loss_grad(kind, s, 0.0)
+    if len(idx):
+        b, j = idx[:, 0], idx[:, 1]
+        losses[b, j] = cwise_loss(kind, s[b, j], vals)
+        grad[b, j] = cwise_loss_grad(kind, s[b, j], vals)
+    return losses, grad

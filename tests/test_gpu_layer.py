@@ -232,3 +232,27 @@ def test_layer_keeps_connections_arranged(ffi):
     want_mom = torch.where(selected, torch.zeros_like(mom), mom).view(units, K).cpu().numpy()
     order_b, order_a = np.argsort(wb, 1, kind="stable"), np.argsort(wa, 1, kind="stable")
     np.testing.assert_array_equal(np.take_along_axis(want_mom, order_b, 1), np.take_along_axis(new_mom.view(units, K).cpu().numpy(), order_a, 1))
+
+
+def test_layer_forward_loss_matches_loss_of_forward(ffi):
+    # one fused call (scores never written) against loss(y, layer(x)), values and parameter gradients
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    layer = ffi.StratifiedRewireLayerV2(units=1500, input_dim=200, connections=1500 * 24, generator=gen)
+    with torch.no_grad():
+        layer.bias.fill_(-0.2)
+    x = torch.rand((48, 200), device="cuda", generator=gen)
+    rows = torch.arange(48, device="cuda").repeat_interleave(3)
+    cols = torch.randint(0, 1500, (48 * 3,), device="cuda", generator=gen)
+    y = (torch.stack([rows, cols], dim=1), None)
+    loss_fn = ffi.SparseSquaredHingeLoss()
+    plain = loss_fn(y, layer(x))
+    plain.backward()
+    gw0, gb0 = layer.kernel_weights.grad.clone(), layer.bias.grad.clone()
+    layer.zero_grad()
+    fused, scores = layer.forward_loss(x, y, loss_fn, want_scores=True)
+    fused.backward()
+    torch.cuda.synchronize()
+    assert abs(float(plain.detach()) - float(fused.detach())) <= 1e-5 * abs(float(plain.detach()))
+    assert rel_err(layer.kernel_weights.grad.cpu().numpy(), gw0.cpu().numpy()) <= GRAD_RTOL
+    assert rel_err(layer.bias.grad.cpu().numpy(), gb0.cpu().numpy()) <= GRAD_RTOL
+    assert rel_err(scores.cpu().numpy(), layer(x).detach().cpu().numpy()) <= FWD_RTOL

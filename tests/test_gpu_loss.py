@@ -1,0 +1,231 @@
+"""The producer of out_grad: losses on sparse label matrices (sparse/metrics.py:132-173) through the
+C ABI, alone (`ffi_loss_grad_f32`) and fused into the forward kernel (`ffi_forward_loss_f32`),
+against the numpy oracle (pinned in tests/test_oracle.py by known values, a dense autograd
+restatement and central differences).
+
+Gates: gradients and loss sums within 1e-5 of the largest reference magnitude; where the loss
+consumes scores computed on the GPU, the oracle is fed the oracle's own forward scores, and
+entries within 1e-5 of a kink of the hinge (margin exactly 1) are left out of the comparison.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from conftest import load_package, rel_err
+
+pytestmark = pytest.mark.gpu
+
+RTOL = 1e-5
+KINDS = [oracle.LOSS_HINGE, oracle.LOSS_SQUARED_HINGE, oracle.LOSS_BCE]
+
+
+@pytest.fixture(scope="module")
+def ffi():
+    pkg = load_package()
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    return pkg
+
+
+def label_list(rng, B, L, per_sample=5, values=True):
+    rows, cols = [], []
+    for b in range(B):
+        c = rng.choice(L, size=min(per_sample, L), replace=False)
+        rows += [b] * len(c)
+        cols += list(np.sort(c))
+    indices = np.stack([np.array(rows), np.array(cols)], axis=1).astype(np.int64)
+    vals = rng.choice([1.0, 1.0, 1.0, 0.5], size=len(rows)).astype(np.float32) if values else None
+    return indices, vals
+
+
+def away_from_kinks(scores, indices, values, kind, tol=1e-5):
+    """Mask of entries whose hinge margin is not within `tol` of 1 (where the hinge slope jumps)."""
+    if kind != oracle.LOSS_HINGE:
+        return np.ones(scores.shape, bool)
+    y = np.zeros(scores.shape)
+    if len(indices):
+        y[indices[:, 0], indices[:, 1]] = 1.0 if values is None else values
+    return np.abs(1.0 - (2.0 * y - 1.0) * scores) > tol
+
+
+def call_loss_grad(ffi, scores_t, indices, values, kind, scale, in_place=False):
+    lib = ffi._lib.lib()
+    B, L = scores_t.shape
+    idx_t = torch.from_numpy(indices).cuda() if len(indices) else None
+    val_t = torch.from_numpy(values).cuda() if values is not None and len(values) else None
+    g = scores_t if in_place else torch.full_like(scores_t, float("nan"))
+    loss = torch.full((1,), float("nan"), device="cuda")
+    ffi._lib.check(lib.ffi_loss_grad_f32(scores_t.data_ptr(), idx_t.data_ptr() if idx_t is not None else None,
+                                         val_t.data_ptr() if val_t is not None else None, len(indices), kind,
+                                         ctypes.c_float(scale), g.data_ptr(), loss.data_ptr(), B, L,
+                                         torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    return g.cpu().numpy(), float(loss.cpu()[0])
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("shape", [(128, 5000), (37, 1001), (3, 7), (1, 1), (64, 4099)])
+def test_loss_grad_against_oracle(ffi, kind, shape):
+    B, L = shape
+    rng = np.random.default_rng(B * 131 + L + kind)
+    scores = rng.normal(-0.5, 1.5, (B, L)).astype(np.float32)
+    indices, values = label_list(rng, B, L, per_sample=min(5, L))
+    scale = 1.0 / (B * L)
+    losses, grad = oracle.sparse_loss(scores, indices, values, kind)
+    g, loss_sum = call_loss_grad(ffi, torch.from_numpy(scores).cuda(), indices, values, kind, scale)
+    ok = away_from_kinks(scores, indices, values, kind)
+    assert rel_err(np.where(ok, g, 0), np.where(ok, grad * scale, 0)) <= RTOL
+    assert abs(loss_sum - losses.sum()) <= RTOL * abs(losses.sum())
+
+
+@pytest.mark.parametrize("kind", KINDS)
+def test_loss_grad_in_place_and_default_values(ffi, kind):
+    # out_grad may be the score buffer itself; label_values NULL means all ones
+    B, L = 33, 777
+    rng = np.random.default_rng(kind)
+    scores = rng.normal(0, 1, (B, L)).astype(np.float32)
+    indices, _ = label_list(rng, B, L, values=False)
+    losses, grad = oracle.sparse_loss(scores, indices, None, kind)
+    g, loss_sum = call_loss_grad(ffi, torch.from_numpy(scores).cuda(), indices, None, kind, 0.25, in_place=True)
+    ok = away_from_kinks(scores, indices, None, kind)
+    assert rel_err(np.where(ok, g, 0), np.where(ok, grad * 0.25, 0)) <= RTOL
+    assert abs(loss_sum - losses.sum()) <= RTOL * abs(losses.sum())
+
+
+def test_loss_grad_no_labels_and_skipped_pairs(ffi):
+    # nnz = 0 (NULL lists); pairs outside the matrix are skipped and change nothing
+    B, L = 16, 300
+    rng = np.random.default_rng(9)
+    scores = rng.normal(0, 1, (B, L)).astype(np.float32)
+    empty = np.zeros((0, 2), np.int64)
+    losses, grad = oracle.sparse_loss(scores, empty, None, oracle.LOSS_SQUARED_HINGE)
+    g, loss_sum = call_loss_grad(ffi, torch.from_numpy(scores).cuda(), empty, None, oracle.LOSS_SQUARED_HINGE, 1.0)
+    assert rel_err(g, grad) <= RTOL and abs(loss_sum - losses.sum()) <= RTOL * losses.sum()
+    good = np.array([[2, 5], [7, 299]], np.int64)
+    bad = np.array([[B, 0], [0, L], [-1, 3], [3, -1]], np.int64)
+    losses, grad = oracle.sparse_loss(scores, good, None, oracle.LOSS_SQUARED_HINGE)
+    g, loss_sum = call_loss_grad(ffi, torch.from_numpy(scores).cuda(), np.concatenate([good, bad]), None,
+                                 oracle.LOSS_SQUARED_HINGE, 1.0)
+    assert rel_err(g, grad) <= RTOL and abs(loss_sum - losses.sum()) <= RTOL * losses.sum()
+
+
+def test_loss_grad_argument_errors(ffi):
+    lib = ffi._lib.lib()
+    s = torch.zeros((4, 8), device="cuda")
+    g = torch.zeros_like(s)
+    sh = torch.cuda.current_stream().cuda_stream
+    one = ctypes.c_float(1.0)
+    assert lib.ffi_loss_grad_f32(None, None, None, 0, 2, one, g.data_ptr(), None, 4, 8, sh) == -1
+    assert lib.ffi_loss_grad_f32(s.data_ptr(), None, None, 3, 2, one, g.data_ptr(), None, 4, 8, sh) == -1   # nnz without a list
+    assert lib.ffi_loss_grad_f32(s.data_ptr(), None, None, 0, 7, one, g.data_ptr(), None, 4, 8, sh) == -8   # unknown loss
+    assert lib.ffi_loss_grad_f32(s.data_ptr(), None, None, 0, 2, one, g.data_ptr(), None, 0, 8, sh) == -2
+    assert lib.ffi_loss_grad_f32(s.data_ptr(), None, None, -1, 2, one, g.data_ptr(), None, 4, 8, sh) == -2
+    assert lib.ffi_loss_grad_f32(s.data_ptr(), None, None, 0, 2, one, g.data_ptr(), None, 4, 8, sh) == 0    # loss_sum may be NULL
+    f = lib.ffi_forward_loss_f32
+    assert f(s.data_ptr(), s.data_ptr(), s.data_ptr(), None, None, None, 0, 2, one, g.data_ptr(), g.data_ptr(), None,
+             4, 8, 4, 2, 0, sh) == -8                                                                        # scores == out_grad
+
+
+#           B    N     L     K  transposed
+FUSED = [(128, 768, 5000, 32, True),
+         (37, 300, 1001, 7, False),
+         (64, 512, 2100, 64, True),
+         (33, 3000, 333, 12, True),        # wide inputs: forward kernel, then the loss as a pass of its own
+         (130, 2048, 260, 72, False)]
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("shape", FUSED)
+@pytest.mark.parametrize("want_scores,use_bias", [(False, True), (True, True), (False, False)])
+def test_forward_loss_fused_against_oracle(ffi, kind, shape, want_scores, use_bias):
+    B, N, L, K, tp = shape
+    rng = np.random.default_rng(B + N + L + K + kind)
+    x = np.maximum(rng.standard_normal((B, N)), 0).astype(np.float32)
+    lookup = rng.integers(0, N, size=(L, K)).astype(np.int32)
+    w = (rng.standard_normal((L, K)) * 0.4).astype(np.float32)
+    bias = (rng.standard_normal(L) * 0.5 - 0.5).astype(np.float32) if use_bias else None
+    indices, values = label_list(rng, B, L)
+    feats = np.ascontiguousarray(x.T) if tp else x
+    ref_scores = oracle.forward(feats, lookup, w, transposed=tp)
+    if use_bias:
+        ref_scores = ref_scores + bias[None, :]
+    losses, grad = oracle.sparse_loss(ref_scores, indices, values, kind)
+    scale = 1.0 / (B * L)
+
+    dev = lambda a: torch.from_numpy(a).cuda()  # noqa: E731
+    scores_t, g_t, loss_t = ffi.metrics.forward_loss(dev(feats), dev(lookup), dev(w), dev(bias) if use_bias else None,
+                                                     (dev(indices), dev(values)), kind, transposed=tp, want_scores=want_scores)
+    torch.cuda.synchronize()
+    if want_scores:
+        assert rel_err(scores_t.cpu().numpy(), ref_scores) <= RTOL
+    else:
+        assert scores_t is None
+    # a score differs from the oracle's by rounding (1e-5 gate); the gradient inherits that difference,
+    # scaled by the loss's curvature (at most 2), except across a kink of the hinge
+    ok = away_from_kinks(ref_scores, indices, values, kind, tol=2 * RTOL * max(1.0, float(np.abs(ref_scores).max())))
+    g = g_t.cpu().numpy()
+    assert np.abs(np.where(ok, g - grad * scale, 0)).max() <= 4 * RTOL * scale * max(1.0, np.abs(ref_scores).max())
+    assert abs(float(loss_t.cpu()[0]) - losses.sum()) <= RTOL * abs(losses.sum())
+
+
+def test_fused_loss_trains_like_the_unfused_ops(ffi):
+    # loss.fused(...) and loss(y, op(...) ) are the same differentiable function: equal value and gradients
+    B, N, L, K = 64, 256, 3000, 16
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.rand((B, N), device="cuda", generator=g)
+    lookup = torch.randint(0, N, (L, K), device="cuda", generator=g, dtype=torch.int64).to(torch.int32)
+    rng = np.random.default_rng(1)
+    indices, _ = label_list(rng, B, L, values=False)
+    y = (torch.from_numpy(indices).cuda(), None)
+    loss_fn = ffi.SparseSquaredHingeLoss()
+    results = []
+    for fused in (False, True):
+        w = ((torch.arange(L * K, device="cuda", dtype=torch.float32).reshape(L, K) % 13) / 13 - 0.5).requires_grad_(True)
+        bias = torch.full((L,), -0.3, device="cuda", requires_grad=True)
+        xin = x.clone().requires_grad_(True)
+        if fused:
+            loss, _ = loss_fn.fused(xin, lookup, w, bias, y)
+        else:
+            loss = loss_fn(y, ffi.fan_in_sparse_matmul_bias(xin, lookup, w, bias))
+        loss.backward()
+        torch.cuda.synchronize()
+        results.append((float(loss.detach()), w.grad.cpu().numpy(), bias.grad.cpu().numpy(), xin.grad.cpu().numpy()))
+    (l0, gw0, gb0, gx0), (l1, gw1, gb1, gx1) = results
+    assert abs(l0 - l1) <= 1e-5 * abs(l0)
+    assert rel_err(gw1, gw0) <= 1e-4 and rel_err(gb1, gb0) <= 1e-4 and rel_err(gx1, gx0) <= 1e-4
+    # and the value is the reference's: mean over labels, then over the batch
+    scores = oracle.forward(x.cpu().numpy(), lookup.cpu().numpy(), w.detach().cpu().numpy()) - 0.3
+    losses, _ = oracle.sparse_loss(scores, indices, None, oracle.LOSS_SQUARED_HINGE)
+    assert abs(l0 - losses.mean(axis=-1).mean()) <= 1e-5 * losses.mean()
+
+
+def test_loss_sum_is_reproducible(ffi):
+    B, L = 128, 20000
+    rng = np.random.default_rng(2)
+    scores = torch.from_numpy(rng.normal(0, 1, (B, L)).astype(np.float32)).cuda()
+    indices, values = label_list(rng, B, L)
+    a = call_loss_grad(ffi, scores, indices, values, oracle.LOSS_SQUARED_HINGE, 1.0)
+    b = call_loss_grad(ffi, scores, indices, values, oracle.LOSS_SQUARED_HINGE, 1.0)
+    assert a[1] == b[1] and np.array_equal(a[0], b[0])
+
+
+@pytest.mark.parametrize("k", [1, 3, 5])
+def test_precision_at_k(ffi, k):
+    # sparse/metrics.py:31-71: label values at the k best-scored positions, over batch * k
+    B, L = 50, 4000
+    rng = np.random.default_rng(k)
+    scores = rng.normal(0, 1, (B, L)).astype(np.float32)
+    indices, _ = label_list(rng, B, L, per_sample=4, values=False)
+    for b in range(0, B, 2):                      # make some labels rank high
+        scores[b, indices[indices[:, 0] == b][0, 1]] += 10.0
+    truth = np.zeros((B, L), bool)
+    truth[indices[:, 0], indices[:, 1]] = True
+    top = np.argsort(-scores, axis=1, kind="stable")[:, :k]
+    expected = truth[np.arange(B)[:, None], top].sum() / (B * k)
+    metric = ffi.PrecisionAtK(k=k)
+    metric.update_state((torch.from_numpy(indices).cuda(), None), torch.from_numpy(scores).cuda())
+    assert abs(metric.result() - expected) < 1e-12
+    metric.update_state((torch.from_numpy(indices).cuda(), None), torch.from_numpy(scores).cuda())
+    assert abs(metric.result() - expected) < 1e-12          # accumulates numerator and denominator

@@ -202,3 +202,84 @@ def test_topk_matches_sort_with_lower_index_first():
         order = np.lexsort((np.arange(s.shape[1]), -s[b]))[:5]
         assert np.array_equal(indices[b], order)
         assert np.array_equal(values[b], s[b, order])
+
+
+# ---- loss oracle (sparse/metrics.py:132-173 over sparse/utils.py:11-17) ----------------------------
+# Pinned by what the mathematics fixes: known values, a dense torch restatement differentiated by
+# autograd (torch's own relu / binary_cross_entropy_with_logits, not the oracle's formulas), and
+# central differences.
+def _loss_case(seed, B=7, L=23, nnz=19):
+    rng = np.random.default_rng(seed)
+    scores = rng.normal(0, 1.5, (B, L))
+    flat = rng.choice(B * L, size=nnz, replace=False)
+    indices = np.stack([flat // L, flat % L], axis=1).astype(np.int64)
+    values = rng.choice([1.0, 1.0, 0.5, 2.0], size=nnz)
+    return scores, indices, values
+
+
+def test_loss_oracle_known_values():
+    # score 0: hinge 1, squared hinge 1, bce log 2 whatever the label
+    for y in (0.0, 1.0):
+        assert oracle.cwise_loss(oracle.LOSS_HINGE, 0.0, y) == 1.0
+        assert oracle.cwise_loss(oracle.LOSS_SQUARED_HINGE, 0.0, y) == 1.0
+        assert abs(oracle.cwise_loss(oracle.LOSS_BCE, 0.0, y) - np.log(2.0)) < 1e-15
+    # a satisfied margin costs nothing and has zero gradient: negative at -1.5, positive at +1.5
+    for kind in (oracle.LOSS_HINGE, oracle.LOSS_SQUARED_HINGE):
+        assert oracle.cwise_loss(kind, -1.5, 0.0) == 0.0 and oracle.cwise_loss_grad(kind, -1.5, 0.0) == 0.0
+        assert oracle.cwise_loss(kind, 1.5, 1.0) == 0.0 and oracle.cwise_loss_grad(kind, 1.5, 1.0) == 0.0
+    # violated margins: negative at +2 -> relu(1+2) = 3, squared 9, slopes +1 and +6; positive at -2 -> same, slopes negated
+    assert oracle.cwise_loss(oracle.LOSS_HINGE, 2.0, 0.0) == 3.0 and oracle.cwise_loss_grad(oracle.LOSS_HINGE, 2.0, 0.0) == 1.0
+    assert oracle.cwise_loss(oracle.LOSS_SQUARED_HINGE, 2.0, 0.0) == 9.0 and oracle.cwise_loss_grad(oracle.LOSS_SQUARED_HINGE, 2.0, 0.0) == 6.0
+    assert oracle.cwise_loss(oracle.LOSS_SQUARED_HINGE, -2.0, 1.0) == 9.0 and oracle.cwise_loss_grad(oracle.LOSS_SQUARED_HINGE, -2.0, 1.0) == -6.0
+    # exactly on the margin the relu gradient is 0
+    assert oracle.cwise_loss_grad(oracle.LOSS_HINGE, -1.0, 0.0) == 0.0
+    # bce slope = sigmoid(s) - y
+    assert abs(oracle.cwise_loss_grad(oracle.LOSS_BCE, 0.0, 1.0) + 0.5) < 1e-15
+    assert abs(oracle.cwise_loss(oracle.LOSS_BCE, 30.0, 1.0)) < 1e-12 and abs(oracle.cwise_loss(oracle.LOSS_BCE, 30.0, 0.0) - 30.0) < 1e-12
+
+
+@pytest.mark.parametrize("kind", [1, 2, 3])
+def test_loss_oracle_against_dense_autograd(kind):
+    import torch
+    scores, indices, values = _loss_case(5 + kind)
+    losses, grad = oracle.sparse_loss(scores, indices, values, kind)
+    y = torch.zeros(scores.shape, dtype=torch.float64)
+    y[indices[:, 0], indices[:, 1]] = torch.from_numpy(values)
+    s = torch.from_numpy(scores).requires_grad_(True)
+    if kind == oracle.LOSS_BCE:
+        dense = torch.nn.functional.binary_cross_entropy_with_logits(s, y, reduction="none")
+    else:
+        hinge = torch.relu(1.0 - (2.0 * y - 1.0) * s)
+        dense = hinge if kind == oracle.LOSS_HINGE else hinge.square()
+    dense.sum().backward()
+    np.testing.assert_allclose(losses, dense.detach().numpy(), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(grad, s.grad.numpy(), rtol=1e-12, atol=1e-12)
+
+
+@pytest.mark.parametrize("kind", [2, 3])
+def test_loss_oracle_gradient_is_the_derivative(kind):
+    # central differences of the summed loss (smooth kinds; the hinge has kinks)
+    scores, indices, values = _loss_case(11)
+    _, grad = oracle.sparse_loss(scores, indices, values, kind)
+    rng = np.random.default_rng(0)
+    for _ in range(40):
+        b, j = rng.integers(scores.shape[0]), rng.integers(scores.shape[1])
+        h = 1e-6
+        up, dn = scores.copy(), scores.copy()
+        up[b, j] += h
+        dn[b, j] -= h
+        fd = (oracle.sparse_loss(up, indices, values, kind)[0].sum() - oracle.sparse_loss(dn, indices, values, kind)[0].sum()) / (2 * h)
+        assert abs(fd - grad[b, j]) < 1e-5 * max(1.0, abs(grad[b, j]))
+
+
+def test_loss_oracle_label_list_overrides_dense_part():
+    # an empty label list charges every entry as a negative; a listed entry changes only its own cell
+    scores, indices, values = _loss_case(3)
+    dense_l, dense_g = oracle.sparse_loss(scores, np.zeros((0, 2), np.int64), None, oracle.LOSS_SQUARED_HINGE)
+    np.testing.assert_array_equal(dense_l, np.maximum(1.0 + scores, 0.0) ** 2)
+    l, g = oracle.sparse_loss(scores, indices, None, oracle.LOSS_SQUARED_HINGE)
+    mask = np.zeros(scores.shape, bool)
+    mask[indices[:, 0], indices[:, 1]] = True
+    np.testing.assert_array_equal(l[~mask], dense_l[~mask])
+    np.testing.assert_array_equal(g[~mask], dense_g[~mask])
+    np.testing.assert_array_equal(l[mask], np.maximum(1.0 - scores[mask], 0.0) ** 2)
