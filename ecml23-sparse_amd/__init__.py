@@ -25,6 +25,7 @@ from .fixed_fan_in_ops import (  # noqa: E402
     fan_in_sparse_matmul_bias,
     fan_in_sparse_matmul_tp_bias,
     arrange_connections,
+    backward_sparse,
 )
 from . import custom_layer, metrics  # noqa: E402
 from .metrics import (  # noqa: E402
@@ -48,6 +49,7 @@ __all__ = [
     "fan_in_sparse_matmul_bias",
     "fan_in_sparse_matmul_tp_bias",
     "arrange_connections",
+    "backward_sparse",
     "StratifiedRewireLayerV2",
     "FixedFractionSelector",
     "FixedMagnitudeSelector",

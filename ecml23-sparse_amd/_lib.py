@@ -36,8 +36,9 @@ SIGNATURES = {
     "ffi_forward_bf16_f32": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "ffi_forward_topk_bf16": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "ffi_topk_f32": (_int, [_vp, _i64, _i64, _int, _vp, _vp, _vp]),
-    "ffi_loss_grad_f32": (_int, [_vp, _vp, _vp, _i64, _int, _f32, _vp, _vp, _i64, _i64, _vp]),
-    "ffi_forward_loss_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _int, _f32, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
+    "ffi_loss_grad_f32": (_int, [_vp, _vp, _vp, _i64, _int, _f32, _vp, _vp, _vp, _i64, _i64, _vp]),
+    "ffi_forward_loss_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _int, _f32, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
+    "ffi_backward_sparse_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _f32, _vp, _vp, _vp, ctypes.POINTER(_int), _i64, _i64, _i64, _i64, _int, _vp]),
 }
 
 _lib = None

@@ -27,6 +27,7 @@ SOURCES = [
     "ffi_wide.hip",
     "ffi_bf16.hip",
     "ffi_loss.hip",
+    "ffi_sparse_grad.hip",
 ]
 
 # gfx950 only.  Packed-fp32 VALU forms are switched off for all device code.

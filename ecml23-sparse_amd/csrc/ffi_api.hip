@@ -248,25 +248,55 @@ static int check_loss_args(const int64_t* label_indices, int64_t nnz, int loss_k
 }
 
 int ffi_loss_grad_f32(const float* scores, const int64_t* label_indices, const float* label_values, int64_t nnz,
-                      int loss_kind, float grad_scale, float* out_grad, float* loss_sum, int64_t batch, int64_t num_units,
-                      ffi_stream_t stream) {
+                      int loss_kind, float grad_scale, float* out_grad, float* loss_sum, uint32_t* nz_words, int64_t batch,
+                      int64_t num_units, ffi_stream_t stream) {
     if (!scores || !out_grad) return FFI_ERR_NULL_POINTER;
     FFI_TRY(check_loss_args(label_indices, nnz, loss_kind, batch, num_units));
-    const LossArgs la{label_indices, label_values, (int)nnz, loss_kind, grad_scale, loss_sum};
+    const LossArgs la{label_indices, label_values, (int)nnz, loss_kind, grad_scale, loss_sum, nz_words};
     return launch_loss_grad(la, scores, out_grad, (int)batch, (int)num_units, (hipStream_t)stream);
 }
 
 int ffi_forward_loss_f32(const float* features, const int32_t* lookup, const float* weights, const float* bias,
                          const int64_t* label_indices, const float* label_values, int64_t nnz, int loss_kind,
-                         float grad_scale, float* scores, float* out_grad, float* loss_sum, int64_t batch,
-                         int64_t num_features, int64_t num_units, int64_t fan_in, int transposed, ffi_stream_t stream) {
+                         float grad_scale, float* scores, float* out_grad, float* loss_sum, uint32_t* nz_words,
+                         int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in, int transposed,
+                         ffi_stream_t stream) {
     if (!features || !lookup || !weights || !out_grad) return FFI_ERR_NULL_POINTER;
     if (scores == out_grad) return FFI_ERR_BAD_ARGUMENT;
     Dims d;
     FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
     FFI_TRY(check_loss_args(label_indices, nnz, loss_kind, batch, num_units));
-    const LossArgs la{label_indices, label_values, (int)nnz, loss_kind, grad_scale, loss_sum};
+    const LossArgs la{label_indices, label_values, (int)nnz, loss_kind, grad_scale, loss_sum, nz_words};
     return launch_forward_loss(features, lookup, weights, bias, la, scores, out_grad, d, (hipStream_t)stream);
+}
+
+int ffi_backward_sparse_f32(const float* features, const int32_t* lookup, const float* weights, const float* out_grad,
+                            const uint32_t* nz_words, float max_density, float* feature_grad, float* weight_grad,
+                            float* bias_grad, int* sparse_path_taken, int64_t batch, int64_t num_features,
+                            int64_t num_units, int64_t fan_in, int transposed, ffi_stream_t stream) {
+    if (!features || !lookup || !weights || !out_grad) return FFI_ERR_NULL_POINTER;
+    if (!feature_grad && !weight_grad) return FFI_ERR_NULL_POINTER;
+    if (bias_grad && !weight_grad) return FFI_ERR_NULL_POINTER;
+    Dims d;
+    FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
+    hipStream_t s = (hipStream_t)stream;
+    const unsigned* words = nullptr;
+    unsigned long long set_bits = 0;
+    FFI_TRY(nonzero_count(out_grad, nz_words, d.B, d.L, s, &words, &set_bits));
+    const double limit = (double)(max_density > 0.f ? max_density : kSparseDefaultMaxDensity) * (double)d.B * (double)d.L;
+    const bool sparse = (double)set_bits <= limit;
+    if (sparse_path_taken) *sparse_path_taken = sparse ? 1 : 0;
+    auto wgrad = [&](const ffi_plan* plan) {
+        if (!weight_grad) return (int)FFI_OK;
+        if (sparse) return launch_weight_grad_sparse(features, lookup, out_grad, words, weight_grad, bias_grad, d, s);
+        return launch_weight_grad(features, lookup, out_grad, weight_grad, bias_grad, d, s, plan);
+    };
+    if (!feature_grad) return wgrad(nullptr);
+    if (sparse && sparse_input_grad_fits(d.N, d.K)) {
+        FFI_TRY(wgrad(nullptr));
+        return launch_input_grad_sparse(lookup, weights, out_grad, words, feature_grad, d, s);
+    }
+    return input_grad_cached(lookup, weights, out_grad, feature_grad, d, s, wgrad);
 }
 
 int ffi_plan_create(const int32_t* lookup, int64_t num_units, int64_t fan_in, int64_t num_features,

@@ -43,6 +43,7 @@ enum FwdEpilogue { kEpiScores = 0, kEpiLossGrad = 1, kEpiLossGradAndScores = 2 }
 struct FwdLoss {
     float* gout;        // [B,L] gradients (kEpiLossGradAndScores), else unused
     double* partial;    // [gridDim.x * wavefronts per workgroup] loss sums
+    unsigned* words;    // [ceil(B/32)][L] masks of the non-zero gradients to fill in, or null
     float scale;
     int kind;
 };
@@ -149,6 +150,12 @@ __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* _
 #pragma unroll
                 for (int b = 0; b < 32; ++b)
                     __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, acc[b]), EPI == kEpiLossGrad ? orsrc : grsrc, lane_off, (unsigned)b * stride, 0);
+                if (fl.words != nullptr) {
+                    unsigned m = 0;
+#pragma unroll
+                    for (int b = 0; b < 32; ++b) m |= (b < nrows && acc[b] != 0.f ? 1u : 0u) << b;
+                    fl.words[(size_t)bt * L + j] = m;
+                }
             }
         }
     }
@@ -190,7 +197,7 @@ int forward_tiles(const float* x, const int32_t* idx, const float* w, const floa
     const int per_stream = (d.L + streams - 1) / streams;
     streams = (d.L + per_stream - 1) / per_stream;
     const int blocks = streams * nbt;
-    FwdLoss fl{gout, nullptr, 0.f, 0};
+    FwdLoss fl{gout, nullptr, nullptr, 0.f, 0};
     if (epi == kEpiScores)
         return vec4 ? launch_lane32<true, kEpiScores>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, s)
                     : launch_lane32<false, kEpiScores>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, s);
@@ -199,6 +206,7 @@ int forward_tiles(const float* x, const int32_t* idx, const float* w, const floa
     FFI_TRY(loss_partial_buffer(s, npartial, la->nnz, &fl.partial, &corr, nullptr));
     fl.scale = la->scale;
     fl.kind = la->kind;
+    fl.words = la->nz_words;
     if (epi == kEpiLossGrad) {
         FFI_TRY(vec4 ? (launch_lane32<true, kEpiLossGrad>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, s))
                      : (launch_lane32<false, kEpiLossGrad>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, s)));

@@ -38,7 +38,7 @@ int hip_fail(hipError_t e);
 
 // Library-owned device scratch, one buffer per (device, stream, slot), grown on demand and kept.
 // Work that uses a buffer is ordered by the stream it belongs to.
-enum WorkspaceSlot { kWsFeaturesT = 0, kWsPartials = 1, kWsSlots = 2, kWsLoss = 3 };
+enum WorkspaceSlot { kWsFeaturesT = 0, kWsPartials = 1, kWsSlots = 2, kWsLoss = 3, kWsNonzero = 4 };
 int workspace_get(hipStream_t s, int slot, size_t bytes, void** out);
 void workspace_clear(int device);
 size_t workspace_bytes(int device);
@@ -76,6 +76,7 @@ struct LossArgs {
     int kind;                 // ffi_loss_kind
     float scale;              // factor on the gradient
     float* loss_sum;          // device float or null
+    unsigned* nz_words;       // [ceil(B/32)][L] non-zero masks of the gradient to fill in, or null
 };
 // partial[npartial] loss sums, corr[nnz] loss corrections and saved[nnz] scores of the listed positions
 int loss_partial_buffer(hipStream_t s, int npartial, int nnz, double** partial, double** corr, float** saved);
@@ -89,6 +90,22 @@ int launch_loss_grad(const LossArgs& la, const float* scores, float* g, int B, i
 // forward pass whose epilogue turns the scores into loss gradients (scores may be null)
 int launch_forward_loss(const float* x, const int32_t* idx, const float* w, const float* bias, const LossArgs& la,
                         float* scores, float* g, const Dims& d, hipStream_t s);
+
+// ---- backward pass over the non-zero entries of out_grad only (ffi_sparse_grad.hip) -------------
+// words[t][j]: bit i set <=> out_grad[32 t + i, j] may be non-zero
+constexpr int kSparseMaxFeatures = 3072;   // the sparse input gradient keeps 8 x N floats in LDS
+constexpr float kSparseDefaultMaxDensity = 0.01f;   // above this share of non-zeros the dense kernels are used
+// fills words from g
+int launch_nonzero_scan(const float* g, unsigned* words, int B, int L, hipStream_t s);
+// the masks to use (the caller's, or a scan of g into a workspace) and their number of set bits;
+// synchronises the stream
+int nonzero_count(const float* g, const unsigned* given_words, int B, int L, hipStream_t s, const unsigned** words_out,
+                  unsigned long long* count_out);
+int launch_weight_grad_sparse(const float* x, const int32_t* idx, const float* g, const unsigned* words, float* gw,
+                              float* bias_grad, const Dims& d, hipStream_t s);
+bool sparse_input_grad_fits(int N, int K);
+int launch_input_grad_sparse(const int32_t* idx, const float* w, const float* g, const unsigned* words, float* gx,
+                             const Dims& d, hipStream_t s);
 
 }  // namespace ffi
 

@@ -71,7 +71,7 @@ __global__ __launch_bounds__(kLossThreads) void loss_positive_kernel(
     const int64_t* __restrict__ label_indices, const float* __restrict__ label_values, int nnz,
     const float* __restrict__ saved, const float* __restrict__ scores, const float* __restrict__ x, size_t xsb, size_t xsn,
     const int32_t* __restrict__ idx, const float* __restrict__ w, const float* __restrict__ bias, float* __restrict__ g,
-    float scale, int kind, int B, int N, int L, int K, double* __restrict__ corr) {
+    float scale, int kind, int B, int N, int L, int K, double* __restrict__ corr, unsigned* __restrict__ nz_words) {
     const int p = blockIdx.x * kLossThreads + threadIdx.x;
     if (p >= nnz) return;
     const int64_t b = label_indices[2 * (size_t)p], j = label_indices[2 * (size_t)p + 1];
@@ -92,7 +92,10 @@ __global__ __launch_bounds__(kLossThreads) void loss_positive_kernel(
             if (bias != nullptr) s += bias[j];
         }
         const float y = label_values ? label_values[p] : 1.f;
-        g[(size_t)b * L + j] = scale * cwise_loss_grad(kind, s, y);
+        const float gv = scale * cwise_loss_grad(kind, s, y);
+        g[(size_t)b * L + j] = gv;
+        // the bulk pass set this position's mask bit from its gradient as a negative; a set bit over a zero is harmless
+        if (nz_words != nullptr && gv != 0.f) atomicOr(&nz_words[(size_t)(b >> 5) * L + j], 1u << (b & 31));
         // minus what the bulk pass charged this position as a negative (the same arithmetic as there)
         float l0, g0;
         cwise_loss_and_grad<false>(kind, s, 0.f, l0, g0);
@@ -136,7 +139,7 @@ int launch_loss_positives(const LossArgs& la, const float* saved, const float* s
         const size_t xsb = d.tp ? 1 : (size_t)d.N, xsn = d.tp ? (size_t)d.B : 1;
         hipLaunchKernelGGL(loss_positive_kernel, dim3((la.nnz + kLossThreads - 1) / kLossThreads), dim3(kLossThreads), 0, s,
                            la.indices, la.values, la.nnz, saved, scores, x, xsb, xsn, idx, w, bias, g, la.scale, la.kind, d.B, d.N,
-                           d.L, d.K, corr);
+                           d.L, d.K, corr, la.nz_words);
         FFI_HIP_TRY(hipGetLastError());
     }
     if (la.loss_sum != nullptr) {
@@ -164,8 +167,13 @@ int launch_loss_grad(const LossArgs& la, const float* scores, float* g, int B, i
     }
     hipLaunchKernelGGL(loss_dense_kernel, dim3(blocks), dim3(kLossThreads), 0, s, scores, g, total, la.scale, la.kind, partial);
     FFI_HIP_TRY(hipGetLastError());
+    // masks of the non-zero gradients, if asked for: a scan of the finished gradient (the listed positions included)
+    LossArgs la_pos = la;
+    la_pos.nz_words = nullptr;
     Dims d{B, 1, L, 1, false};
-    return launch_loss_positives(la, in_place ? saved : nullptr, scores, nullptr, nullptr, nullptr, nullptr, g, d, partial, npartial, corr, s);
+    FFI_TRY(launch_loss_positives(la_pos, in_place ? saved : nullptr, scores, nullptr, nullptr, nullptr, nullptr, g, d, partial, npartial, corr, s));
+    if (la.nz_words != nullptr) FFI_TRY(launch_nonzero_scan(g, la.nz_words, B, L, s));
+    return FFI_OK;
 }
 
 }  // namespace ffi

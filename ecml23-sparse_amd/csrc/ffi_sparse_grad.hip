@@ -1,0 +1,432 @@
+// Backward pass for an out_grad that is mostly exact zeros (a hinge loss late in training: every
+// satisfied margin has gradient 0).  The reference's GPU kernels skip such entries one by one
+// (`if(out == 0) continue`, tfsparse/cc/kernels/backward.cu.h:73,94,131,151); here the zero pattern is
+// made explicit once, as bit masks, and the kernels walk the set bits only:
+//
+//   words[t][j]      bit i set  <=>  out_grad[32 t + i, j] may be non-zero          (per label: weight gradient)
+//   bits[b][j / 64]  bit j % 64 set  <=>  the same for sample b                      (per sample: input gradient)
+//
+//   nz_scan_kernel          words from out_grad
+//   nz_count_kernel, nz_count_finish_kernel   the number of set bits (two steps, no atomics)
+//   nz_transpose_kernel     bits from words
+//   wgrad_sparse_kernel     lane <-> label: every lane walks the set bits of its own label and keeps 32 sums
+//                           (one chunk of connections) in registers; labels with many set bits are done by
+//                           the whole wavefront afterwards, lane <-> connection; rows of labels without a
+//                           set bit come out as zeros
+//   igrad_sparse_kernel     one workgroup per (sample, label segment): expands the sample's set bits to a list
+//                           of labels, then lanes <-> (label, connection) add g * w into per-wavefront
+//                           accumulators gx[n] in LDS (LDS float adds issued in a fixed order)
+//   igrad_sparse_reduce_kernel  sums the segments in ascending order into feature_grad
+#include "ffi_internal.h"
+
+#include <algorithm>
+#include <mutex>
+
+namespace ffi {
+namespace {
+
+constexpr int kScanThreads = 256;
+constexpr int kCountBlocks = 1024;
+
+__global__ __launch_bounds__(kScanThreads) void nz_scan_kernel(const float* __restrict__ g, unsigned* __restrict__ words,
+                                                               int B, int L) {
+    // two labels per thread (j and j + kScanThreads): 64 independent loads in flight
+    const int j0 = blockIdx.x * (2 * kScanThreads) + threadIdx.x;
+    const int t = blockIdx.y;
+    const int rows = min(32, B - 32 * t);
+    const float* tile = g + (size_t)(32 * t) * L;
+    float v[2][32];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int j = min(j0 + h * kScanThreads, L - 1);
+#pragma unroll
+        for (int i = 0; i < 32; ++i) v[h][i] = i < rows ? tile[(size_t)i * L + j] : 0.f;
+    }
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int j = j0 + h * kScanThreads;
+        unsigned m = 0;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) m |= (v[h][i] != 0.f ? 1u : 0u) << i;
+        if (j < L) words[(size_t)t * L + j] = m;
+    }
+}
+
+__global__ __launch_bounds__(kScanThreads) void nz_count_kernel(const unsigned* __restrict__ words, size_t n,
+                                                                unsigned long long* __restrict__ block_counts) {
+    __shared__ unsigned red[kScanThreads / 64];
+    unsigned c = 0;
+    for (size_t i = (size_t)blockIdx.x * kScanThreads + threadIdx.x; i < n; i += (size_t)gridDim.x * kScanThreads)
+        c += __popc(words[i]);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) c += __shfl_xor(c, off, 64);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = c;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned long long t = 0;
+        for (int i = 0; i < kScanThreads / 64; ++i) t += red[i];
+        block_counts[blockIdx.x] = t;
+    }
+}
+
+__global__ __launch_bounds__(64) void nz_count_finish_kernel(const unsigned long long* __restrict__ block_counts, int n,
+                                                             unsigned long long* __restrict__ host_count) {
+    unsigned long long t = 0;
+    for (int i = threadIdx.x; i < n; i += 64) t += block_counts[i];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) t += __shfl_xor(t, off, 64);
+    if (threadIdx.x == 0) *host_count = t;              // pinned host memory: the host reads it after the stream has drained
+}
+
+// One wavefront per (batch tile t, block of 64 labels): bits[32 t + i][blk] = ballot of bit i.
+__global__ __launch_bounds__(kScanThreads) void nz_transpose_kernel(const unsigned* __restrict__ words,
+                                                                    unsigned long long* __restrict__ bits, int B, int L,
+                                                                    int nwords) {
+    const int lane = threadIdx.x & 63;
+    const int blk = blockIdx.x * (kScanThreads / 64) + (threadIdx.x >> 6);
+    const int t = blockIdx.y;
+    if (blk >= nwords) return;
+    const int j = blk * 64 + lane;
+    const unsigned m = j < L ? words[(size_t)t * L + j] : 0u;
+    unsigned long long mine = 0;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+        const unsigned long long bl = __ballot((m >> i) & 1u);
+        if (lane == i) mine = bl;
+    }
+    const int b = 32 * t + lane;
+    if (lane < 32 && b < B) bits[(size_t)b * nwords + blk] = mine;
+}
+
+constexpr int kHeavyBits = 12;     // labels with more set bits than this are left to the whole wavefront
+
+// x is addressed as x[b * xsb + n * xsn] (either layout).
+template <bool VEC4>
+__global__ __launch_bounds__(256) void wgrad_sparse_kernel(const float* __restrict__ x, size_t xsb, size_t xsn,
+                                                           const int32_t* __restrict__ idx, const float* __restrict__ g,
+                                                           const unsigned* __restrict__ words, float* __restrict__ gw,
+                                                           float* __restrict__ bias_grad, int B, int N, int L, int K,
+                                                           int nbt) {
+    const int lane = threadIdx.x & 63;
+    const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int nwaves = gridDim.x * 4;
+    const int nblk = (L + 63) / 64;
+    const unsigned tail = (B & 31) ? (1u << (B & 31)) - 1u : 0xffffffffu;   // bits past the batch are ignored
+    for (int blk = wave; blk < nblk; blk += nwaves) {
+        const int base = blk * 64;
+        const int rows = min(64, L - base);
+        const int j = base + min(lane, rows - 1);
+        const bool mine = lane < rows;
+        int cnt = 0;
+        for (int t = 0; t < nbt; ++t) {
+            unsigned m = words[(size_t)t * L + j];
+            if (t == nbt - 1) m &= tail;
+            cnt += __popc(m);
+        }
+        const bool heavy = cnt > kHeavyBits;
+        const bool light = mine && !heavy;
+        // rows of labels without a set bit: zeros, written by the whole wavefront (the block's rows are contiguous in gw)
+        {
+            const unsigned long long zero_rows = __ballot(mine && cnt == 0);
+            float* blockrows = gw + (size_t)base * K;
+            if (VEC4) {
+                const int k4 = K / 4;
+                for (int e = lane; e < rows * k4; e += 64)
+                    if ((zero_rows >> (e / k4)) & 1ull) reinterpret_cast<float4*>(blockrows)[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+            } else {
+                for (int e = lane; e < rows * K; e += 64)
+                    if ((zero_rows >> (e / K)) & 1ull) blockrows[e] = 0.f;
+            }
+        }
+        // ---- every lane its own label ----
+        float gsum = 0.f;
+        for (int k0 = 0; k0 < K; k0 += 32) {
+            unsigned ids[32];
+            if (light && cnt) {
+                if (VEC4 && k0 + 32 <= K) {
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) {
+                        const int4 v = *reinterpret_cast<const int4*>(idx + (size_t)j * K + k0 + 4 * q);
+                        ids[4 * q] = (unsigned)v.x; ids[4 * q + 1] = (unsigned)v.y; ids[4 * q + 2] = (unsigned)v.z; ids[4 * q + 3] = (unsigned)v.w;
+                    }
+                } else {
+#pragma unroll
+                    for (int k = 0; k < 32; ++k) ids[k] = k0 + k < K ? (unsigned)idx[(size_t)j * K + k0 + k] : 0u;
+                }
+#pragma unroll
+                for (int k = 0; k < 32; ++k) ids[k] = ids[k] < (unsigned)N ? ids[k] : 0u;
+            } else {
+#pragma unroll
+                for (int k = 0; k < 32; ++k) ids[k] = 0u;
+            }
+            float acc[32];
+#pragma unroll
+            for (int k = 0; k < 32; ++k) acc[k] = 0.f;
+            for (int t = 0; t < nbt; ++t) {
+                unsigned m = light ? words[(size_t)t * L + j] : 0u;
+                if (t == nbt - 1) m &= tail;
+                while (__ballot(m != 0)) {
+                    if (m) {
+                        const int b = 32 * t + __ffs((int)m) - 1;
+                        m &= m - 1;
+                        const float gv = g[(size_t)b * L + j];
+                        const float* xrow = x + (size_t)b * xsb;
+#pragma unroll
+                        for (int k = 0; k < 32; ++k) acc[k] = fmaf(gv, xrow[(size_t)ids[k] * xsn], acc[k]);
+                        if (k0 == 0) gsum += gv;
+                    }
+                }
+            }
+            if (light && cnt) {
+                float* orow = gw + (size_t)j * K + k0;
+                if (VEC4 && k0 + 32 <= K) {
+#pragma unroll
+                    for (int q = 0; q < 8; ++q)
+                        *reinterpret_cast<float4*>(orow + 4 * q) = make_float4(acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]);
+                } else {
+#pragma unroll
+                    for (int k = 0; k < 32; ++k)
+                        if (k0 + k < K) orow[k] = acc[k];
+                }
+            }
+        }
+        if (bias_grad != nullptr && light) bias_grad[j] = gsum;
+        // ---- labels with many set bits: the whole wavefront on one label, lane <-> connection ----
+        unsigned long long todo = __ballot(mine && heavy);
+        while (todo) {
+            const int r = __builtin_amdgcn_readfirstlane(__ffsll((long long)todo) - 1);
+            todo &= todo - 1;
+            const int jh = base + r;
+            float hsum = 0.f;
+            for (int k0 = 0; k0 < K; k0 += 64) {
+                const int k = k0 + lane;
+                const unsigned id = k < K ? (unsigned)idx[(size_t)jh * K + k] : 0u;
+                const float* xcol = x + (size_t)(id < (unsigned)N ? id : 0u) * xsn;
+                float acc = 0.f;
+                hsum = 0.f;
+                for (int t = 0; t < nbt; ++t) {
+                    unsigned m = __builtin_amdgcn_readfirstlane(words[(size_t)t * L + jh]);
+                    if (t == nbt - 1) m &= tail;
+                    // up to four set bits per step, their loads in flight together
+                    while (m) {
+                        int bb[4];
+                        float gv[4], xv[4];
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            bb[u] = m ? 32 * t + __ffs((int)m) - 1 : -1;
+                            m &= m ? m - 1 : 0u;
+                        }
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            const int b = bb[u] < 0 ? 0 : bb[u];
+                            gv[u] = bb[u] < 0 ? 0.f : g[(size_t)b * L + jh];
+                            xv[u] = xcol[(size_t)b * xsb];
+                        }
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            acc = fmaf(gv[u], xv[u], acc);
+                            hsum += gv[u];
+                        }
+                    }
+                }
+                if (k < K) gw[(size_t)jh * K + k] = acc;
+            }
+            if (bias_grad != nullptr && lane == 0) bias_grad[jh] = hsum;
+        }
+    }
+}
+
+constexpr int kSgThreads = 512;
+constexpr int kSgWaves = kSgThreads / 64;
+constexpr int kSgChunkWords = 256;                     // 64-bit words expanded per round (one per thread of the first 256)
+constexpr int kSgListCap = kSgChunkWords * 64;         // labels of one round
+constexpr int kSgUnroll = 4;                           // entries a lane has in flight
+
+__global__ __launch_bounds__(kSgThreads) void igrad_sparse_kernel(const unsigned long long* __restrict__ bits, int nwords,
+                                                                  const int32_t* __restrict__ idx,
+                                                                  const float* __restrict__ w, const float* __restrict__ g,
+                                                                  float* __restrict__ partial, int B, int N, int L, int K,
+                                                                  int S, int words_per_seg, int kp) {
+    extern __shared__ __align__(16) unsigned char sg_lds[];
+    float* acc = reinterpret_cast<float*>(sg_lds);                                        // [kSgWaves][N]
+    unsigned short* list = reinterpret_cast<unsigned short*>(acc + (size_t)kSgWaves * N);   // [kSgListCap]
+    __shared__ int wave_total[kSgWaves];
+    const int b = blockIdx.x / S, seg = blockIdx.x % S;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    for (int i = threadIdx.x; i < kSgWaves * N; i += kSgThreads) acc[i] = 0.f;
+    const int w_begin = seg * words_per_seg;
+    const int w_end = min(w_begin + words_per_seg, nwords);
+    const unsigned long long* row = bits + (size_t)b * nwords;
+    const float* grow = g + (size_t)b * L;
+    float* myacc = acc + (size_t)wv * N;
+    // kp = fan-in rounded up to a power of two (at most 64): kp lanes per entry, 64 / kp entries per step
+    const int sub = lane / kp, kl = lane % kp, per = 64 / kp;
+    for (int w0 = w_begin; w0 < w_end; w0 += kSgChunkWords) {
+        const int wi = w0 + (int)threadIdx.x;
+        unsigned long long m = (threadIdx.x < kSgChunkWords && wi < w_end) ? row[wi] : 0ull;
+        const int c = __popcll(m);
+        // exclusive prefix of c over the workgroup
+        int incl = c;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int up = __shfl_up(incl, off, 64);
+            if (lane >= off) incl += up;
+        }
+        __syncthreads();                                   // the previous round's list and totals are no longer read
+        if (lane == 63) wave_total[wv] = incl;
+        __syncthreads();
+        int before = 0, total = 0;
+#pragma unroll
+        for (int i = 0; i < kSgWaves; ++i) {
+            if (i < wv) before += wave_total[i];
+            total += wave_total[i];
+        }
+        int pos = before + incl - c;
+        const unsigned short rel = (unsigned short)(threadIdx.x * 64);
+        while (m) {
+            list[pos++] = (unsigned short)(rel + (__ffsll((long long)m) - 1));
+            m &= m - 1;
+        }
+        __syncthreads();
+        // wavefront wv takes a contiguous share of the listed labels
+        const int e_begin = (int)((long long)total * wv / kSgWaves);
+        const int e_end = (int)((long long)total * (wv + 1) / kSgWaves);
+        const int jbase = w0 * 64;
+        for (int e0 = e_begin + sub; e0 < e_end; e0 += per * kSgUnroll) {
+            int jj[kSgUnroll];
+            float gv[kSgUnroll];
+#pragma unroll
+            for (int u = 0; u < kSgUnroll; ++u) {
+                const int e = e0 + u * per;
+                jj[u] = e < e_end ? jbase + list[e] : -1;
+            }
+#pragma unroll
+            for (int u = 0; u < kSgUnroll; ++u) gv[u] = jj[u] >= 0 ? grow[jj[u]] : 0.f;
+            for (int k = kl; k < K; k += kp) {
+                unsigned n[kSgUnroll];
+                float wk[kSgUnroll];
+#pragma unroll
+                for (int u = 0; u < kSgUnroll; ++u) {
+                    const size_t at = (size_t)(jj[u] >= 0 ? jj[u] : 0) * K + k;
+                    n[u] = (unsigned)idx[at];
+                    wk[u] = w[at];
+                }
+#pragma unroll
+                for (int u = 0; u < kSgUnroll; ++u)
+                    if (jj[u] >= 0 && n[u] < (unsigned)N) atomicAdd(&myacc[n[u]], gv[u] * wk[u]);
+            }
+        }
+    }
+    __syncthreads();
+    float* out = partial + ((size_t)seg * B + b) * N;
+    for (int n = threadIdx.x; n < N; n += kSgThreads) {
+        float t = acc[n];
+#pragma unroll
+        for (int i = 1; i < kSgWaves; ++i) t += acc[(size_t)i * N + n];
+        out[n] = t;
+    }
+}
+
+__global__ __launch_bounds__(256) void igrad_sparse_reduce_kernel(const float* __restrict__ partial, int S, int B, int N,
+                                                                  float* __restrict__ gx, int tp) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (size_t)B * N) return;
+    float t = 0.f;
+    for (int s = 0; s < S; ++s) t += partial[(size_t)s * B * N + i];
+    const int b = (int)(i / N), n = (int)(i - (size_t)b * N);
+    gx[tp ? (size_t)n * B + b : i] = t;
+}
+
+// pinned word the set-bit count is copied to; one per device, calls on a device take turns
+std::mutex g_count_mutex;
+unsigned long long* g_count_host[64] = {nullptr};
+
+}  // namespace
+
+int launch_nonzero_scan(const float* g, unsigned* words, int B, int L, hipStream_t s) {
+    const int nbt = (B + 31) / 32;
+    hipLaunchKernelGGL(nz_scan_kernel, dim3((L + 2 * kScanThreads - 1) / (2 * kScanThreads), nbt), dim3(kScanThreads), 0, s, g, words, B, L);
+    FFI_HIP_TRY(hipGetLastError());
+    return FFI_OK;
+}
+
+int nonzero_count(const float* g, const unsigned* given_words, int B, int L, hipStream_t s, const unsigned** words_out,
+                  unsigned long long* count_out) {
+    const int nbt = (B + 31) / 32;
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return FFI_ERR_NO_DEVICE;
+    const size_t head = (size_t)kCountBlocks * sizeof(unsigned long long);           // block counts
+    const size_t words_bytes = (size_t)nbt * L * sizeof(unsigned);
+    unsigned char* ws = nullptr;
+    FFI_TRY(workspace_get(s, kWsNonzero, head + (given_words ? 0 : words_bytes), (void**)&ws));
+    unsigned long long* block_counts = reinterpret_cast<unsigned long long*>(ws);
+    const unsigned* words = given_words;
+    if (!given_words) {
+        unsigned* scanned = reinterpret_cast<unsigned*>(ws + head);
+        FFI_TRY(launch_nonzero_scan(g, scanned, B, L, s));
+        words = scanned;
+    }
+    *words_out = words;
+    std::lock_guard<std::mutex> lock(g_count_mutex);
+    if (!g_count_host[dev]) {
+        if (hipHostMalloc((void**)&g_count_host[dev], 64) != hipSuccess) { (void)hipGetLastError(); return FFI_ERR_OUT_OF_MEMORY; }
+    }
+    hipLaunchKernelGGL(nz_count_kernel, dim3(kCountBlocks), dim3(kScanThreads), 0, s, words, (size_t)nbt * L, block_counts);
+    hipLaunchKernelGGL(nz_count_finish_kernel, dim3(1), dim3(64), 0, s, block_counts, kCountBlocks, g_count_host[dev]);
+    FFI_HIP_TRY(hipGetLastError());
+    FFI_HIP_TRY(hipStreamSynchronize(s));
+    *count_out = *reinterpret_cast<volatile unsigned long long*>(g_count_host[dev]);
+    return FFI_OK;
+}
+
+int launch_weight_grad_sparse(const float* x, const int32_t* idx, const float* g, const unsigned* words, float* gw,
+                              float* bias_grad, const Dims& d, hipStream_t s) {
+    const int nbt = (d.B + 31) / 32;
+    const int nblk = (d.L + 63) / 64;
+    const int blocks = std::max(1, std::min((nblk + 3) / 4, device_cu_count() * 8));
+    const size_t xsb = d.tp ? 1 : (size_t)d.N, xsn = d.tp ? (size_t)d.B : 1;
+    const bool vec4 = (d.K % 4 == 0) && (((uintptr_t)gw | (uintptr_t)idx) % 16 == 0);
+    if (vec4)
+        hipLaunchKernelGGL(wgrad_sparse_kernel<true>, dim3(blocks), dim3(256), 0, s, x, xsb, xsn, idx, g, words, gw, bias_grad, d.B,
+                           d.N, d.L, d.K, nbt);
+    else
+        hipLaunchKernelGGL(wgrad_sparse_kernel<false>, dim3(blocks), dim3(256), 0, s, x, xsb, xsn, idx, g, words, gw, bias_grad, d.B,
+                           d.N, d.L, d.K, nbt);
+    FFI_HIP_TRY(hipGetLastError());
+    return FFI_OK;
+}
+
+bool sparse_input_grad_fits(int N, int K) { return N <= kSparseMaxFeatures && K <= 65535; }
+
+int launch_input_grad_sparse(const int32_t* idx, const float* w, const float* g, const unsigned* words, float* gx,
+                             const Dims& d, hipStream_t s) {
+    const int nbt = (d.B + 31) / 32;
+    const int nwords = (d.L + 63) / 64;
+    // label segments per sample: enough workgroups to fill the GPU, each with at least one round of words
+    int S = std::max(1, (4 * device_cu_count() + d.B - 1) / d.B);
+    S = std::max(1, std::min(S, (nwords + kSgChunkWords - 1) / kSgChunkWords));
+    const int words_per_seg = (nwords + S - 1) / S;
+    S = (nwords + words_per_seg - 1) / words_per_seg;
+    const size_t bits_bytes = (size_t)d.B * nwords * sizeof(unsigned long long);
+    const size_t partial_bytes = (size_t)S * d.B * d.N * sizeof(float);
+    unsigned char* ws = nullptr;
+    FFI_TRY(workspace_get(s, kWsPartials, bits_bytes + partial_bytes, (void**)&ws));
+    unsigned long long* bits = reinterpret_cast<unsigned long long*>(ws);
+    float* partial = reinterpret_cast<float*>(ws + bits_bytes);
+    hipLaunchKernelGGL(nz_transpose_kernel, dim3((nwords + 3) / 4, nbt), dim3(kScanThreads), 0, s, words, bits, d.B, d.L, nwords);
+    FFI_HIP_TRY(hipGetLastError());
+    int kp = 1;
+    while (kp < d.K && kp < 64) kp *= 2;
+    const size_t lds = (size_t)kSgWaves * d.N * sizeof(float) + (size_t)kSgListCap * sizeof(unsigned short);
+    FFI_HIP_TRY(hipFuncSetAttribute((const void*)igrad_sparse_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(igrad_sparse_kernel, dim3(d.B * S), dim3(kSgThreads), lds, s, bits, nwords, idx, w, g, partial, d.B, d.N,
+                       d.L, d.K, S, words_per_seg, kp);
+    FFI_HIP_TRY(hipGetLastError());
+    const size_t total = (size_t)d.B * d.N;
+    hipLaunchKernelGGL(igrad_sparse_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, partial, S, d.B, d.N,
+                       gx, d.tp ? 1 : 0);
+    FFI_HIP_TRY(hipGetLastError());
+    return FFI_OK;
+}
+
+}  // namespace ffi

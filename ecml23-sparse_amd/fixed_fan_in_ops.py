@@ -274,6 +274,36 @@ def fan_in_sparse_matmul_tp_bias(features, lookup, weights, bias):
     return FanInSparseMatmulBiasTp.apply(features, lookup, weights, bias)
 
 
+def backward_sparse(features, lookup, weights, out_grad, nz_words=None, max_density=None, transposed=False,
+                    need_feature_grad=True, need_bias_grad=False):
+    """Backward pass that walks only the non-zero entries of ``out_grad`` (what the reference's GPU
+    kernels do entry by entry, tfsparse/cc/kernels/backward.cu.h:73,94,131,151).
+
+    ``nz_words`` ([ceil(B/32), L] int32 bit masks from ``metrics.forward_loss(..., want_masks=True)``)
+    saves the scan of ``out_grad``.  Above ``max_density`` (share of non-zeros; default: the
+    library's) the dense kernels run instead.  Returns ``(feature_grad or None, weight_grad,
+    bias_grad or None, sparse_kernels_ran)``."""
+    import ctypes
+
+    batch, num_features, num_units, fan_in = _check_inputs(features, lookup, weights, transposed, out_grad)
+    features, lookup, weights, out_grad = features.contiguous(), lookup.contiguous(), weights.contiguous(), out_grad.contiguous()
+    if nz_words is not None:
+        if nz_words.dtype != torch.int32 or tuple(nz_words.shape) != ((batch + 31) // 32, num_units) or not nz_words.is_contiguous():
+            raise ValueError(f"nz_words must be a contiguous int32 tensor of shape {((batch + 31) // 32, num_units)}")
+    taken = ctypes.c_int(-1)
+    with torch.cuda.device(features.device):
+        feature_grad = torch.empty_like(features) if need_feature_grad else None
+        weight_grad = torch.empty_like(weights)
+        bias_grad = torch.empty((num_units,), dtype=torch.float32, device=features.device) if need_bias_grad else None
+        _lib.check(_lib.lib().ffi_backward_sparse_f32(
+            features.data_ptr(), lookup.data_ptr(), weights.data_ptr(), out_grad.data_ptr(),
+            nz_words.data_ptr() if nz_words is not None else None, float(max_density or 0.0),
+            feature_grad.data_ptr() if need_feature_grad else None, weight_grad.data_ptr(),
+            bias_grad.data_ptr() if need_bias_grad else None, ctypes.byref(taken),
+            batch, num_features, num_units, fan_in, int(transposed), _stream_handle(features.device)))
+    return feature_grad, weight_grad, bias_grad, bool(taken.value)
+
+
 def arrange_connections(lookup, *arrays):
     """Reorders, in place, the connections inside every row of ``lookup`` ([L,K] int32/uint32) so that
     even and odd column ids alternate (which the kernels read faster), and applies the same

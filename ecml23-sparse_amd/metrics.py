@@ -14,7 +14,7 @@ from __future__ import annotations
 import torch
 
 from . import _lib
-from .fixed_fan_in_ops import _check_bias, _check_inputs, _backward_bias, _backward, _stream_handle, topk_scores
+from .fixed_fan_in_ops import _check_bias, _check_inputs, _stream_handle, backward_sparse, topk_scores
 
 LOSS_HINGE, LOSS_SQUARED_HINGE, LOSS_BCE = 1, 2, 3
 
@@ -38,10 +38,11 @@ def _labels(y_true, device):
     return indices, values
 
 
-def sparse_loss_grad(scores, y_true, kind, grad_scale=None, in_place=False):
+def sparse_loss_grad(scores, y_true, kind, grad_scale=None, in_place=False, want_masks=False):
     """``(out_grad [B,L], loss_sum [1])``: ``out_grad = grad_scale * d loss / d scores`` and the
     un-scaled sum of the element losses.  ``grad_scale`` defaults to ``1 / (B * L)``;
-    ``in_place`` overwrites ``scores`` with the gradient."""
+    ``in_place`` overwrites ``scores`` with the gradient.  With ``want_masks`` a third result holds
+    the bit masks of the non-zero gradients (``[ceil(B/32), L]`` int32) for ``backward_sparse``."""
     if scores.dim() != 2 or scores.dtype != torch.float32:
         raise TypeError("scores must be a float32 [batch, num_units] matrix")
     if not scores.is_cuda:
@@ -55,15 +56,19 @@ def sparse_loss_grad(scores, y_true, kind, grad_scale=None, in_place=False):
     with torch.cuda.device(scores.device):
         out_grad = scores if in_place else torch.empty_like(scores)
         loss_sum = torch.empty((1,), dtype=torch.float32, device=scores.device)
+        masks = torch.empty(((batch + 31) // 32, num_units), dtype=torch.int32, device=scores.device) if want_masks else None
         _lib.check(_lib.lib().ffi_loss_grad_f32(
             scores.data_ptr(), indices.data_ptr() if indices.numel() else None,
             values.data_ptr() if values is not None and values.numel() else None, indices.shape[0], int(kind), scale,
-            out_grad.data_ptr(), loss_sum.data_ptr(), batch, num_units, _stream_handle(scores.device)))
-    return out_grad, loss_sum
+            out_grad.data_ptr(), loss_sum.data_ptr(), masks.data_ptr() if want_masks else None, batch, num_units,
+            _stream_handle(scores.device)))
+    return (out_grad, loss_sum, masks) if want_masks else (out_grad, loss_sum)
 
 
-def forward_loss(features, lookup, weights, bias, y_true, kind, grad_scale=None, transposed=False, want_scores=False):
-    """Forward pass, bias add and loss gradient in one kernel: ``(scores or None, out_grad, loss_sum)``."""
+def forward_loss(features, lookup, weights, bias, y_true, kind, grad_scale=None, transposed=False, want_scores=False,
+                 want_masks=False):
+    """Forward pass, bias add and loss gradient in one kernel: ``(scores or None, out_grad, loss_sum)``,
+    plus the bit masks of the non-zero gradients with ``want_masks``."""
     batch, num_features, num_units, fan_in = _check_inputs(features, lookup, weights, transposed)
     if bias is not None:
         _check_bias(bias, weights, num_units)
@@ -75,13 +80,15 @@ def forward_loss(features, lookup, weights, bias, y_true, kind, grad_scale=None,
         out_grad = torch.empty((batch, num_units), dtype=torch.float32, device=features.device)
         scores = torch.empty_like(out_grad) if want_scores else None
         loss_sum = torch.empty((1,), dtype=torch.float32, device=features.device)
+        masks = torch.empty(((batch + 31) // 32, num_units), dtype=torch.int32, device=features.device) if want_masks else None
         _lib.check(_lib.lib().ffi_forward_loss_f32(
             features.data_ptr(), lookup.data_ptr(), weights.data_ptr(), bias.data_ptr() if bias is not None else None,
             indices.data_ptr() if indices.numel() else None,
             values.data_ptr() if values is not None and values.numel() else None, indices.shape[0], int(kind), scale,
             scores.data_ptr() if want_scores else None, out_grad.data_ptr(), loss_sum.data_ptr(),
+            masks.data_ptr() if want_masks else None,
             batch, num_features, num_units, fan_in, int(transposed), _stream_handle(features.device)))
-    return scores, out_grad, loss_sum
+    return (scores, out_grad, loss_sum, masks) if want_masks else (scores, out_grad, loss_sum)
 
 
 def _scaled(out_grad, upstream):
@@ -109,9 +116,9 @@ class _LayerLossFn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, features, lookup, weights, bias, indices, values, kind, transposed, want_scores):
-        scores, out_grad, loss_sum = forward_loss(features, lookup, weights, bias, (indices, values), kind,
-                                                  transposed=transposed, want_scores=want_scores)
-        ctx.save_for_backward(features, lookup, weights, out_grad)
+        scores, out_grad, loss_sum, masks = forward_loss(features, lookup, weights, bias, (indices, values), kind,
+                                                         transposed=transposed, want_scores=want_scores, want_masks=True)
+        ctx.save_for_backward(features, lookup, weights, out_grad, masks)
         ctx.transposed = transposed
         ctx.has_bias = bias is not None
         batch = features.shape[1] if transposed else features.shape[0]
@@ -123,14 +130,13 @@ class _LayerLossFn(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad, _grad_scores):
-        features, lookup, weights, out_grad = ctx.saved_tensors
+        features, lookup, weights, out_grad, masks = ctx.saved_tensors
         g = _scaled(out_grad, grad)
-        if ctx.has_bias:
-            feature_grad, weight_grad, bias_grad = _backward_bias(features, lookup, weights, g, ctx.transposed,
-                                                                  need_feature_grad=ctx.needs_input_grad[0])
-        else:
-            feature_grad, weight_grad = _backward(features, lookup, weights, g, ctx.transposed)
-            bias_grad = None
+        # the masks say where the gradient is not zero: the backward pass skips the rest when they are few
+        feature_grad, weight_grad, bias_grad, _ = backward_sparse(features, lookup, weights, g, nz_words=masks,
+                                                                  transposed=ctx.transposed,
+                                                                  need_feature_grad=ctx.needs_input_grad[0],
+                                                                  need_bias_grad=ctx.has_bias)
         return feature_grad, None, weight_grad, bias_grad, None, None, None, None, None
 
 

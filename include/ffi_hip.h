@@ -195,6 +195,8 @@ int ffi_topk_f32(const float* scores, int64_t batch, int64_t num_units, int k,
  *   out_grad[b,j]  = grad_scale * d loss / d score  (Keras' mean over labels, then over the batch,
  *                    is grad_scale = 1 / (batch * num_units)); may alias `scores`;
  *   loss_sum       one float on the device: the un-scaled sum of the element losses; may be NULL.
+ *   nz_words       [ceil(batch/32), num_units] uint32, may be NULL: bit i of nz_words[t, j] is set where
+ *                  out_grad[32 t + i, j] is not zero, the masks ffi_backward_sparse_f32 accepts.
  * Sums are formed in a fixed order (no atomics).
  */
 enum ffi_loss_kind {
@@ -203,7 +205,7 @@ enum ffi_loss_kind {
     FFI_LOSS_BCE = 3              /* SparseBinaryCrossEntropyLoss  sparse/metrics.py:167-173 */
 };
 int ffi_loss_grad_f32(const float* scores, const int64_t* label_indices, const float* label_values, int64_t nnz,
-                      int loss_kind, float grad_scale, float* out_grad, float* loss_sum,
+                      int loss_kind, float grad_scale, float* out_grad, float* loss_sum, uint32_t* nz_words,
                       int64_t batch, int64_t num_units, ffi_stream_t stream);
 
 /*
@@ -216,8 +218,30 @@ int ffi_loss_grad_f32(const float* scores, const int64_t* label_indices, const f
 int ffi_forward_loss_f32(const float* features, const int32_t* lookup, const float* weights, const float* bias,
                          const int64_t* label_indices, const float* label_values, int64_t nnz,
                          int loss_kind, float grad_scale, float* scores, float* out_grad, float* loss_sum,
+                         uint32_t* nz_words,
                          int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in,
                          int transposed, ffi_stream_t stream);
+
+/*
+ * Backward pass that skips the exact zeros of out_grad, as the reference's GPU kernels do entry by
+ * entry (`if(out == 0) continue`, tfsparse/cc/kernels/backward.cu.h:73,94,131,151): with a hinge loss
+ * every satisfied margin has gradient 0, and late in training that is nearly all of them.  Same
+ * results as ffi_backward_bias_f32 (bias_grad may be NULL here) up to summation order.
+ *   nz_words      the masks of the non-zero entries as ffi_forward_loss_f32 / ffi_loss_grad_f32 write
+ *                 them (a set bit over a zero entry is allowed, a clear bit over a non-zero entry is
+ *                 not), or NULL: out_grad is then scanned first (one read of the matrix);
+ *   max_density   share of set bits up to which the sparse kernels are used (<= 0: library default);
+ *                 above it the call runs the dense kernels of ffi_backward_bias_f32;
+ *   sparse_path_taken  HOST int, may be NULL: 1 if the sparse kernels ran, 0 if the dense ones did.
+ * Synchronises `stream` once (the host reads the number of set bits).  The sparse input gradient
+ * covers num_features <= 3072; wider inputs take the dense input-gradient kernels.  It accumulates
+ * with LDS float adds issued in a fixed order, no global atomics.
+ */
+int ffi_backward_sparse_f32(const float* features, const int32_t* lookup, const float* weights,
+                            const float* out_grad, const uint32_t* nz_words, float max_density,
+                            float* feature_grad, float* weight_grad, float* bias_grad, int* sparse_path_taken,
+                            int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in,
+                            int transposed, ffi_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,180 @@
+"""Backward pass over the non-zero entries of out_grad only (`ffi_backward_sparse_f32`), against the
+oracle's backward (backward.cpp:8-73 restated) on the same inputs: the reference's GPU kernels skip
+exact zeros entry by entry (backward.cu.h:73,94,131,151) and get the same sums.
+
+Gate: 1e-4 of the largest reference magnitude, as for the dense gradients.  out_grad is drawn with a
+given share of non-zeros; masks are either computed here from out_grad, handed in with extra set
+bits, produced by the loss kernels, or left to the library (NULL).
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from conftest import load_package, rel_err
+
+pytestmark = pytest.mark.gpu
+
+GRAD_RTOL = 1e-4
+
+#          B    N     L     K  transposed
+SHAPES = [(128, 768, 5000, 32, True),
+          (37, 300, 1001, 7, False),
+          (64, 512, 2100, 64, True),
+          (200, 96, 700, 72, False),
+          (33, 3000, 333, 12, True),
+          (40, 5000, 400, 20, False),       # wider than the sparse input gradient covers: dense kernels for gx
+          (1, 16, 70, 3, False)]
+
+
+@pytest.fixture(scope="module")
+def ffi():
+    pkg = load_package()
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    return pkg
+
+
+def make_case(shape, density, seed):
+    B, N, L, K, tp = shape
+    rng = np.random.default_rng(seed)
+    x = np.maximum(rng.standard_normal((B, N)), 0).astype(np.float32)
+    lookup = rng.integers(0, N, size=(L, K)).astype(np.int32)
+    w = rng.standard_normal((L, K)).astype(np.float32)
+    g = rng.standard_normal((B, L)).astype(np.float32)
+    g[rng.random((B, L)) >= density] = 0.0
+    if density > 0 and L > 5:
+        g[:, 3] = rng.standard_normal(B)            # one label that every sample pushes on
+    feats = np.ascontiguousarray(x.T) if tp else x
+    return feats, lookup, w, g
+
+
+def masks_of(g):
+    B, L = g.shape
+    nbt = (B + 31) // 32
+    words = np.zeros((nbt, L), np.uint32)
+    for b in range(B):
+        words[b // 32] |= (g[b] != 0).astype(np.uint32) << np.uint32(b % 32)
+    return words.view(np.int32)
+
+
+def run(ffi, feats, lookup, w, g, tp, words=None, max_density=1.0):
+    dev = lambda a: torch.from_numpy(a).cuda()  # noqa: E731
+    gx, gw, gb, sparse = ffi.backward_sparse(dev(feats), dev(lookup), dev(w), dev(g),
+                                             nz_words=dev(words) if words is not None else None,
+                                             max_density=max_density, transposed=tp, need_bias_grad=True)
+    torch.cuda.synchronize()
+    return gx.cpu().numpy(), gw.cpu().numpy(), gb.cpu().numpy(), sparse
+
+
+@pytest.mark.parametrize("density", [0.001, 0.02, 0.3])
+@pytest.mark.parametrize("given_masks", [False, True])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_sparse_backward_against_oracle(ffi, shape, density, given_masks):
+    tp = shape[4]
+    feats, lookup, w, g = make_case(shape, density, seed=sum(shape[:4]))
+    ref_gx, ref_gw = oracle.backward(feats, lookup, w, g, transposed=tp)
+    gx, gw, gb, sparse = run(ffi, feats, lookup, w, g, tp, words=masks_of(g) if given_masks else None)
+    assert sparse                                   # max_density = 1 forces the sparse kernels
+    assert rel_err(gw, ref_gw) <= GRAD_RTOL
+    assert rel_err(gx, ref_gx) <= GRAD_RTOL
+    assert rel_err(gb, g.astype(np.float64).sum(axis=0)) <= GRAD_RTOL
+
+
+def test_default_threshold_picks_dense_kernels_for_dense_gradients(ffi):
+    shape = (128, 768, 5000, 32, True)
+    feats, lookup, w, g = make_case(shape, 0.5, seed=1)
+    ref_gx, ref_gw = oracle.backward(feats, lookup, w, g, transposed=True)
+    gx, gw, gb, sparse = run(ffi, feats, lookup, w, g, True, max_density=None)
+    assert not sparse
+    assert rel_err(gw, ref_gw) <= GRAD_RTOL and rel_err(gx, ref_gx) <= GRAD_RTOL
+    assert rel_err(gb, g.astype(np.float64).sum(axis=0)) <= GRAD_RTOL
+    feats, lookup, w, g = make_case(shape, 0.002, seed=2)
+    ref_gx, ref_gw = oracle.backward(feats, lookup, w, g, transposed=True)
+    gx, gw, gb, sparse = run(ffi, feats, lookup, w, g, True, max_density=None)
+    assert sparse
+    assert rel_err(gw, ref_gw) <= GRAD_RTOL and rel_err(gx, ref_gx) <= GRAD_RTOL
+
+
+def test_all_zero_gradient_gives_exact_zeros(ffi):
+    shape = (70, 200, 900, 16, False)
+    feats, lookup, w, g = make_case(shape, 0.0, seed=3)
+    gx, gw, gb, sparse = run(ffi, feats, lookup, w, g, False)
+    assert sparse and not gx.any() and not gw.any() and not gb.any()
+
+
+def test_masks_may_cover_zero_entries(ffi):
+    # a set bit over a zero entry only costs time
+    shape = (64, 256, 1500, 24, True)
+    feats, lookup, w, g = make_case(shape, 0.01, seed=4)
+    words = masks_of(g).view(np.uint32).copy()
+    rng = np.random.default_rng(0)
+    words |= (rng.random(words.shape) < 0.05).astype(np.uint32) << np.uint32(7)
+    words[:, 10:20] = 0xFFFFFFFF
+    ref_gx, ref_gw = oracle.backward(feats, lookup, w, g, transposed=True)
+    gx, gw, gb, sparse = run(ffi, feats, lookup, w, g, True, words=words.view(np.int32))
+    assert sparse and rel_err(gw, ref_gw) <= GRAD_RTOL and rel_err(gx, ref_gx) <= GRAD_RTOL
+
+
+def test_sparse_backward_is_reproducible(ffi):
+    shape = (128, 768, 20000, 32, True)
+    feats, lookup, w, g = make_case(shape, 0.01, seed=5)
+    a = run(ffi, feats, lookup, w, g, True)
+    b = run(ffi, feats, lookup, w, g, True)
+    assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1]) and np.array_equal(a[2], b[2])
+
+
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("shape", [(128, 768, 5000, 32, True), (37, 300, 1001, 7, False), (33, 3000, 333, 12, True)])
+def test_loss_kernels_write_the_masks_of_their_gradient(ffi, shape, fused):
+    B, N, L, K, tp = shape
+    rng = np.random.default_rng(6)
+    feats, lookup, w, _ = make_case(shape, 0.0, seed=6)
+    w *= 0.3
+    bias = np.full(L, -1.5, np.float32)             # most margins satisfied: a sparse gradient
+    rows = np.repeat(np.arange(B), 3)
+    cols = rng.integers(0, L, B * 3)
+    keys = np.unique(rows * L + cols)
+    indices = np.stack([keys // L, keys % L], axis=1).astype(np.int64)
+    dev = lambda a: torch.from_numpy(a).cuda()  # noqa: E731
+    y = (dev(indices), None)
+    if fused:
+        _, g_t, _, masks = ffi.metrics.forward_loss(dev(feats), dev(lookup), dev(w), dev(bias), y, oracle.LOSS_SQUARED_HINGE,
+                                                    transposed=tp, want_masks=True)
+    else:
+        scores = ffi.fan_in_sparse_matmul_tp_bias(dev(feats), dev(lookup), dev(w), dev(bias)) if tp else \
+            ffi.fan_in_sparse_matmul_bias(dev(feats), dev(lookup), dev(w), dev(bias))
+        g_t, _, masks = ffi.metrics.sparse_loss_grad(scores, y, oracle.LOSS_SQUARED_HINGE, want_masks=True)
+    torch.cuda.synchronize()
+    g = g_t.cpu().numpy()
+    got = masks.cpu().numpy().view(np.uint32)
+    want = masks_of(g).view(np.uint32)
+    assert 0 < (g != 0).mean() < 0.5
+    assert not (want & ~got).any()                  # every non-zero entry is covered
+    # nothing else is, except listed label positions whose gradient as a negative was non-zero
+    # and whose gradient as a positive is zero (the fused kernel sets bits before the labels are applied)
+    allowed = np.zeros_like(want)
+    np.bitwise_or.at(allowed, (indices[:, 0] // 32, indices[:, 1]), np.uint32(1) << (indices[:, 0] % 32).astype(np.uint32))
+    assert not (got & ~want & ~allowed).any()
+
+
+def test_fused_loss_backward_uses_the_sparse_kernels(ffi):
+    # end to end through autograd: fused loss forward, masks kept, sparse backward; against the dense route
+    B, N, L, K = 64, 256, 4000, 16
+    gen = torch.Generator(device="cuda").manual_seed(8)
+    x = torch.rand((B, N), device="cuda", generator=gen)
+    lookup = torch.randint(0, N, (L, K), device="cuda", generator=gen, dtype=torch.int64).to(torch.int32)
+    rows = torch.arange(B, device="cuda").repeat_interleave(2)
+    cols = torch.randint(0, L, (B * 2,), device="cuda", generator=gen)
+    y = (torch.stack([rows, cols], dim=1), None)
+    loss_fn = ffi.SparseSquaredHingeLoss()
+    grads = []
+    for fused in (False, True):
+        w = ((torch.arange(L * K, device="cuda", dtype=torch.float32).reshape(L, K) % 11) / 40 - 0.12).requires_grad_(True)
+        bias = torch.full((L,), -1.2, device="cuda", requires_grad=True)
+        xin = x.clone().requires_grad_(True)
+        loss = loss_fn.fused(xin, lookup, w, bias, y)[0] if fused else loss_fn(y, ffi.fan_in_sparse_matmul_bias(xin, lookup, w, bias))
+        loss.backward()
+        torch.cuda.synchronize()
+        grads.append((w.grad.cpu().numpy(), bias.grad.cpu().numpy(), xin.grad.cpu().numpy()))
+    for a, b in zip(grads[1], grads[0]):
+        assert rel_err(a, b) <= GRAD_RTOL
