@@ -27,7 +27,8 @@ from .fixed_fan_in_ops import (  # noqa: E402
     arrange_connections,
     backward_sparse,
 )
-from . import custom_layer, metrics  # noqa: E402
+from . import custom_layer, metrics, optimizer  # noqa: E402
+from .optimizer import SparseAdam  # noqa: E402
 from .metrics import (  # noqa: E402
     SparseHingeLoss,
     SparseSquaredHingeLoss,
@@ -57,4 +58,5 @@ __all__ = [
     "SparseSquaredHingeLoss",
     "SparseBinaryCrossEntropyLoss",
     "PrecisionAtK",
+    "SparseAdam",
 ]

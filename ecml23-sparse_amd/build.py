@@ -28,6 +28,7 @@ SOURCES = [
     "ffi_bf16.hip",
     "ffi_loss.hip",
     "ffi_sparse_grad.hip",
+    "ffi_optimizer.hip",
 ]
 
 # gfx950 only.  Packed-fp32 VALU forms are switched off for all device code.

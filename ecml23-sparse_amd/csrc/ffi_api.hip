@@ -299,6 +299,15 @@ int ffi_backward_sparse_f32(const float* features, const int32_t* lookup, const 
     return input_grad_cached(lookup, weights, out_grad, feature_grad, d, s, wgrad);
 }
 
+int ffi_adam_step_f32(float* variable, float* m, float* v, const float* gradient, int64_t count, float learning_rate,
+                      float beta_1, float beta_2, float epsilon, int64_t step, ffi_stream_t stream) {
+    if (!variable || !m || !v || !gradient) return FFI_ERR_NULL_POINTER;
+    if (count <= 0) return FFI_ERR_BAD_SHAPE;
+    if (step < 1) return FFI_ERR_BAD_ARGUMENT;
+    return launch_adam_step(variable, m, v, gradient, (size_t)count, learning_rate, beta_1, beta_2, epsilon, (long long)step,
+                            (hipStream_t)stream);
+}
+
 int ffi_plan_create(const int32_t* lookup, int64_t num_units, int64_t fan_in, int64_t num_features,
                     int64_t batch_hint, ffi_stream_t stream, ffi_plan** plan) {
     if (!lookup || !plan) return FFI_ERR_NULL_POINTER;

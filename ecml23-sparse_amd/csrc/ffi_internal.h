@@ -107,6 +107,11 @@ bool sparse_input_grad_fits(int N, int K);
 int launch_input_grad_sparse(const int32_t* idx, const float* w, const float* g, const unsigned* words, float* gx,
                              const Dims& d, hipStream_t s);
 
+// ---- optimizer (ffi_optimizer.hip) ---------------------------------------------------------------
+// one Adam step (Keras' update rule) on `count` float32 variables; arrays 16-byte aligned; step is 1-based
+int launch_adam_step(float* var, float* m, float* v, const float* g, size_t count, float lr, float beta_1, float beta_2,
+                     float eps, long long step, hipStream_t s);
+
 }  // namespace ffi
 
 // Column-ordered view of one lookup matrix, in one of two forms.

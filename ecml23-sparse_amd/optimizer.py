@@ -1,0 +1,68 @@
+"""The optimizer of the reference's training loop: ``SparseAdam`` (sparse/optimizer.py:9-23), a Keras
+Adam that also resets its moments where a sparse layer rewires.
+
+The update of every float32 parameter is one pass of ``ffi_adam_step_f32`` in libffi_hip.so (Keras'
+update rule, with its defaults ``beta_1=0.9, beta_2=0.999, epsilon=1e-7``); torch holds the tensors.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from .fixed_fan_in_ops import _stream_handle
+
+
+def adam_step(variable, m, v, gradient, learning_rate, beta_1, beta_2, epsilon, step):
+    """One in-place Adam step on contiguous float32 device tensors of equal size; ``step`` counts from 1."""
+    for name, t in (("variable", variable), ("m", m), ("v", v), ("gradient", gradient)):
+        if t.dtype != torch.float32 or not t.is_cuda or not t.is_contiguous():
+            raise TypeError(f"{name} must be a contiguous float32 device tensor")
+        if t.numel() != variable.numel():
+            raise ValueError(f"{name} has {t.numel()} elements, variable has {variable.numel()}")
+    with torch.cuda.device(variable.device):
+        _lib.check(_lib.lib().ffi_adam_step_f32(variable.data_ptr(), m.data_ptr(), v.data_ptr(), gradient.data_ptr(),
+                                                variable.numel(), float(learning_rate), float(beta_1), float(beta_2),
+                                                float(epsilon), int(step), _stream_handle(variable.device)))
+
+
+class SparseAdam:
+    """``SparseAdam(params, learning_rate, update_moments=True)``; ``step()`` applies the gradients
+    held in ``param.grad`` (Keras' ``apply_gradients``), ``update_sparse(layer)`` rewires a layer and
+    clears the moments of the rewired connections (sparse/optimizer.py:14-23)."""
+
+    def __init__(self, params, learning_rate=0.001, beta_1=0.9, beta_2=0.999, epsilon=1e-7, update_moments=True):
+        self.params = list(params)
+        self.learning_rate = float(learning_rate)
+        self.beta_1, self.beta_2, self.epsilon = float(beta_1), float(beta_2), float(epsilon)
+        self.update_moments = bool(update_moments)
+        self.iterations = 0
+        self._momentums = [torch.zeros_like(p.data) for p in self.params]
+        self._velocities = [torch.zeros_like(p.data) for p in self.params]
+
+    def zero_grad(self):
+        for p in self.params:
+            p.grad = None
+
+    @torch.no_grad()
+    def step(self):
+        self.iterations += 1
+        for p, m, v in zip(self.params, self._momentums, self._velocities):
+            if p.grad is None:
+                continue
+            adam_step(p.data, m, v, p.grad.contiguous(), self.learning_rate, self.beta_1, self.beta_2, self.epsilon,
+                      self.iterations)
+
+    def _index_of(self, variable):
+        for i, p in enumerate(self.params):
+            if p is variable:
+                return i
+        raise KeyError("the variable is not one of this optimizer's parameters")
+
+    def update_sparse(self, layer):
+        if self.update_moments:
+            i = self._index_of(layer.kernel_weights)
+            new_m, new_v = layer.rewire([self._momentums[i], self._velocities[i]])
+            self._momentums[i].copy_(new_m)
+            self._velocities[i].copy_(new_v)
+        else:
+            layer.rewire(None)

@@ -243,6 +243,20 @@ int ffi_backward_sparse_f32(const float* features, const int32_t* lookup, const 
                             int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in,
                             int transposed, ffi_stream_t stream);
 
+/*
+ * One Adam step on `count` float32 variables (weights [num_units * fan_in], or the bias), the
+ * optimizer the reference trains the layer with: SparseAdam (sparse/optimizer.py:9-23) is a
+ * keras.optimizers.Adam (run.py:126) and this is that class's update rule,
+ *   alpha = learning_rate * sqrt(1 - beta_2^step) / (1 - beta_1^step)
+ *   m += (gradient - m) * (1 - beta_1);   v += (gradient^2 - v) * (1 - beta_2)
+ *   variable -= (m * alpha) / (sqrt(v) + epsilon)
+ * with `step` counted from 1.  variable, m and v are updated in place; all four arrays must be
+ * 16-byte aligned.  Keras' defaults: beta_1 0.9, beta_2 0.999, epsilon 1e-7.
+ */
+int ffi_adam_step_f32(float* variable, float* m, float* v, const float* gradient, int64_t count,
+                      float learning_rate, float beta_1, float beta_2, float epsilon, int64_t step,
+                      ffi_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -249,3 +249,24 @@ def sparse_loss(scores, label_indices, label_values, kind):
         losses[b, j] = cwise_loss(kind, s[b, j], vals)
         grad[b, j] = cwise_loss_grad(kind, s[b, j], vals)
     return losses, grad
+
+
+# ---- Adam (numpy, float32 like the variables) -----------------------------------------------------
+def adam_step(variable, m, v, gradient, learning_rate=0.001, beta_1=0.9, beta_2=0.999, epsilon=1e-7, step=1):
+    """One step of keras.optimizers.Adam, the base class of the reference's SparseAdam
+    (sparse/optimizer.py:9-12; created in run.py:126).  TensorFlow is not part of the reference tree;
+    this restates the published update_step of that class (Keras 2.11-2.15, the generation whose
+    ``_momentums`` / ``_velocities`` / ``_index_dict`` fields sparse/optimizer.py:16-18 reads):
+        alpha = lr * sqrt(1 - beta_2^t) / (1 - beta_1^t)
+        m += (g - m) * (1 - beta_1);  v += (g^2 - v) * (1 - beta_2);  var -= (m * alpha) / (sqrt(v) + epsilon)
+    all in float32.  Returns new (variable, m, v).  PARITY UNPINNED against the reference itself (it holds
+    no optimizer test or vector); tests/test_oracle.py pins the arithmetic against the closed form of the
+    first step and against torch.optim.Adam with the epsilon rescaled to Keras' placement."""
+    f = np.float32
+    var, m, v, g = (np.asarray(a, dtype=f).copy() for a in (variable, m, v, gradient))
+    b1p, b2p = f(beta_1) ** f(step), f(beta_2) ** f(step)
+    alpha = f(learning_rate) * np.sqrt(f(1) - b2p, dtype=f) / (f(1) - b1p)
+    m += (g - m) * (f(1) - f(beta_1))
+    v += (g * g - v) * (f(1) - f(beta_2))
+    var -= (m * alpha) / (np.sqrt(v, dtype=f) + f(epsilon))
+    return var, m, v

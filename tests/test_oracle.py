@@ -283,3 +283,42 @@ def test_loss_oracle_label_list_overrides_dense_part():
     np.testing.assert_array_equal(l[~mask], dense_l[~mask])
     np.testing.assert_array_equal(g[~mask], dense_g[~mask])
     np.testing.assert_array_equal(l[mask], np.maximum(1.0 - scores[mask], 0.0) ** 2)
+
+
+# ---- Adam oracle: closed form of the first step, torch.optim.Adam with Keras' epsilon placement -----
+def test_adam_oracle_first_step_closed_form():
+    # from zero moments: m = (1-b1) g, v = (1-b2) g^2, update = lr * g / (|g| + eps / sqrt(1 - b2))
+    rng = np.random.default_rng(0)
+    w = rng.normal(size=1000).astype(np.float32)
+    g = rng.normal(size=1000).astype(np.float32)
+    var, m, v = oracle.adam_step(w, np.zeros_like(w), np.zeros_like(w), g, learning_rate=0.01, step=1)
+    np.testing.assert_allclose(m, 0.1 * g, rtol=1e-6)
+    np.testing.assert_allclose(v, 0.001 * g * g, rtol=1e-4)
+    expected = w.astype(np.float64) - 0.01 * g / (np.abs(g) + 1e-7 / np.sqrt(1 - 0.999))
+    np.testing.assert_allclose(var, expected, rtol=0, atol=2e-6)
+    # a zero gradient moves nothing on the first step
+    var, m, v = oracle.adam_step(w, np.zeros_like(w), np.zeros_like(w), np.zeros_like(w), step=1)
+    assert np.array_equal(var, w) and not m.any() and not v.any()
+
+
+def test_adam_oracle_against_torch_adam():
+    # torch divides by sqrt(v / (1 - b2^t)) + eps; Keras by sqrt(v) + eps with the bias correction in
+    # the step size: the two agree when torch is given eps / sqrt(1 - b2^t)... per step, so compare
+    # step by step, handing torch the state the oracle produced
+    import torch
+    rng = np.random.default_rng(1)
+    n, lr, eps = 500, 0.003, 1e-7
+    w = rng.normal(size=n).astype(np.float32)
+    m, v = np.zeros(n, np.float32), np.zeros(n, np.float32)
+    for t in range(1, 8):
+        g = (rng.normal(size=n) * (rng.random(n) < 0.7)).astype(np.float32)
+        p = torch.nn.Parameter(torch.from_numpy(w.astype(np.float64)))
+        opt = torch.optim.Adam([p], lr=lr, betas=(0.9, 0.999), eps=eps / np.sqrt(1 - 0.999 ** t))
+        opt.state[p] = {"step": torch.tensor(float(t - 1)), "exp_avg": torch.from_numpy(m.astype(np.float64)),
+                        "exp_avg_sq": torch.from_numpy(v.astype(np.float64))}
+        p.grad = torch.from_numpy(g.astype(np.float64))
+        opt.step()
+        w, m, v = oracle.adam_step(w, m, v, g, learning_rate=lr, epsilon=eps, step=t)
+        np.testing.assert_allclose(w, p.detach().numpy(), rtol=0, atol=3e-6)
+        np.testing.assert_allclose(m, opt.state[p]["exp_avg"].numpy(), rtol=1e-5, atol=1e-7)
+        np.testing.assert_allclose(v, opt.state[p]["exp_avg_sq"].numpy(), rtol=1e-4, atol=1e-9)
