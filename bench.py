@@ -49,6 +49,10 @@ def parse_args():
                     help="reorder every label's connections with ffi_arrange_connections_f32 first (same connection sets)")
     ap.add_argument("--cpu-labels", type=int, default=0, help="labels in the CPU-baseline sample (0 = auto)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--train-step", type=float, default=0.0, metavar="DENSITY",
+                    help="also time one training step of the layer (forward + squared-hinge loss gradient in one kernel, "
+                         "backward over the non-zero gradients, Adam) with the bias set so that this share of the loss "
+                         "gradients is non-zero; reported under 'train_step' in the same JSON line")
     ap.add_argument("--copy-bytes", type=int, default=0,
                     help="also run one plain device copy kernel of this many bytes (read N, write N): the "
                          "known-size reference that rocprofv3 FETCH_SIZE/WRITE_SIZE readings are scaled by")
@@ -96,6 +100,71 @@ def cpu_baseline(cfg, layout_tp, labels, seed):
         "sample": f"{labels} of {cfg.num_units} labels (same B, N, K, laws); fwd+gW+gx in {best:.3f} s (best of 2)"
                   + ("" if labels == cfg.num_units else ", scaled linearly to the full label count"),
     }
+
+
+def train_step(pkg, cfg, x, lookup, w, tp, density, stream, iters):
+    """One training step as the reference's loop runs it (sparse/optimizer.py:43-66): forward + loss,
+    backward, Adam on weights and bias, with synthetic labels (5 per sample) and the bias chosen so that
+    `density` of the squared-hinge gradients are non-zero (late in training nearly every margin is met)."""
+    import ctypes
+
+    import torch
+    B, N, L, K = cfg.batch, cfg.num_features, cfg.num_units, cfg.fan_in
+    lib, check, sh = pkg._lib.lib(), pkg._lib.check, stream.cuda_stream
+    ptr = lambda a: a.data_ptr()  # noqa: E731
+    gen = torch.Generator(device="cuda").manual_seed(7)
+    scores = torch.empty((B, L), device="cuda")
+    check(lib.ffi_forward_f32(ptr(x), ptr(lookup), ptr(w), ptr(scores), B, N, L, K, int(tp), sh))
+    # a negative's gradient is non-zero where 1 + score + bias > 0
+    sample = scores.flatten()[torch.randint(0, B * L, (1 << 20,), device="cuda", generator=gen)]
+    bias = torch.full((L,), -1.0 - float(torch.quantile(sample, 1.0 - density)), device="cuda")
+    rows = torch.arange(B, device="cuda").repeat_interleave(5)
+    labels = torch.stack([rows, torch.randint(0, L, (B * 5,), device="cuda", generator=gen)], dim=1).contiguous()
+    g = torch.empty_like(scores)
+    masks = torch.empty(((B + 31) // 32, L), dtype=torch.int32, device="cuda")
+    loss = torch.empty(1, device="cuda")
+    gx, gw, gb = torch.empty_like(x), torch.empty_like(w), torch.empty_like(bias)
+    mw, vw, mb, vb = torch.zeros_like(w), torch.zeros_like(w), torch.zeros_like(bias), torch.zeros_like(bias)
+    w2, bias2 = w.clone(), bias.clone()              # Adam runs on copies: every timed step sees the same scores
+    scale = ctypes.c_float(1.0 / (B * L))
+    taken = ctypes.c_int(-1)
+    SQH = 2
+
+    def fused_forward_loss():
+        check(lib.ffi_forward_loss_f32(ptr(x), ptr(lookup), ptr(w), ptr(bias), ptr(labels), None, labels.shape[0], SQH, scale,
+                                       None, ptr(g), ptr(loss), ptr(masks), B, N, L, K, int(tp), sh))
+
+    def backward_sparse():
+        check(lib.ffi_backward_sparse_f32(ptr(x), ptr(lookup), ptr(w), ptr(g), ptr(masks), ctypes.c_float(0.0), ptr(gx), ptr(gw),
+                                          ptr(gb), ctypes.byref(taken), B, N, L, K, int(tp), sh))
+
+    def adam():
+        check(lib.ffi_adam_step_f32(ptr(w2), ptr(mw), ptr(vw), ptr(gw), L * K, 1e-3, 0.9, 0.999, 1e-7, 1, sh))
+        check(lib.ffi_adam_step_f32(ptr(bias2), ptr(mb), ptr(vb), ptr(gb), L, 1e-3, 0.9, 0.999, 1e-7, 1, sh))
+
+    def unfused_forward_loss():
+        check(lib.ffi_forward_bias_f32(ptr(x), ptr(lookup), ptr(w), ptr(bias), ptr(scores), B, N, L, K, int(tp), sh))
+        check(lib.ffi_loss_grad_f32(ptr(scores), ptr(labels), None, labels.shape[0], SQH, scale, ptr(g), ptr(loss), None, B, L, sh))
+
+    def backward_dense():
+        check(lib.ffi_backward_bias_f32(ptr(x), ptr(lookup), ptr(w), ptr(g), ptr(gx), ptr(gw), ptr(gb), B, N, L, K, int(tp), sh))
+
+    def whole():
+        fused_forward_loss()
+        backward_sparse()
+        adam()
+
+    out = {"loss": "squared hinge, 5 labels per sample", "target_density": density}
+    out["forward_loss_ms"] = round(time_kernel(fused_forward_loss, stream, iters), 4)
+    out["gradient_density"] = round(float((g != 0).float().mean()), 6)
+    out["backward_sparse_ms"] = round(time_kernel(backward_sparse, stream, iters), 4)
+    out["sparse_kernels_ran"] = bool(taken.value)
+    out["adam_ms"] = round(time_kernel(adam, stream, iters), 4)
+    out["step_ms"] = round(time_kernel(whole, stream, iters), 4)
+    out["samples_per_s"] = round(B / (out["step_ms"] * 1e-3), 1)
+    out["unfused_dense_route_ms"] = {"forward_bias+loss_grad": round(time_kernel(unfused_forward_loss, stream, iters), 4),
+                                     "backward_dense": round(time_kernel(backward_dense, stream, iters), 4)}
+    return out
 
 
 def main():
@@ -202,6 +271,8 @@ def main():
                    "label_samples_per_s": round(B * L / (ms_per_step * 1e-3), 1)},
         "roofline": roofline,
     }
+    if args.train_step > 0:
+        result["train_step"] = train_step(pkg, cfg, x, lookup, w, tp, args.train_step, stream, max(3, min(args.steps, 20)))
     if not args.no_cpu_baseline:
         labels = args.cpu_labels or max(4096, min(L, int(8.0e9 / (B * K))))
         result["cpu_baseline"] = cpu_baseline(cfg, tp, min(labels, L), args.seed)

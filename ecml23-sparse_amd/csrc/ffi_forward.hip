@@ -48,6 +48,35 @@ struct FwdLoss {
     int kind;
 };
 
+// Scores of one label for the 32 samples of a batch tile -> scaled loss gradients (in place), the sum of the
+// losses of the first `nrows` samples, and the mask of the non-zero gradients among them.
+template <int KIND>
+__device__ __forceinline__ void loss_epilogue(float (&acc)[32], int nrows, float scale, float& loss, unsigned& mask) {
+    float l = 0.f;
+    unsigned m = 0;
+    if (nrows == 32) {
+#pragma unroll
+        for (int b = 0; b < 32; ++b) {
+            float lb, gb;
+            cwise_loss_and_grad(KIND, acc[b], 0.f, lb, gb);
+            l += lb;
+            m |= (gb != 0.f ? 1u : 0u) << b;
+            acc[b] = scale * gb;
+        }
+    } else {                               // last batch tile: rows past the batch count for nothing
+#pragma unroll
+        for (int b = 0; b < 32; ++b) {
+            float lb, gb;
+            cwise_loss_and_grad(KIND, acc[b], 0.f, lb, gb);
+            l += b < nrows ? lb : 0.f;
+            m |= (b < nrows && gb != 0.f ? 1u : 0u) << b;
+            acc[b] = scale * gb;
+        }
+    }
+    loss = l;
+    mask = m;
+}
+
 template <bool VEC4, int EPI>
 __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* __restrict__ xT,
                                                                   const int32_t* __restrict__ idx,
@@ -138,24 +167,17 @@ __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* _
         }
         if (EPI != kEpiScores) {
             float l = 0.f;
-#pragma unroll
-            for (int b = 0; b < 32; ++b) {
-                float lb, gb;
-                cwise_loss_and_grad(fl.kind, acc[b], 0.f, lb, gb);
-                l += b < nrows ? lb : 0.f;
-                acc[b] = fl.scale * gb;
-            }
+            unsigned m = 0;
+            // the loss kind is the same for the whole launch: one straight-line epilogue per kind
+            if (fl.kind == FFI_LOSS_SQUARED_HINGE) loss_epilogue<FFI_LOSS_SQUARED_HINGE>(acc, nrows, fl.scale, l, m);
+            else if (fl.kind == FFI_LOSS_HINGE) loss_epilogue<FFI_LOSS_HINGE>(acc, nrows, fl.scale, l, m);
+            else loss_epilogue<FFI_LOSS_BCE>(acc, nrows, fl.scale, l, m);
             if (valid) {
                 lsum += l;
 #pragma unroll
                 for (int b = 0; b < 32; ++b)
                     __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, acc[b]), EPI == kEpiLossGrad ? orsrc : grsrc, lane_off, (unsigned)b * stride, 0);
-                if (fl.words != nullptr) {
-                    unsigned m = 0;
-#pragma unroll
-                    for (int b = 0; b < 32; ++b) m |= (b < nrows && acc[b] != 0.f ? 1u : 0u) << b;
-                    fl.words[(size_t)bt * L + j] = m;
-                }
+                if (fl.words != nullptr) fl.words[(size_t)bt * L + j] = m;
             }
         }
     }

@@ -66,13 +66,14 @@ __global__ __launch_bounds__(kLossThreads) void loss_gather_kernel(const int64_t
     saved[p] = (b >= 0 && b < B && j >= 0 && j < L) ? scores[(size_t)b * L + j] : 0.f;
 }
 
-// One thread per listed label position.  x is addressed as x[b * xsb + n * xsn] (either layout).
+// One wavefront per listed label position.  x is addressed as x[b * xsb + n * xsn] (either layout).
 __global__ __launch_bounds__(kLossThreads) void loss_positive_kernel(
     const int64_t* __restrict__ label_indices, const float* __restrict__ label_values, int nnz,
     const float* __restrict__ saved, const float* __restrict__ scores, const float* __restrict__ x, size_t xsb, size_t xsn,
     const int32_t* __restrict__ idx, const float* __restrict__ w, const float* __restrict__ bias, float* __restrict__ g,
     float scale, int kind, int B, int N, int L, int K, double* __restrict__ corr, unsigned* __restrict__ nz_words) {
-    const int p = blockIdx.x * kLossThreads + threadIdx.x;
+    const int lane = threadIdx.x & 63;
+    const int p = blockIdx.x * (kLossThreads / 64) + (threadIdx.x >> 6);
     if (p >= nnz) return;
     const int64_t b = label_indices[2 * (size_t)p], j = label_indices[2 * (size_t)p + 1];
     double c = 0.0;
@@ -83,40 +84,48 @@ __global__ __launch_bounds__(kLossThreads) void loss_positive_kernel(
         } else if (scores != nullptr) {
             s = scores[(size_t)b * L + j];
         } else {
-            // the same sum the forward kernel forms: ascending k, fused multiply-adds, bias last
-            s = 0.f;
-            for (int k = 0; k < K; ++k) {
+            // the score was never written: recompute it from the label's row, lane <-> connection
+            // (a different summation order than the forward kernel's, the same value up to rounding)
+            float part = 0.f;
+            for (int k = lane; k < K; k += 64) {
                 const unsigned id = (unsigned)idx[(size_t)j * K + k];
-                s = fmaf(w[(size_t)j * K + k], x[(size_t)b * xsb + (size_t)(id < (unsigned)N ? id : 0u) * xsn], s);
+                part = fmaf(w[(size_t)j * K + k], x[(size_t)b * xsb + (size_t)(id < (unsigned)N ? id : 0u) * xsn], part);
             }
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
+            s = part;
             if (bias != nullptr) s += bias[j];
         }
         const float y = label_values ? label_values[p] : 1.f;
         const float gv = scale * cwise_loss_grad(kind, s, y);
-        g[(size_t)b * L + j] = gv;
-        // the bulk pass set this position's mask bit from its gradient as a negative; a set bit over a zero is harmless
-        if (nz_words != nullptr && gv != 0.f) atomicOr(&nz_words[(size_t)(b >> 5) * L + j], 1u << (b & 31));
         // minus what the bulk pass charged this position as a negative (the same arithmetic as there)
         float l0, g0;
         cwise_loss_and_grad<false>(kind, s, 0.f, l0, g0);
         c = (double)cwise_loss(kind, s, y) - (double)l0;
+        if (lane == 0) {
+            g[(size_t)b * L + j] = gv;
+            // the bulk pass set this position's mask bit from its gradient as a negative; a set bit over a zero is harmless
+            if (nz_words != nullptr && gv != 0.f) atomicOr(&nz_words[(size_t)(b >> 5) * L + j], 1u << (b & 31));
+        }
     }
-    corr[p] = c;
+    if (lane == 0) corr[p] = c;
 }
 
-__global__ __launch_bounds__(kLossThreads) void loss_finish_kernel(const double* __restrict__ partial, int npartial,
-                                                                   const double* __restrict__ corr, int ncorr,
-                                                                   float* __restrict__ loss_sum) {
-    __shared__ double red[kLossThreads / 64];
+constexpr int kFinishThreads = 1024;
+
+__global__ __launch_bounds__(kFinishThreads) void loss_finish_kernel(const double* __restrict__ partial, int npartial,
+                                                                     const double* __restrict__ corr, int ncorr,
+                                                                     float* __restrict__ loss_sum) {
+    __shared__ double red[kFinishThreads / 64];
     double a = 0.0;
-    for (int i = threadIdx.x; i < npartial; i += kLossThreads) a += partial[i];
-    for (int i = threadIdx.x; i < ncorr; i += kLossThreads) a += corr[i];
+    for (int i = threadIdx.x; i < npartial; i += kFinishThreads) a += partial[i];
+    for (int i = threadIdx.x; i < ncorr; i += kFinishThreads) a += corr[i];
     a = wave_sum(a);
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = a;
     __syncthreads();
     if (threadIdx.x == 0) {
         double t = 0.0;
-        for (int i = 0; i < kLossThreads / 64; ++i) t += red[i];
+        for (int i = 0; i < kFinishThreads / 64; ++i) t += red[i];
         *loss_sum = (float)t;
     }
 }
@@ -137,13 +146,13 @@ int launch_loss_positives(const LossArgs& la, const float* saved, const float* s
                           hipStream_t s) {
     if (la.nnz > 0) {
         const size_t xsb = d.tp ? 1 : (size_t)d.N, xsn = d.tp ? (size_t)d.B : 1;
-        hipLaunchKernelGGL(loss_positive_kernel, dim3((la.nnz + kLossThreads - 1) / kLossThreads), dim3(kLossThreads), 0, s,
+        hipLaunchKernelGGL(loss_positive_kernel, dim3((la.nnz + kLossThreads / 64 - 1) / (kLossThreads / 64)), dim3(kLossThreads), 0, s,
                            la.indices, la.values, la.nnz, saved, scores, x, xsb, xsn, idx, w, bias, g, la.scale, la.kind, d.B, d.N,
                            d.L, d.K, corr, la.nz_words);
         FFI_HIP_TRY(hipGetLastError());
     }
     if (la.loss_sum != nullptr) {
-        hipLaunchKernelGGL(loss_finish_kernel, dim3(1), dim3(kLossThreads), 0, s, partial, npartial, corr, la.nnz, la.loss_sum);
+        hipLaunchKernelGGL(loss_finish_kernel, dim3(1), dim3(kFinishThreads), 0, s, partial, npartial, corr, la.nnz, la.loss_sum);
         FFI_HIP_TRY(hipGetLastError());
     }
     return FFI_OK;

@@ -59,7 +59,7 @@ def call_loss_grad(ffi, scores_t, indices, values, kind, scale, in_place=False):
     loss = torch.full((1,), float("nan"), device="cuda")
     ffi._lib.check(lib.ffi_loss_grad_f32(scores_t.data_ptr(), idx_t.data_ptr() if idx_t is not None else None,
                                          val_t.data_ptr() if val_t is not None else None, len(indices), kind,
-                                         ctypes.c_float(scale), g.data_ptr(), loss.data_ptr(), B, L,
+                                         ctypes.c_float(scale), g.data_ptr(), loss.data_ptr(), None, B, L,
                                          torch.cuda.current_stream().cuda_stream))
     torch.cuda.synchronize()
     return g.cpu().numpy(), float(loss.cpu()[0])
@@ -117,14 +117,14 @@ def test_loss_grad_argument_errors(ffi):
     g = torch.zeros_like(s)
     sh = torch.cuda.current_stream().cuda_stream
     one = ctypes.c_float(1.0)
-    assert lib.ffi_loss_grad_f32(None, None, None, 0, 2, one, g.data_ptr(), None, 4, 8, sh) == -1
-    assert lib.ffi_loss_grad_f32(s.data_ptr(), None, None, 3, 2, one, g.data_ptr(), None, 4, 8, sh) == -1   # nnz without a list
-    assert lib.ffi_loss_grad_f32(s.data_ptr(), None, None, 0, 7, one, g.data_ptr(), None, 4, 8, sh) == -8   # unknown loss
-    assert lib.ffi_loss_grad_f32(s.data_ptr(), None, None, 0, 2, one, g.data_ptr(), None, 0, 8, sh) == -2
-    assert lib.ffi_loss_grad_f32(s.data_ptr(), None, None, -1, 2, one, g.data_ptr(), None, 4, 8, sh) == -2
-    assert lib.ffi_loss_grad_f32(s.data_ptr(), None, None, 0, 2, one, g.data_ptr(), None, 4, 8, sh) == 0    # loss_sum may be NULL
+    assert lib.ffi_loss_grad_f32(None, None, None, 0, 2, one, g.data_ptr(), None, None, 4, 8, sh) == -1
+    assert lib.ffi_loss_grad_f32(s.data_ptr(), None, None, 3, 2, one, g.data_ptr(), None, None, 4, 8, sh) == -1   # nnz without a list
+    assert lib.ffi_loss_grad_f32(s.data_ptr(), None, None, 0, 7, one, g.data_ptr(), None, None, 4, 8, sh) == -8   # unknown loss
+    assert lib.ffi_loss_grad_f32(s.data_ptr(), None, None, 0, 2, one, g.data_ptr(), None, None, 0, 8, sh) == -2
+    assert lib.ffi_loss_grad_f32(s.data_ptr(), None, None, -1, 2, one, g.data_ptr(), None, None, 4, 8, sh) == -2
+    assert lib.ffi_loss_grad_f32(s.data_ptr(), None, None, 0, 2, one, g.data_ptr(), None, None, 4, 8, sh) == 0    # loss_sum may be NULL
     f = lib.ffi_forward_loss_f32
-    assert f(s.data_ptr(), s.data_ptr(), s.data_ptr(), None, None, None, 0, 2, one, g.data_ptr(), g.data_ptr(), None,
+    assert f(s.data_ptr(), s.data_ptr(), s.data_ptr(), None, None, None, 0, 2, one, g.data_ptr(), g.data_ptr(), None, None,
              4, 8, 4, 2, 0, sh) == -8                                                                        # scores == out_grad
 
 
