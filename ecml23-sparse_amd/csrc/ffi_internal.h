@@ -154,10 +154,10 @@ struct ffi_plan {
     int nblocks = 0;
     int32_t* perm = nullptr;
     int32_t* col_ptr = nullptr;
-    unsigned long long* d_scratch = nullptr;  // fingerprint / counters (device)
+    unsigned long long* d_scratch = nullptr;  // counters of the build, fingerprint partial sums (device)
     unsigned long long* h_scratch = nullptr;  // pinned mirror
     hipEvent_t fp_done = nullptr;             // recorded behind the fingerprint kernel and its copy to h_scratch
-    int fp_slot = 0;                          // which pair of d_scratch words the next fingerprint adds into (0: [0,1], 1: [4,5])
+    int fp_blocks = 0;                        // workgroups of the fingerprint kernel in flight: that many pairs of partial sums
     size_t bytes = 0;
 };
 

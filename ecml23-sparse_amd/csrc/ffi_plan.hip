@@ -16,6 +16,8 @@ namespace ffi {
 namespace {
 
 constexpr int kBlock = 256;
+constexpr int kFingerprintBlocks = 1024;                 // workgroups of the fingerprint kernel (at most)
+constexpr int kScratchWords = 8 + 2 * kFingerprintBlocks;  // plan scratch: 8 words for the build, then fingerprint partial sums
 
 __device__ __forceinline__ unsigned mix32(unsigned v) {
     v ^= v >> 16; v *= 0x7feb352du;
@@ -25,12 +27,12 @@ __device__ __forceinline__ unsigned mix32(unsigned v) {
 }
 
 // Order-independent 64-bit content fingerprint: sum over positions p of mix(id_p + p * odd), plus
-// the number of ids outside [0,N).  Integer adds only, so the value does not depend on the order
-// of the atomics.  Four ids per load when the array allows it.
+// the number of ids outside [0,N).  Every workgroup writes its own pair of partial sums (no atomics:
+// thousands of adds to one address serialise); the host adds them up.  Four ids per load when the
+// array allows it.
 __global__ __launch_bounds__(kBlock) void fingerprint_kernel(const int32_t* __restrict__ idx,
                                                               size_t total, unsigned N,
-                                                              unsigned long long* __restrict__ out,
-                                                              unsigned long long* __restrict__ out_next) {
+                                                              unsigned long long* __restrict__ out) {
     unsigned long long h = 0;
     unsigned bad = 0;
     const size_t stride = (size_t)gridDim.x * kBlock;
@@ -38,6 +40,7 @@ __global__ __launch_bounds__(kBlock) void fingerprint_kernel(const int32_t* __re
     const bool vec = ((uintptr_t)idx & 15) == 0;
     const size_t nvec = vec ? total / 4 : 0;
     const int4* idx4 = reinterpret_cast<const int4*>(idx);
+#pragma unroll 4
     for (size_t q = tid; q < nvec; q += stride) {
         const int4 v = idx4[q];
         const unsigned p = (unsigned)(q * 4);
@@ -58,7 +61,6 @@ __global__ __launch_bounds__(kBlock) void fingerprint_kernel(const int32_t* __re
         h += __shfl_down(h, off);
         b64 += __shfl_down(b64, off);
     }
-    // one pair of atomics per workgroup: thousands of wavefronts adding to one address serialise
     __shared__ unsigned long long part[2][kBlock / 64];
     if ((threadIdx.x & 63) == 0) { part[0][threadIdx.x >> 6] = h; part[1][threadIdx.x >> 6] = b64; }
     __syncthreads();
@@ -66,10 +68,8 @@ __global__ __launch_bounds__(kBlock) void fingerprint_kernel(const int32_t* __re
         unsigned long long hs = 0, bs = 0;
 #pragma unroll
         for (int i = 0; i < kBlock / 64; ++i) { hs += part[0][i]; bs += part[1][i]; }
-        atomicAdd(&out[0], hs);
-        if (bs) atomicAdd(&out[1], bs);
-        // the words the next call will add into (calls alternate between two pairs) start from zero
-        if (blockIdx.x == 0) { out_next[0] = 0; out_next[1] = 0; }
+        out[2 * blockIdx.x] = hs;
+        out[2 * blockIdx.x + 1] = bs;
     }
 }
 
@@ -417,10 +417,10 @@ int build_arranged(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
 
 // device/pinned scratch words and the fingerprint event of a plan
 int plan_scratch_alloc(ffi_plan* p) {
-    const bool ok = hipMalloc(&p->d_scratch, 8 * sizeof(unsigned long long)) == hipSuccess &&
-                    hipHostMalloc(&p->h_scratch, 8 * sizeof(unsigned long long)) == hipSuccess &&
+    const bool ok = hipMalloc(&p->d_scratch, kScratchWords * sizeof(unsigned long long)) == hipSuccess &&
+                    hipHostMalloc(&p->h_scratch, kScratchWords * sizeof(unsigned long long)) == hipSuccess &&
                     hipEventCreateWithFlags(&p->fp_done, hipEventDisableTiming) == hipSuccess &&
-                    hipMemset(p->d_scratch, 0, 8 * sizeof(unsigned long long)) == hipSuccess;
+                    hipMemset(p->d_scratch, 0, kScratchWords * sizeof(unsigned long long)) == hipSuccess;
     if (!ok) {
         (void)hipGetLastError();
         return FFI_ERR_OUT_OF_MEMORY;
@@ -430,21 +430,26 @@ int plan_scratch_alloc(ffi_plan* p) {
 
 int plan_fingerprint_begin(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     const size_t total = (size_t)p->L * p->K;
-    const unsigned blocks = (unsigned)std::min<size_t>((total / 4 + kBlock - 1) / kBlock + 1, 2048);
-    unsigned long long* cur = p->d_scratch + (p->fp_slot ? 4 : 0);
-    unsigned long long* next = p->d_scratch + (p->fp_slot ? 0 : 4);
-    p->fp_slot ^= 1;
-    hipLaunchKernelGGL(fingerprint_kernel, dim3(blocks), dim3(kBlock), 0, s, lookup, total, (unsigned)p->N, cur, next);
+    const unsigned blocks = (unsigned)std::min<size_t>((total / 4 + kBlock - 1) / kBlock + 1, kFingerprintBlocks);
+    // words 0..7 of the scratch arrays belong to the plan build; the workgroups' partial sums follow
+    unsigned long long* partials = p->d_scratch + 8;
+    hipLaunchKernelGGL(fingerprint_kernel, dim3(blocks), dim3(kBlock), 0, s, lookup, total, (unsigned)p->N, partials);
     FFI_HIP_TRY(hipGetLastError());
-    FFI_HIP_TRY(hipMemcpyAsync(p->h_scratch, cur, 2 * sizeof(unsigned long long), hipMemcpyDeviceToHost, s));
+    FFI_HIP_TRY(hipMemcpyAsync(p->h_scratch + 8, partials, 2 * (size_t)blocks * sizeof(unsigned long long), hipMemcpyDeviceToHost, s));
     FFI_HIP_TRY(hipEventRecord(p->fp_done, s));
+    p->fp_blocks = (int)blocks;
     return FFI_OK;
 }
 
 int plan_fingerprint_end(ffi_plan* p, unsigned long long* out, unsigned long long* bad_ids) {
     FFI_HIP_TRY(hipEventSynchronize(p->fp_done));
-    *out = p->h_scratch[0];
-    *bad_ids = p->h_scratch[1];
+    unsigned long long h = 0, bad = 0;
+    for (int i = 0; i < p->fp_blocks; ++i) {
+        h += p->h_scratch[8 + 2 * i];
+        bad += p->h_scratch[8 + 2 * i + 1];
+    }
+    *out = h;
+    *bad_ids = bad;
     return FFI_OK;
 }
 
