@@ -252,7 +252,7 @@ int ffi_loss_grad_f32(const float* scores, const int64_t* label_indices, const f
                       int64_t num_units, ffi_stream_t stream) {
     if (!scores || !out_grad) return FFI_ERR_NULL_POINTER;
     FFI_TRY(check_loss_args(label_indices, nnz, loss_kind, batch, num_units));
-    const LossArgs la{label_indices, label_values, (int)nnz, loss_kind, grad_scale, loss_sum, nz_words};
+    const LossArgs la{label_indices, label_values, (int)nnz, loss_kind, grad_scale, loss_sum, nz_words, false};
     return launch_loss_grad(la, scores, out_grad, (int)batch, (int)num_units, (hipStream_t)stream);
 }
 
@@ -265,18 +265,22 @@ int ffi_forward_loss_f32(const float* features, const int32_t* lookup, const flo
     if (scores == out_grad) return FFI_ERR_BAD_ARGUMENT;
     Dims d;
     FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
+    const bool skip = (loss_kind & FFI_LOSS_SKIP_ZERO_STORES) != 0;
+    loss_kind &= ~FFI_LOSS_SKIP_ZERO_STORES;
+    if (skip && !nz_words) return FFI_ERR_NULL_POINTER;
     FFI_TRY(check_loss_args(label_indices, nnz, loss_kind, batch, num_units));
-    const LossArgs la{label_indices, label_values, (int)nnz, loss_kind, grad_scale, loss_sum, nz_words};
+    const LossArgs la{label_indices, label_values, (int)nnz, loss_kind, grad_scale, loss_sum, nz_words, skip};
     return launch_forward_loss(features, lookup, weights, bias, la, scores, out_grad, d, (hipStream_t)stream);
 }
 
-int ffi_backward_sparse_f32(const float* features, const int32_t* lookup, const float* weights, const float* out_grad,
-                            const uint32_t* nz_words, float max_density, float* feature_grad, float* weight_grad,
+int ffi_backward_sparse_f32(const float* features, const int32_t* lookup, const float* weights, float* out_grad,
+                            const uint32_t* nz_words, int grad_is_partial, float max_density, float* feature_grad, float* weight_grad,
                             float* bias_grad, int* sparse_path_taken, int64_t batch, int64_t num_features,
                             int64_t num_units, int64_t fan_in, int transposed, ffi_stream_t stream) {
     if (!features || !lookup || !weights || !out_grad) return FFI_ERR_NULL_POINTER;
     if (!feature_grad && !weight_grad) return FFI_ERR_NULL_POINTER;
     if (bias_grad && !weight_grad) return FFI_ERR_NULL_POINTER;
+    if (grad_is_partial && !nz_words) return FFI_ERR_NULL_POINTER;
     Dims d;
     FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
     hipStream_t s = (hipStream_t)stream;
@@ -286,6 +290,8 @@ int ffi_backward_sparse_f32(const float* features, const int32_t* lookup, const 
     const double limit = (double)(max_density > 0.f ? max_density : kSparseDefaultMaxDensity) * (double)d.B * (double)d.L;
     const bool sparse = (double)set_bits <= limit;
     if (sparse_path_taken) *sparse_path_taken = sparse ? 1 : 0;
+    // the dense kernels read all of out_grad
+    if (!sparse && grad_is_partial) FFI_TRY(launch_zero_unmasked(out_grad, words, d.B, d.L, s));
     auto wgrad = [&](const ffi_plan* plan) {
         if (!weight_grad) return (int)FFI_OK;
         if (sparse) return launch_weight_grad_sparse(features, lookup, out_grad, words, weight_grad, bias_grad, d, s);

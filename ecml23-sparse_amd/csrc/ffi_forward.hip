@@ -46,6 +46,7 @@ struct FwdLoss {
     unsigned* words;    // [ceil(B/32)][L] masks of the non-zero gradients to fill in, or null
     float scale;
     int kind;
+    int skip_zero_stores;   // != 0: gradients that are exactly zero are not stored (needs words)
 };
 
 // Scores of one label for the 32 samples of a batch tile -> scaled loss gradients (in place), the sum of the
@@ -174,9 +175,16 @@ __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* _
             else loss_epilogue<FFI_LOSS_BCE>(acc, nrows, fl.scale, l, m);
             if (valid) {
                 lsum += l;
+                if (fl.skip_zero_stores) {
 #pragma unroll
-                for (int b = 0; b < 32; ++b)
-                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, acc[b]), EPI == kEpiLossGrad ? orsrc : grsrc, lane_off, (unsigned)b * stride, 0);
+                    for (int b = 0; b < 32; ++b)
+                        if ((m >> b) & 1u)
+                            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, acc[b]), EPI == kEpiLossGrad ? orsrc : grsrc, lane_off, (unsigned)b * stride, 0);
+                } else {
+#pragma unroll
+                    for (int b = 0; b < 32; ++b)
+                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, acc[b]), EPI == kEpiLossGrad ? orsrc : grsrc, lane_off, (unsigned)b * stride, 0);
+                }
                 if (fl.words != nullptr) fl.words[(size_t)bt * L + j] = m;
             }
         }
@@ -219,7 +227,7 @@ int forward_tiles(const float* x, const int32_t* idx, const float* w, const floa
     const int per_stream = (d.L + streams - 1) / streams;
     streams = (d.L + per_stream - 1) / per_stream;
     const int blocks = streams * nbt;
-    FwdLoss fl{gout, nullptr, nullptr, 0.f, 0};
+    FwdLoss fl{gout, nullptr, nullptr, 0.f, 0, 0};
     if (epi == kEpiScores)
         return vec4 ? launch_lane32<true, kEpiScores>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, s)
                     : launch_lane32<false, kEpiScores>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, s);
@@ -229,6 +237,7 @@ int forward_tiles(const float* x, const int32_t* idx, const float* w, const floa
     fl.scale = la->scale;
     fl.kind = la->kind;
     fl.words = la->nz_words;
+    fl.skip_zero_stores = la->skip_zero_stores ? 1 : 0;
     if (epi == kEpiLossGrad) {
         FFI_TRY(vec4 ? (launch_lane32<true, kEpiLossGrad>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, s))
                      : (launch_lane32<false, kEpiLossGrad>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, s)));

@@ -77,6 +77,7 @@ struct LossArgs {
     float scale;              // factor on the gradient
     float* loss_sum;          // device float or null
     unsigned* nz_words;       // [ceil(B/32)][L] non-zero masks of the gradient to fill in, or null
+    bool skip_zero_stores;    // leave out the stores of zero gradients (fused forward kernel only; needs nz_words)
 };
 // partial[npartial] loss sums, corr[nnz] loss corrections and saved[nnz] scores of the listed positions
 int loss_partial_buffer(hipStream_t s, int npartial, int nnz, double** partial, double** corr, float** saved);
@@ -104,6 +105,8 @@ int nonzero_count(const float* g, const unsigned* given_words, int B, int L, hip
 int launch_weight_grad_sparse(const float* x, const int32_t* idx, const float* g, const unsigned* words, float* gw,
                               float* bias_grad, const Dims& d, hipStream_t s);
 bool sparse_input_grad_fits(int N, int K);
+// g[b,j] = 0 wherever the mask bit of (b,j) is clear
+int launch_zero_unmasked(float* g, const unsigned* words, int B, int L, hipStream_t s);
 int launch_input_grad_sparse(const int32_t* idx, const float* w, const float* g, const unsigned* words, float* gx,
                              const Dims& d, hipStream_t s);
 

@@ -52,6 +52,20 @@ __global__ __launch_bounds__(kScanThreads) void nz_scan_kernel(const float* __re
     }
 }
 
+// g[32 t + i, j] = 0 wherever bit i of words[t][j] is clear (thread <-> label, rows written 256 bytes per wavefront).
+__global__ __launch_bounds__(kScanThreads) void nz_zero_unmasked_kernel(float* __restrict__ g, const unsigned* __restrict__ words,
+                                                                        int B, int L) {
+    const int j = blockIdx.x * kScanThreads + threadIdx.x;
+    const int t = blockIdx.y;
+    if (j >= L) return;
+    const int rows = min(32, B - 32 * t);
+    const unsigned m = words[(size_t)t * L + j];
+    float* col = g + (size_t)(32 * t) * L + j;
+#pragma unroll
+    for (int i = 0; i < 32; ++i)
+        if (i < rows && !((m >> i) & 1u)) col[(size_t)i * L] = 0.f;
+}
+
 __global__ __launch_bounds__(kScanThreads) void nz_count_kernel(const unsigned* __restrict__ words, size_t n,
                                                                 unsigned long long* __restrict__ block_counts) {
     __shared__ unsigned red[kScanThreads / 64];
@@ -346,6 +360,14 @@ unsigned long long* g_count_host[64] = {nullptr};
 int launch_nonzero_scan(const float* g, unsigned* words, int B, int L, hipStream_t s) {
     const int nbt = (B + 31) / 32;
     hipLaunchKernelGGL(nz_scan_kernel, dim3((L + 2 * kScanThreads - 1) / (2 * kScanThreads), nbt), dim3(kScanThreads), 0, s, g, words, B, L);
+    FFI_HIP_TRY(hipGetLastError());
+    return FFI_OK;
+}
+
+int launch_zero_unmasked(float* g, const unsigned* words, int B, int L, hipStream_t s) {
+    const int nbt = (B + 31) / 32;
+    hipLaunchKernelGGL(nz_zero_unmasked_kernel, dim3((L + kScanThreads - 1) / kScanThreads, nbt), dim3(kScanThreads), 0, s, g, words,
+                       B, L);
     FFI_HIP_TRY(hipGetLastError());
     return FFI_OK;
 }

@@ -17,6 +17,7 @@ from . import _lib
 from .fixed_fan_in_ops import _check_bias, _check_inputs, _stream_handle, backward_sparse, topk_scores
 
 LOSS_HINGE, LOSS_SQUARED_HINGE, LOSS_BCE = 1, 2, 3
+SKIP_ZERO_STORES = 0x100      # flag on the loss kind of forward_loss: zero gradients are not stored
 
 
 def _labels(y_true, device):
@@ -66,14 +67,18 @@ def sparse_loss_grad(scores, y_true, kind, grad_scale=None, in_place=False, want
 
 
 def forward_loss(features, lookup, weights, bias, y_true, kind, grad_scale=None, transposed=False, want_scores=False,
-                 want_masks=False):
+                 want_masks=False, skip_zero_stores=False):
     """Forward pass, bias add and loss gradient in one kernel: ``(scores or None, out_grad, loss_sum)``,
-    plus the bit masks of the non-zero gradients with ``want_masks``."""
+    plus the bit masks of the non-zero gradients with ``want_masks``.  With ``skip_zero_stores`` (needs
+    ``want_masks``) ``out_grad`` is written only where its mask bit is set and is undefined elsewhere:
+    hand it to ``backward_sparse(..., grad_is_partial=True)``."""
     batch, num_features, num_units, fan_in = _check_inputs(features, lookup, weights, transposed)
     if bias is not None:
         _check_bias(bias, weights, num_units)
         bias = bias.contiguous()
     features, lookup, weights = features.contiguous(), lookup.contiguous(), weights.contiguous()
+    if skip_zero_stores and not want_masks:
+        raise ValueError("skip_zero_stores needs want_masks: the masks say which entries of out_grad were written")
     indices, values = _labels(y_true, features.device)
     scale = 1.0 / (batch * num_units) if grad_scale is None else float(grad_scale)
     with torch.cuda.device(features.device):
@@ -84,7 +89,8 @@ def forward_loss(features, lookup, weights, bias, y_true, kind, grad_scale=None,
         _lib.check(_lib.lib().ffi_forward_loss_f32(
             features.data_ptr(), lookup.data_ptr(), weights.data_ptr(), bias.data_ptr() if bias is not None else None,
             indices.data_ptr() if indices.numel() else None,
-            values.data_ptr() if values is not None and values.numel() else None, indices.shape[0], int(kind), scale,
+            values.data_ptr() if values is not None and values.numel() else None, indices.shape[0],
+            int(kind) | (SKIP_ZERO_STORES if skip_zero_stores else 0), scale,
             scores.data_ptr() if want_scores else None, out_grad.data_ptr(), loss_sum.data_ptr(),
             masks.data_ptr() if want_masks else None,
             batch, num_features, num_units, fan_in, int(transposed), _stream_handle(features.device)))
@@ -117,7 +123,8 @@ class _LayerLossFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, features, lookup, weights, bias, indices, values, kind, transposed, want_scores):
         scores, out_grad, loss_sum, masks = forward_loss(features, lookup, weights, bias, (indices, values), kind,
-                                                         transposed=transposed, want_scores=want_scores, want_masks=True)
+                                                         transposed=transposed, want_scores=want_scores, want_masks=True,
+                                                         skip_zero_stores=True)
         ctx.save_for_backward(features, lookup, weights, out_grad, masks)
         ctx.transposed = transposed
         ctx.has_bias = bias is not None
@@ -136,7 +143,7 @@ class _LayerLossFn(torch.autograd.Function):
         feature_grad, weight_grad, bias_grad, _ = backward_sparse(features, lookup, weights, g, nz_words=masks,
                                                                   transposed=ctx.transposed,
                                                                   need_feature_grad=ctx.needs_input_grad[0],
-                                                                  need_bias_grad=ctx.has_bias)
+                                                                  need_bias_grad=ctx.has_bias, grad_is_partial=True)
         return feature_grad, None, weight_grad, bias_grad, None, None, None, None, None
 
 

@@ -202,7 +202,11 @@ int ffi_topk_f32(const float* scores, int64_t batch, int64_t num_units, int k,
 enum ffi_loss_kind {
     FFI_LOSS_HINGE = 1,           /* SparseHingeLoss          sparse/metrics.py:147-154 */
     FFI_LOSS_SQUARED_HINGE = 2,   /* SparseSquaredHingeLoss   sparse/metrics.py:157-164 */
-    FFI_LOSS_BCE = 3              /* SparseBinaryCrossEntropyLoss  sparse/metrics.py:167-173 */
+    FFI_LOSS_BCE = 3,             /* SparseBinaryCrossEntropyLoss  sparse/metrics.py:167-173 */
+    /* flag for ffi_forward_loss_f32, OR-ed into loss_kind: gradients that are exactly zero are not stored
+       (out_grad keeps what it held there); needs nz_words, which then says which entries were written.
+       Such an out_grad goes to ffi_backward_sparse_f32 with grad_is_partial != 0. */
+    FFI_LOSS_SKIP_ZERO_STORES = 0x100
 };
 int ffi_loss_grad_f32(const float* scores, const int64_t* label_indices, const float* label_values, int64_t nnz,
                       int loss_kind, float grad_scale, float* out_grad, float* loss_sum, uint32_t* nz_words,
@@ -214,6 +218,8 @@ int ffi_loss_grad_f32(const float* scores, const int64_t* label_indices, const f
  * memory): the forward kernel turns each finished score into its loss gradient before storing it.
  * `bias` may be NULL; `scores` may be NULL when only the gradient and the loss are wanted (the
  * scores of the listed label positions are then recomputed from their rows of lookup / weights).
+ * With FFI_LOSS_SKIP_ZERO_STORES in loss_kind the kernel leaves out the stores of zero gradients: with
+ * a hinge loss late in training that is nearly all of the [batch, num_units] matrix.
  */
 int ffi_forward_loss_f32(const float* features, const int32_t* lookup, const float* weights, const float* bias,
                          const int64_t* label_indices, const float* label_values, int64_t nnz,
@@ -230,6 +236,9 @@ int ffi_forward_loss_f32(const float* features, const int32_t* lookup, const flo
  *   nz_words      the masks of the non-zero entries as ffi_forward_loss_f32 / ffi_loss_grad_f32 write
  *                 them (a set bit over a zero entry is allowed, a clear bit over a non-zero entry is
  *                 not), or NULL: out_grad is then scanned first (one read of the matrix);
+ *   grad_is_partial  != 0: out_grad holds values only where nz_words (required then) has a bit set, as
+ *                 ffi_forward_loss_f32 leaves it with FFI_LOSS_SKIP_ZERO_STORES; if the dense kernels have
+ *                 to run, the call first writes zeros into out_grad wherever the bit is clear;
  *   max_density   share of set bits up to which the sparse kernels are used (<= 0: library default);
  *                 above it the call runs the dense kernels of ffi_backward_bias_f32;
  *   sparse_path_taken  HOST int, may be NULL: 1 if the sparse kernels ran, 0 if the dense ones did.
@@ -238,7 +247,7 @@ int ffi_forward_loss_f32(const float* features, const int32_t* lookup, const flo
  * with LDS float adds issued in a fixed order, no global atomics.
  */
 int ffi_backward_sparse_f32(const float* features, const int32_t* lookup, const float* weights,
-                            const float* out_grad, const uint32_t* nz_words, float max_density,
+                            float* out_grad, const uint32_t* nz_words, int grad_is_partial, float max_density,
                             float* feature_grad, float* weight_grad, float* bias_grad, int* sparse_path_taken,
                             int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in,
                             int transposed, ffi_stream_t stream);

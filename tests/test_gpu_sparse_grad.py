@@ -178,3 +178,34 @@ def test_fused_loss_backward_uses_the_sparse_kernels(ffi):
         grads.append((w.grad.cpu().numpy(), bias.grad.cpu().numpy(), xin.grad.cpu().numpy()))
     for a, b in zip(grads[1], grads[0]):
         assert rel_err(a, b) <= GRAD_RTOL
+
+
+@pytest.mark.parametrize("force_dense", [False, True])
+def test_gradient_stored_only_where_it_is_not_zero(ffi, force_dense):
+    # forward_loss(skip_zero_stores): out_grad is written at the masks' set bits only; the backward pass, told
+    # so, gives the results of the full gradient on the sparse kernels and (zeros filled in first) on the dense ones
+    B, N, L, K, tp = 96, 384, 3000, 32, True
+    rng = np.random.default_rng(12)
+    feats, lookup, w, _ = make_case((B, N, L, K, tp), 0.0, seed=12)
+    w *= 0.3
+    bias = np.full(L, -1.5, np.float32)
+    keys = np.unique(np.repeat(np.arange(B), 3) * L + rng.integers(0, L, B * 3))
+    indices = np.stack([keys // L, keys % L], axis=1).astype(np.int64)
+    dev = lambda a: torch.from_numpy(a).cuda()  # noqa: E731
+    y = (dev(indices), None)
+    args = (dev(feats), dev(lookup), dev(w), dev(bias), y, oracle.LOSS_SQUARED_HINGE)
+    _, g_full, loss_full, masks_full = ffi.metrics.forward_loss(*args, transposed=tp, want_masks=True)
+    _, g_part, loss_part, masks = ffi.metrics.forward_loss(*args, transposed=tp, want_masks=True, skip_zero_stores=True)
+    torch.cuda.synchronize()
+    assert torch.equal(masks, masks_full) and float(loss_full) == float(loss_part)
+    written = torch.from_numpy(np.unpackbits(masks.cpu().numpy().view(np.uint8).reshape(-1, L, 4), axis=2, bitorder="little")
+                               .reshape(-1, L, 32).transpose(0, 2, 1).reshape(-1, L)[:B].astype(bool)).cuda()
+    assert torch.equal(g_part[written], g_full[written])
+    g_part[~written] = float("nan")                  # whatever was there must not matter
+    ref_gx, ref_gw = oracle.backward(feats, lookup, w, g_full.cpu().numpy(), transposed=tp)
+    gx, gw, gb, sparse = ffi.backward_sparse(dev(feats), dev(lookup), dev(w), g_part, nz_words=masks, transposed=tp,
+                                             max_density=1e-9 if force_dense else 1.0, need_bias_grad=True, grad_is_partial=True)
+    torch.cuda.synchronize()
+    assert sparse == (not force_dense)
+    assert rel_err(gw.cpu().numpy(), ref_gw) <= GRAD_RTOL and rel_err(gx.cpu().numpy(), ref_gx) <= GRAD_RTOL
+    assert rel_err(gb.cpu().numpy(), g_full.cpu().numpy().astype(np.float64).sum(axis=0)) <= GRAD_RTOL
