@@ -51,7 +51,7 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--train-step", type=float, default=0.0, metavar="DENSITY",
                     help="also time one training step of the layer (forward + squared-hinge loss gradient in one kernel, "
-                         "backward over the non-zero gradients, Adam) with the bias set so that this share of the loss "
+                         "backward over the non-zero gradients and Adam in one call) with the bias set so that this share of the loss "
                          "gradients is non-zero; reported under 'train_step' in the same JSON line")
     ap.add_argument("--copy-bytes", type=int, default=0,
                     help="also run one plain device copy kernel of this many bytes (read N, write N): the "
@@ -149,10 +149,15 @@ def train_step(pkg, cfg, x, lookup, w, tp, density, stream, iters):
     def backward_dense():
         check(lib.ffi_backward_bias_f32(ptr(x), ptr(lookup), ptr(w), ptr(g), ptr(gx), ptr(gw), ptr(gb), B, N, L, K, int(tp), sh))
 
+    def backward_adam():
+        # learning rate 0: all the memory traffic and arithmetic of the step, and the same scores in every timed pass
+        check(lib.ffi_backward_sparse_adam_f32(ptr(x), ptr(lookup), ptr(w), ptr(g), ptr(masks), 1, ctypes.c_float(0.0), ptr(gx),
+                                               ptr(mw), ptr(vw), ptr(bias), ptr(mb), ptr(vb), 0.0, 0.9, 0.999, 1e-7, 1,
+                                               ctypes.byref(taken), B, N, L, K, int(tp), sh))
+
     def whole():
         fused_forward_loss()
-        backward_sparse()
-        adam()
+        backward_adam()
 
     out = {"loss": "squared hinge, 5 labels per sample", "target_density": density}
     out["forward_loss_ms"] = round(time_kernel(fused_forward_loss, stream, iters), 4)
@@ -162,6 +167,7 @@ def train_step(pkg, cfg, x, lookup, w, tp, density, stream, iters):
     out["backward_sparse_ms"] = round(time_kernel(backward_sparse, stream, iters), 4)
     out["sparse_kernels_ran"] = bool(taken.value)
     out["adam_ms"] = round(time_kernel(adam, stream, iters), 4)
+    out["backward_sparse_with_adam_ms"] = round(time_kernel(backward_adam, stream, iters), 4)
     out["step_ms"] = round(time_kernel(whole, stream, iters), 4)
     out["samples_per_s"] = round(B / (out["step_ms"] * 1e-3), 1)
     out["unfused_dense_route_ms"] = {"forward_bias+loss_grad": round(time_kernel(unfused_forward_loss, stream, iters), 4),

@@ -288,13 +288,13 @@ int ffi_backward_sparse_f32(const float* features, const int32_t* lookup, const 
     unsigned long long set_bits = 0;
     FFI_TRY(nonzero_count(out_grad, nz_words, d.B, d.L, s, &words, &set_bits));
     const double limit = (double)(max_density > 0.f ? max_density : kSparseDefaultMaxDensity) * (double)d.B * (double)d.L;
-    const bool sparse = (double)set_bits <= limit;
+    const bool sparse = (double)set_bits <= limit && sparse_weight_grad_fits(d.B, d.N);
     if (sparse_path_taken) *sparse_path_taken = sparse ? 1 : 0;
     // the dense kernels read all of out_grad
     if (!sparse && grad_is_partial) FFI_TRY(launch_zero_unmasked(out_grad, words, d.B, d.L, s));
     auto wgrad = [&](const ffi_plan* plan) {
         if (!weight_grad) return (int)FFI_OK;
-        if (sparse) return launch_weight_grad_sparse(features, lookup, out_grad, words, weight_grad, bias_grad, d, s);
+        if (sparse) return launch_weight_grad_sparse(features, lookup, out_grad, words, weight_grad, bias_grad, nullptr, d, s);
         return launch_weight_grad(features, lookup, out_grad, weight_grad, bias_grad, d, s, plan);
     };
     if (!feature_grad) return wgrad(nullptr);
@@ -312,6 +312,59 @@ int ffi_adam_step_f32(float* variable, float* m, float* v, const float* gradient
     if (step < 1) return FFI_ERR_BAD_ARGUMENT;
     return launch_adam_step(variable, m, v, gradient, (size_t)count, learning_rate, beta_1, beta_2, epsilon, (long long)step,
                             (hipStream_t)stream);
+}
+
+int ffi_backward_sparse_adam_f32(const float* features, const int32_t* lookup, float* weights, float* out_grad,
+                                 const uint32_t* nz_words, int grad_is_partial, float max_density, float* feature_grad,
+                                 float* weight_m, float* weight_v, float* bias, float* bias_m, float* bias_v,
+                                 float learning_rate, float beta_1, float beta_2, float epsilon, int64_t step,
+                                 int* sparse_path_taken, int64_t batch, int64_t num_features, int64_t num_units,
+                                 int64_t fan_in, int transposed, ffi_stream_t stream) {
+    if (!features || !lookup || !weights || !out_grad || !weight_m || !weight_v) return FFI_ERR_NULL_POINTER;
+    if (bias && (!bias_m || !bias_v)) return FFI_ERR_NULL_POINTER;
+    if (grad_is_partial && !nz_words) return FFI_ERR_NULL_POINTER;
+    if (step < 1) return FFI_ERR_BAD_ARGUMENT;
+    Dims d;
+    FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
+    hipStream_t s = (hipStream_t)stream;
+    const unsigned* words = nullptr;
+    unsigned long long set_bits = 0;
+    FFI_TRY(nonzero_count(out_grad, nz_words, d.B, d.L, s, &words, &set_bits));
+    const double limit = (double)(max_density > 0.f ? max_density : kSparseDefaultMaxDensity) * (double)d.B * (double)d.L;
+    const bool sparse = (double)set_bits <= limit && sparse_weight_grad_fits(d.B, d.N);
+    if (sparse_path_taken) *sparse_path_taken = sparse ? 1 : 0;
+    // the gradients live in a workspace: [L*K] weight gradient (16-byte aligned end), [L] bias gradient, [L] row flags
+    const size_t wcount = (size_t)d.L * d.K;
+    const size_t bias_at = (wcount + 3) / 4 * 4;
+    float* grads = nullptr;
+    FFI_TRY(workspace_get(s, kWsGradients, (bias_at + (size_t)d.L) * sizeof(float) + (size_t)d.L, (void**)&grads));
+    float* gw = grads;
+    float* gb = bias ? grads + bias_at : nullptr;
+    unsigned char* active = reinterpret_cast<unsigned char*>(grads + bias_at + d.L);
+    if (sparse) {
+        // the weight gradient of labels without a non-zero out_grad entry is neither written nor read: the Adam
+        // pass takes a zero for them
+        FFI_TRY(launch_weight_grad_sparse(features, lookup, out_grad, words, gw, gb, active, d, s));
+        if (feature_grad) {
+            if (sparse_input_grad_fits(d.N, d.K)) {
+                FFI_TRY(launch_input_grad_sparse(lookup, weights, out_grad, words, feature_grad, d, s));
+            } else {
+                FFI_TRY(input_grad_cached(lookup, weights, out_grad, feature_grad, d, s, [](const ffi_plan*) { return (int)FFI_OK; }));
+            }
+        }
+        FFI_TRY(launch_adam_step_rows(weights, weight_m, weight_v, gw, active, d.L, d.K, learning_rate, beta_1, beta_2, epsilon,
+                                      (long long)step, s));
+        if (bias) FFI_TRY(launch_adam_step(bias, bias_m, bias_v, gb, (size_t)d.L, learning_rate, beta_1, beta_2, epsilon, (long long)step, s));
+        return FFI_OK;
+    }
+    // dense kernels: gradients into a workspace, then the Adam pass
+    if (grad_is_partial) FFI_TRY(launch_zero_unmasked(out_grad, words, d.B, d.L, s));
+    auto wgrad = [&](const ffi_plan* plan) { return launch_weight_grad(features, lookup, out_grad, gw, gb, d, s, plan); };
+    if (feature_grad) FFI_TRY(input_grad_cached(lookup, weights, out_grad, feature_grad, d, s, wgrad));
+    else FFI_TRY(wgrad(nullptr));
+    FFI_TRY(launch_adam_step(weights, weight_m, weight_v, gw, wcount, learning_rate, beta_1, beta_2, epsilon, (long long)step, s));
+    if (bias) FFI_TRY(launch_adam_step(bias, bias_m, bias_v, gb, (size_t)d.L, learning_rate, beta_1, beta_2, epsilon, (long long)step, s));
+    return FFI_OK;
 }
 
 int ffi_plan_create(const int32_t* lookup, int64_t num_units, int64_t fan_in, int64_t num_features,

@@ -38,7 +38,7 @@ int hip_fail(hipError_t e);
 
 // Library-owned device scratch, one buffer per (device, stream, slot), grown on demand and kept.
 // Work that uses a buffer is ordered by the stream it belongs to.
-enum WorkspaceSlot { kWsFeaturesT = 0, kWsPartials = 1, kWsSlots = 2, kWsLoss = 3, kWsNonzero = 4 };
+enum WorkspaceSlot { kWsFeaturesT = 0, kWsPartials = 1, kWsSlots = 2, kWsLoss = 3, kWsNonzero = 4, kWsGradients = 5 };
 int workspace_get(hipStream_t s, int slot, size_t bytes, void** out);
 void workspace_clear(int device);
 size_t workspace_bytes(int device);
@@ -102,9 +102,13 @@ int launch_nonzero_scan(const float* g, unsigned* words, int B, int L, hipStream
 // synchronises the stream
 int nonzero_count(const float* g, const unsigned* given_words, int B, int L, hipStream_t s, const unsigned** words_out,
                   unsigned long long* count_out);
+// active == null: every row of gw is written (zeros for labels without a set bit).  active != null ([L] bytes):
+// only the rows of labels with a set bit are written and active[j] tells which
 int launch_weight_grad_sparse(const float* x, const int32_t* idx, const float* g, const unsigned* words, float* gw,
-                              float* bias_grad, const Dims& d, hipStream_t s);
+                              float* bias_grad, unsigned char* active, const Dims& d, hipStream_t s);
 bool sparse_input_grad_fits(int N, int K);
+bool sparse_weight_grad_fits(int B, int N);   // x within 32-bit byte offsets
+bool sparse_weight_grad_fits(int B, int N);   // x within 32-bit byte offsets
 // g[b,j] = 0 wherever the mask bit of (b,j) is clear
 int launch_zero_unmasked(float* g, const unsigned* words, int B, int L, hipStream_t s);
 int launch_input_grad_sparse(const int32_t* idx, const float* w, const float* g, const unsigned* words, float* gx,
@@ -114,6 +118,9 @@ int launch_input_grad_sparse(const int32_t* idx, const float* w, const float* g,
 // one Adam step (Keras' update rule) on `count` float32 variables; arrays 16-byte aligned; step is 1-based
 int launch_adam_step(float* var, float* m, float* v, const float* g, size_t count, float lr, float beta_1, float beta_2,
                      float eps, long long step, hipStream_t s);
+// the same for a [rows, row_len] variable whose gradient rows are valid only where active[row] != 0 (zero elsewhere)
+int launch_adam_step_rows(float* var, float* m, float* v, const float* g, const unsigned char* active, int rows, int row_len,
+                          float lr, float beta_1, float beta_2, float eps, long long step, hipStream_t s);
 
 }  // namespace ffi
 

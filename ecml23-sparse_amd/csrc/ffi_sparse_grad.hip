@@ -18,6 +18,7 @@
 //                           accumulators gx[n] in LDS (LDS float adds issued in a fixed order)
 //   igrad_sparse_reduce_kernel  sums the segments in ascending order into feature_grad
 #include "ffi_internal.h"
+#include "ffi_lds_tile.h"
 
 #include <algorithm>
 #include <mutex>
@@ -114,18 +115,24 @@ __global__ __launch_bounds__(kScanThreads) void nz_transpose_kernel(const unsign
 
 constexpr int kHeavyBits = 12;     // labels with more set bits than this are left to the whole wavefront
 
-// x is addressed as x[b * xsb + n * xsn] (either layout).
-template <bool VEC4>
-__global__ __launch_bounds__(256) void wgrad_sparse_kernel(const float* __restrict__ x, size_t xsb, size_t xsn,
-                                                           const int32_t* __restrict__ idx, const float* __restrict__ g,
-                                                           const unsigned* __restrict__ words, float* __restrict__ gw,
-                                                           float* __restrict__ bias_grad, int B, int N, int L, int K,
-                                                           int nbt) {
+// x is addressed as x[b * xsb + n * xsn] (either layout; byte strides), through a buffer resource with 32-bit
+// offsets: batch * num_features * 4 < 2^32, checked by the launcher.
+// ZERO_FILL == true: rows of labels without a set bit are written as zeros.
+// ZERO_FILL == false: those rows are left alone and active[j] (one byte per label) says which rows were written:
+// for a consumer that does not want to read 4 * K bytes of zeros per idle label.
+template <bool VEC4, bool ZERO_FILL>
+__global__ __launch_bounds__(256, 4) void wgrad_sparse_kernel(const float* __restrict__ x, unsigned xsb, unsigned xsn,
+                                                              const int32_t* __restrict__ idx, const float* __restrict__ g,
+                                                              const unsigned* __restrict__ words, float* __restrict__ gw,
+                                                              float* __restrict__ bias_grad,
+                                                              unsigned char* __restrict__ active, int B, int N, int L,
+                                                              int K, int nbt) {
     const int lane = threadIdx.x & 63;
     const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
     const int nwaves = gridDim.x * 4;
     const int nblk = (L + 63) / 64;
     const unsigned tail = (B & 31) ? (1u << (B & 31)) - 1u : 0xffffffffu;   // bits past the batch are ignored
+    const buffer_rsrc xr = make_rsrc(x, (size_t)B * (size_t)N * sizeof(float));
     for (int blk = wave; blk < nblk; blk += nwaves) {
         const int base = blk * 64;
         const int rows = min(64, L - base);
@@ -139,18 +146,24 @@ __global__ __launch_bounds__(256) void wgrad_sparse_kernel(const float* __restri
         }
         const bool heavy = cnt > kHeavyBits;
         const bool light = mine && !heavy;
-        // rows of labels without a set bit: zeros, written by the whole wavefront (the block's rows are contiguous in gw)
-        {
+        if (ZERO_FILL) {
+            // rows of labels without a set bit: zeros, written by the whole wavefront (the block's rows are contiguous
+            // in gw).  The row of 16-byte element e is e / (K/4), formed in floating point (exact here: e + 0.5 is at
+            // least 0.5 / (K/4) away from a multiple).
             const unsigned long long zero_rows = __ballot(mine && cnt == 0);
             float* blockrows = gw + (size_t)base * K;
             if (VEC4) {
                 const int k4 = K / 4;
+                const float inv_k4 = 1.f / (float)k4;
                 for (int e = lane; e < rows * k4; e += 64)
-                    if ((zero_rows >> (e / k4)) & 1ull) reinterpret_cast<float4*>(blockrows)[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+                    if ((zero_rows >> (int)(((float)e + 0.5f) * inv_k4)) & 1ull)
+                        reinterpret_cast<float4*>(blockrows)[e] = make_float4(0.f, 0.f, 0.f, 0.f);
             } else {
                 for (int e = lane; e < rows * K; e += 64)
                     if ((zero_rows >> (e / K)) & 1ull) blockrows[e] = 0.f;
             }
+        } else if (mine) {
+            active[j] = cnt != 0;
         }
         // ---- every lane its own label ----
         float gsum = 0.f;
@@ -167,8 +180,9 @@ __global__ __launch_bounds__(256) void wgrad_sparse_kernel(const float* __restri
 #pragma unroll
                     for (int k = 0; k < 32; ++k) ids[k] = k0 + k < K ? (unsigned)idx[(size_t)j * K + k0 + k] : 0u;
                 }
+                // column ids -> byte offsets of the columns in x
 #pragma unroll
-                for (int k = 0; k < 32; ++k) ids[k] = ids[k] < (unsigned)N ? ids[k] : 0u;
+                for (int k = 0; k < 32; ++k) ids[k] = (ids[k] < (unsigned)N ? ids[k] : 0u) * xsn;
             } else {
 #pragma unroll
                 for (int k = 0; k < 32; ++k) ids[k] = 0u;
@@ -184,9 +198,16 @@ __global__ __launch_bounds__(256) void wgrad_sparse_kernel(const float* __restri
                         const int b = 32 * t + __ffs((int)m) - 1;
                         m &= m - 1;
                         const float gv = g[(size_t)b * L + j];
-                        const float* xrow = x + (size_t)b * xsb;
+                        const unsigned xrow = (unsigned)b * xsb;
+                        // 16 gathers in flight at a time
 #pragma unroll
-                        for (int k = 0; k < 32; ++k) acc[k] = fmaf(gv, xrow[(size_t)ids[k] * xsn], acc[k]);
+                        for (int h = 0; h < 2; ++h) {
+                            float xv[16];
+#pragma unroll
+                            for (int k = 0; k < 16; ++k) xv[k] = buffer_load_f32(xr, ids[16 * h + k] + xrow, 0);
+#pragma unroll
+                            for (int k = 0; k < 16; ++k) acc[16 * h + k] = fmaf(gv, xv[k], acc[16 * h + k]);
+                        }
                         if (k0 == 0) gsum += gv;
                     }
                 }
@@ -215,7 +236,7 @@ __global__ __launch_bounds__(256) void wgrad_sparse_kernel(const float* __restri
             for (int k0 = 0; k0 < K; k0 += 64) {
                 const int k = k0 + lane;
                 const unsigned id = k < K ? (unsigned)idx[(size_t)jh * K + k] : 0u;
-                const float* xcol = x + (size_t)(id < (unsigned)N ? id : 0u) * xsn;
+                const unsigned xcol = (id < (unsigned)N ? id : 0u) * xsn;
                 float acc = 0.f;
                 hsum = 0.f;
                 for (int t = 0; t < nbt; ++t) {
@@ -234,7 +255,7 @@ __global__ __launch_bounds__(256) void wgrad_sparse_kernel(const float* __restri
                         for (int u = 0; u < 4; ++u) {
                             const int b = bb[u] < 0 ? 0 : bb[u];
                             gv[u] = bb[u] < 0 ? 0.f : g[(size_t)b * L + jh];
-                            xv[u] = xcol[(size_t)b * xsb];
+                            xv[u] = buffer_load_f32(xr, xcol, (unsigned)b * xsb);
                         }
 #pragma unroll
                         for (int u = 0; u < 4; ++u) {
@@ -402,21 +423,24 @@ int nonzero_count(const float* g, const unsigned* given_words, int B, int L, hip
 }
 
 int launch_weight_grad_sparse(const float* x, const int32_t* idx, const float* g, const unsigned* words, float* gw,
-                              float* bias_grad, const Dims& d, hipStream_t s) {
+                              float* bias_grad, unsigned char* active, const Dims& d, hipStream_t s) {
     const int nbt = (d.B + 31) / 32;
     const int nblk = (d.L + 63) / 64;
     const int blocks = std::max(1, std::min((nblk + 3) / 4, device_cu_count() * 8));
-    const size_t xsb = d.tp ? 1 : (size_t)d.N, xsn = d.tp ? (size_t)d.B : 1;
+    // byte strides of x along the batch and along the features
+    const unsigned xsb = (d.tp ? 1u : (unsigned)d.N) * 4u, xsn = (d.tp ? (unsigned)d.B : 1u) * 4u;
     const bool vec4 = (d.K % 4 == 0) && (((uintptr_t)gw | (uintptr_t)idx) % 16 == 0);
-    if (vec4)
-        hipLaunchKernelGGL(wgrad_sparse_kernel<true>, dim3(blocks), dim3(256), 0, s, x, xsb, xsn, idx, g, words, gw, bias_grad, d.B,
-                           d.N, d.L, d.K, nbt);
-    else
-        hipLaunchKernelGGL(wgrad_sparse_kernel<false>, dim3(blocks), dim3(256), 0, s, x, xsb, xsn, idx, g, words, gw, bias_grad, d.B,
-                           d.N, d.L, d.K, nbt);
+#define FFI_LAUNCH_WS(V, Z)                                                                                                  \
+    hipLaunchKernelGGL((wgrad_sparse_kernel<V, Z>), dim3(blocks), dim3(256), 0, s, x, xsb, xsn, idx, g, words, gw, bias_grad, active, \
+                       d.B, d.N, d.L, d.K, nbt)
+    if (active == nullptr) { if (vec4) FFI_LAUNCH_WS(true, true); else FFI_LAUNCH_WS(false, true); }
+    else                   { if (vec4) FFI_LAUNCH_WS(true, false); else FFI_LAUNCH_WS(false, false); }
+#undef FFI_LAUNCH_WS
     FFI_HIP_TRY(hipGetLastError());
     return FFI_OK;
 }
+
+bool sparse_weight_grad_fits(int B, int N) { return (unsigned long long)B * (unsigned long long)N < (1ull << 30); }
 
 bool sparse_input_grad_fits(int N, int K) { return N <= kSparseMaxFeatures && K <= 65535; }
 

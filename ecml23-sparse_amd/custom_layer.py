@@ -127,6 +127,32 @@ class StratifiedRewireLayerV2(torch.nn.Module):
         weights = self.kernel_weights.view(-1, self.fan_in)
         return loss.fused(inputs.float(), indices, weights, self.bias, y_true, transposed=False, want_scores=want_scores)
 
+    @torch.no_grad()
+    def fused_train_step(self, inputs: torch.Tensor, y_true, loss, optimizer, need_input_grad: bool = False):
+        """Forward, loss, backward and the Adam step on this layer's variables in two library calls: the
+        forward kernel stores loss gradients (non-zero ones only) instead of scores, the backward pass
+        walks them and the Adam pass skips the gradient rows of labels that received none.  ``optimizer`` is a
+        ``SparseAdam`` that owns ``kernel_weights`` (and ``bias``); this uses its moments and
+        ``iterations + 1`` as the step number and leaves ``optimizer.step()`` (other parameters, the
+        counter) to the caller.  Returns ``(loss value, gradient with respect to inputs or None)``."""
+        from . import metrics, optimizer as opt_mod
+        if inputs.dim() != 2 or inputs.shape[1] != self.input_dim:
+            raise ValueError(f"inputs must have shape [batch, {self.input_dim}], got {tuple(inputs.shape)}")
+        inputs = inputs.float().contiguous()
+        indices = self.kernel_indices.view(-1, self.fan_in)
+        weights = self.kernel_weights.data.view(-1, self.fan_in)
+        bias = self.bias.data if self.use_bias else None
+        _, out_grad, loss_sum, masks = metrics.forward_loss(inputs, indices, weights, bias, y_true, loss.kind, want_masks=True,
+                                                            skip_zero_stores=True)
+        iw = optimizer._index_of(self.kernel_weights)
+        ib = optimizer._index_of(self.bias) if self.use_bias else None
+        input_grad, _ = opt_mod.backward_sparse_adam(
+            inputs, indices, weights, out_grad, masks, optimizer._momentums[iw], optimizer._velocities[iw],
+            bias, optimizer._momentums[ib] if self.use_bias else None, optimizer._velocities[ib] if self.use_bias else None,
+            optimizer.learning_rate, optimizer.beta_1, optimizer.beta_2, optimizer.epsilon, optimizer.iterations + 1,
+            grad_is_partial=True, need_feature_grad=need_input_grad)
+        return loss_sum[0] / (inputs.shape[0] * self.units), input_grad
+
     # sparse/layer.py:215-219, 236-237 and sparse/custom_layer.py:20-43
     @torch.no_grad()
     def rewire(self, other_vars=None):

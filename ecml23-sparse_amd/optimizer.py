@@ -66,3 +66,40 @@ class SparseAdam:
             self._velocities[i].copy_(new_v)
         else:
             layer.rewire(None)
+
+
+def backward_sparse_adam(features, lookup, weights, out_grad, nz_words, weight_m, weight_v, bias, bias_m, bias_v,
+                         learning_rate, beta_1, beta_2, epsilon, step, transposed=False, grad_is_partial=False,
+                         max_density=None, need_feature_grad=True):
+    """Backward pass of the layer and the Adam step on its weights (and bias, unless ``None``) in one call:
+    ``weights``, ``bias`` and their moments are updated in place; the weight/bias gradients stay inside the
+    library (gradient rows of labels without a non-zero entry of ``out_grad`` are neither written nor read).  Returns ``(feature_grad or None, sparse_kernels_ran)``;
+    ``feature_grad`` is formed from the weights as they were on entry."""
+    import ctypes
+
+    from .fixed_fan_in_ops import _check_inputs
+
+    batch, num_features, num_units, fan_in = _check_inputs(features, lookup, weights, transposed, out_grad)
+    for name, t in (("weights", weights), ("weight_m", weight_m), ("weight_v", weight_v), ("out_grad", out_grad),
+                    ("features", features), ("lookup", lookup)):
+        if not t.is_contiguous():
+            raise ValueError(f"{name} must be contiguous (it is updated or read in place)")
+    for name, t in (("weight_m", weight_m), ("weight_v", weight_v)):
+        if t.dtype != torch.float32 or t.numel() != weights.numel() or t.device != weights.device:
+            raise TypeError(f"{name} must be a float32 tensor with as many elements as weights, on their device")
+    if bias is not None:
+        for name, t in (("bias", bias), ("bias_m", bias_m), ("bias_v", bias_v)):
+            if t is None or t.dtype != torch.float32 or t.numel() != num_units or not t.is_contiguous() or t.device != weights.device:
+                raise TypeError(f"{name} must be a contiguous float32 tensor of {num_units} elements on the weights' device")
+    taken = ctypes.c_int(-1)
+    with torch.cuda.device(features.device):
+        feature_grad = torch.empty_like(features) if need_feature_grad else None
+        _lib.check(_lib.lib().ffi_backward_sparse_adam_f32(
+            features.data_ptr(), lookup.data_ptr(), weights.data_ptr(), out_grad.data_ptr(),
+            nz_words.data_ptr() if nz_words is not None else None, int(bool(grad_is_partial)), float(max_density or 0.0),
+            feature_grad.data_ptr() if need_feature_grad else None, weight_m.data_ptr(), weight_v.data_ptr(),
+            bias.data_ptr() if bias is not None else None, bias_m.data_ptr() if bias is not None else None,
+            bias_v.data_ptr() if bias is not None else None,
+            float(learning_rate), float(beta_1), float(beta_2), float(epsilon), int(step), ctypes.byref(taken),
+            batch, num_features, num_units, fan_in, int(transposed), _stream_handle(features.device)))
+    return feature_grad, bool(taken.value)

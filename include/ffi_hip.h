@@ -253,6 +253,24 @@ int ffi_backward_sparse_f32(const float* features, const int32_t* lookup, const 
                             int transposed, ffi_stream_t stream);
 
 /*
+ * Backward pass and optimizer step in one call: the results of ffi_backward_sparse_f32 (feature_grad,
+ * from the weights as they are on entry) followed by ffi_adam_step_f32 on `weights` with weight_grad and
+ * on `bias` with bias_grad; the two gradients are not returned (they live in a library workspace).
+ * When the sparse kernels run, the weight gradient of a label without a non-zero out_grad entry is
+ * neither written nor read: the Adam pass takes a zero for it.  `bias` (with bias_m, bias_v) may be
+ * NULL; feature_grad may be NULL.  The other arguments are those of the two calls.
+ * No counterpart in the reference, where the optimizer is a separate TensorFlow op.
+ */
+int ffi_backward_sparse_adam_f32(const float* features, const int32_t* lookup, float* weights, float* out_grad,
+                                 const uint32_t* nz_words, int grad_is_partial, float max_density,
+                                 float* feature_grad, float* weight_m, float* weight_v,
+                                 float* bias, float* bias_m, float* bias_v,
+                                 float learning_rate, float beta_1, float beta_2, float epsilon, int64_t step,
+                                 int* sparse_path_taken,
+                                 int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in,
+                                 int transposed, ffi_stream_t stream);
+
+/*
  * One Adam step on `count` float32 variables (weights [num_units * fan_in], or the bias), the
  * optimizer the reference trains the layer with: SparseAdam (sparse/optimizer.py:9-23) is a
  * keras.optimizers.Adam (run.py:126) and this is that class's update rule,
