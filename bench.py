@@ -170,6 +170,17 @@ def train_step(pkg, cfg, x, lookup, w, tp, density, stream, iters):
     out["backward_sparse_with_adam_ms"] = round(time_kernel(backward_adam, stream, iters), 4)
     out["step_ms"] = round(time_kernel(whole, stream, iters), 4)
     out["samples_per_s"] = round(B / (out["step_ms"] * 1e-3), 1)
+    # rewiring (every rewire_interval steps in the reference): threshold of the 1 % smallest magnitudes, redraw of
+    # their sources, moments cleared -- on a copy of the index matrix, so the layer above is left as it is
+    lookup2 = lookup.clone()
+    thr = torch.empty(1, device="cuda")
+    arrays = (ctypes.c_void_p * 2)(ptr(mw), ptr(vw))
+
+    def rewire():
+        check(lib.ffi_select_threshold_f32(ptr(w), L * K, (L * K) // 100, ptr(thr), sh))
+        check(lib.ffi_rewire_f32(ptr(lookup2), ptr(w), arrays, 2, L * K, N, ptr(thr), 12345, None, sh))
+
+    out["rewire_1pct_ms"] = round(time_kernel(rewire, stream, iters), 4)
     out["unfused_dense_route_ms"] = {"forward_bias+loss_grad": round(time_kernel(unfused_forward_loss, stream, iters), 4),
                                      "backward_dense": round(time_kernel(backward_dense, stream, iters), 4)}
     return out

@@ -40,6 +40,8 @@ SIGNATURES = {
     "ffi_forward_loss_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _int, _f32, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "ffi_backward_sparse_adam_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _f32, _vp, _vp, _vp, _vp, _vp, _vp, _f32, _f32, _f32, _f32,
                                             _i64, ctypes.POINTER(_int), _i64, _i64, _i64, _i64, _int, _vp]),
+    "ffi_select_threshold_f32": (_int, [_vp, _i64, _i64, _vp, _vp]),
+    "ffi_rewire_f32": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _vp, ctypes.c_uint64, _vp, _vp]),
     "ffi_adam_step_f32": (_int, [_vp, _vp, _vp, _vp, _i64, _f32, _f32, _f32, _f32, _i64, _vp]),
     "ffi_backward_sparse_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _f32, _vp, _vp, _vp, ctypes.POINTER(_int), _i64, _i64, _i64, _i64, _int, _vp]),
 }

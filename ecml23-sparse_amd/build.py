@@ -29,6 +29,7 @@ SOURCES = [
     "ffi_loss.hip",
     "ffi_sparse_grad.hip",
     "ffi_optimizer.hip",
+    "ffi_rewire.hip",
 ]
 
 # gfx950 only.  Packed-fp32 VALU forms are switched off for all device code.

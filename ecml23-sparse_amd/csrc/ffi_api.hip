@@ -367,6 +367,25 @@ int ffi_backward_sparse_adam_f32(const float* features, const int32_t* lookup, f
     return FFI_OK;
 }
 
+int ffi_select_threshold_f32(const float* weights, int64_t count, int64_t k, float* threshold, ffi_stream_t stream) {
+    if (!weights || !threshold) return FFI_ERR_NULL_POINTER;
+    if (count <= 0) return FFI_ERR_BAD_SHAPE;
+    if (k < 0 || k > count) return FFI_ERR_BAD_ARGUMENT;
+    return launch_select_threshold(weights, (size_t)count, (unsigned long long)k, threshold, (hipStream_t)stream);
+}
+
+int ffi_rewire_f32(int32_t* lookup, const float* weights, float* const* arrays, int n_arrays, int64_t count,
+                   int64_t num_features, const float* threshold, uint64_t seed, int64_t* rewired_count, ffi_stream_t stream) {
+    if (!lookup || !weights || !threshold || (n_arrays > 0 && !arrays)) return FFI_ERR_NULL_POINTER;
+    if (n_arrays < 0 || n_arrays > 4) return FFI_ERR_BAD_ARGUMENT;
+    for (int i = 0; i < n_arrays; ++i)
+        if (!arrays[i]) return FFI_ERR_NULL_POINTER;
+    if (count <= 0 || num_features <= 0) return FFI_ERR_BAD_SHAPE;
+    if (num_features >= INT32_MAX) return FFI_ERR_TOO_LARGE;
+    return launch_rewire(lookup, weights, arrays, n_arrays, (size_t)count, (unsigned)num_features, threshold,
+                         (unsigned long long)seed, (long long*)rewired_count, (hipStream_t)stream);
+}
+
 int ffi_plan_create(const int32_t* lookup, int64_t num_units, int64_t fan_in, int64_t num_features,
                     int64_t batch_hint, ffi_stream_t stream, ffi_plan** plan) {
     if (!lookup || !plan) return FFI_ERR_NULL_POINTER;

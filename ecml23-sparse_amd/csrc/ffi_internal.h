@@ -38,7 +38,7 @@ int hip_fail(hipError_t e);
 
 // Library-owned device scratch, one buffer per (device, stream, slot), grown on demand and kept.
 // Work that uses a buffer is ordered by the stream it belongs to.
-enum WorkspaceSlot { kWsFeaturesT = 0, kWsPartials = 1, kWsSlots = 2, kWsLoss = 3, kWsNonzero = 4, kWsGradients = 5 };
+enum WorkspaceSlot { kWsFeaturesT = 0, kWsPartials = 1, kWsSlots = 2, kWsLoss = 3, kWsNonzero = 4, kWsGradients = 5, kWsRewire = 6 };
 int workspace_get(hipStream_t s, int slot, size_t bytes, void** out);
 void workspace_clear(int device);
 size_t workspace_bytes(int device);
@@ -121,6 +121,14 @@ int launch_adam_step(float* var, float* m, float* v, const float* g, size_t coun
 // the same for a [rows, row_len] variable whose gradient rows are valid only where active[row] != 0 (zero elsewhere)
 int launch_adam_step_rows(float* var, float* m, float* v, const float* g, const unsigned char* active, int rows, int row_len,
                           float lr, float beta_1, float beta_2, float eps, long long step, hipStream_t s);
+
+// ---- rewiring (ffi_rewire.hip) -------------------------------------------------------------------
+// *threshold (device) = the k-th smallest |w| (k counted from 1; k == 0 gives 0)
+int launch_select_threshold(const float* w, size_t count, unsigned long long k, float* threshold, hipStream_t s);
+// positions with |w| < *threshold get a new source in [0, num_features) and zeros in the listed arrays;
+// *rewired (device, may be null) receives their number
+int launch_rewire(int32_t* lookup, const float* w, float* const* arrays, int n_arrays, size_t count, unsigned num_features,
+                  const float* threshold, unsigned long long seed, long long* rewired, hipStream_t s);
 
 }  // namespace ffi
 

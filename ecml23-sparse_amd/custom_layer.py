@@ -25,6 +25,10 @@ class FixedMagnitudeSelector:
     def select(self, weight_values: torch.Tensor) -> torch.Tensor:
         return weight_values.abs() < self.threshold
 
+    def threshold_tensor(self, weight_values: torch.Tensor) -> torch.Tensor:
+        """The magnitude below which connections are rewired, as a device tensor ``[1]``."""
+        return torch.full((1,), self.threshold, dtype=torch.float32, device=weight_values.device)
+
 
 class FixedFractionSelector:
     """Rewire a fixed fraction of the connections, those of lowest magnitude (sparse/layer.py:60-84).
@@ -45,6 +49,11 @@ class FixedFractionSelector:
             return torch.zeros_like(flat, dtype=torch.bool)
         threshold = torch.kthvalue(flat, num_selected).values
         return flat < threshold
+
+    def threshold_tensor(self, weight_values: torch.Tensor) -> torch.Tensor:
+        """The same threshold by the library's radix select (device tensor ``[1]``; 0 selects nothing)."""
+        flat = weight_values.detach().reshape(-1).contiguous()
+        return ops.select_threshold(flat, int(round(self.fraction * flat.numel())))
 
 
 class StratifiedRewireLayerV2(torch.nn.Module):
@@ -71,6 +80,9 @@ class StratifiedRewireLayerV2(torch.nn.Module):
         self.use_bias = bool(use_bias)
         self.rewire_selector = rewire_selector if rewire_selector is not None else FixedFractionSelector(0.01)
         self._generator = generator
+        # seeds of the rewiring draws: a base taken from the generator (or torch's global seed) plus a call counter
+        self._rewire_seed = int(generator.initial_seed() if generator is not None else torch.initial_seed()) * 1000003
+        self._rewire_count = 0
         # one weight per connection, Keras' default 'glorot_uniform' on a rank-1 shape: fan_in = fan_out = connections
         limit = math.sqrt(6.0 / (2.0 * self.connections))
         w = (torch.rand(self.connections, device=device, generator=generator) * 2.0 - 1.0) * limit
@@ -161,14 +173,23 @@ class StratifiedRewireLayerV2(torch.nn.Module):
         the rewired locations set to zero.  The index buffer is edited in place; the library
         notices through the lookup fingerprint and rebuilds its plan on the next backward call."""
         other_vars = [] if other_vars is None else list(other_vars)
-        locations = torch.nonzero(self.rewire_selector.select(self.kernel_weights.detach())).reshape(-1)
-        if locations.numel():
-            self.kernel_indices[locations] = self._random_sources(locations.numel(), self.kernel_indices.device)
-        outputs = []
-        for other in other_vars:
-            new_v = other.clone()
-            new_v.reshape(-1)[locations] = 0
-            outputs.append(new_v)
+        self._rewire_count += 1
+        if hasattr(self.rewire_selector, "threshold_tensor"):
+            # selection, redraw and clearing in the library: one threshold (radix select), one pass over the variables
+            threshold = self.rewire_selector.threshold_tensor(self.kernel_weights.detach())
+            outputs = [other.clone().contiguous() for other in other_vars]
+            ops.rewire_connections(self.kernel_indices, self.kernel_weights.detach().contiguous(), [o.view(-1) for o in outputs],
+                                   self.input_dim, threshold, self._rewire_seed + self._rewire_count)
+        else:
+            # a selector that only offers a boolean mask: the same steps as torch index operations
+            locations = torch.nonzero(self.rewire_selector.select(self.kernel_weights.detach())).reshape(-1)
+            if locations.numel():
+                self.kernel_indices[locations] = self._random_sources(locations.numel(), self.kernel_indices.device)
+            outputs = []
+            for other in other_vars:
+                new_v = other.clone()
+                new_v.reshape(-1)[locations] = 0
+                outputs.append(new_v)
         if self.arrange:
             self.arrange_connections(outputs)
         return outputs

@@ -328,3 +328,40 @@ def arrange_connections(lookup, *arrays):
     with torch.cuda.device(lookup.device):
         _lib.check(_lib.lib().ffi_arrange_connections_f32(lookup.data_ptr(), ptrs, len(arrays), num_units, fan_in,
                                                           _stream_handle(lookup.device)))
+
+
+def select_threshold(weights, k):
+    """Device tensor ``[1]``: the ``k``-th smallest ``|weights|`` (``k`` from 1; 0 gives 0.0), the threshold
+    ``FixedFractionSelector`` (sparse/layer.py:75-86) derives from ``tf.nn.top_k(-|w|, k)``."""
+    if weights.dtype != torch.float32 or not weights.is_cuda or not weights.is_contiguous():
+        raise TypeError("weights must be a contiguous float32 device tensor")
+    with torch.cuda.device(weights.device):
+        threshold = torch.empty((1,), dtype=torch.float32, device=weights.device)
+        _lib.check(_lib.lib().ffi_select_threshold_f32(weights.data_ptr(), weights.numel(), int(k), threshold.data_ptr(),
+                                                       _stream_handle(weights.device)))
+    return threshold
+
+
+def rewire_connections(lookup, weights, arrays, num_features, threshold, seed):
+    """In place: every connection with ``|weights| < threshold`` (``threshold``: device tensor ``[1]``) gets a
+    new source drawn uniformly from ``[0, num_features)`` and zeros in ``arrays`` (up to four float32 tensors
+    shaped like ``weights``).  Returns a device int64 tensor ``[1]`` with the number of connections changed."""
+    import ctypes
+
+    if lookup.dtype not in _INDEX_DTYPES or not lookup.is_cuda or not lookup.is_contiguous():
+        raise TypeError("lookup must be a contiguous int32/uint32 device tensor")
+    if weights.dtype != torch.float32 or weights.numel() != lookup.numel() or not weights.is_contiguous():
+        raise TypeError("weights must be a contiguous float32 tensor with as many elements as lookup")
+    arrays = list(arrays)
+    if len(arrays) > 4:
+        raise ValueError("at most four arrays per call")
+    for a in arrays:
+        if a.dtype != torch.float32 or a.numel() != lookup.numel() or a.device != lookup.device or not a.is_contiguous():
+            raise TypeError("arrays must be contiguous float32 tensors with as many elements as lookup, on its device")
+    ptrs = (ctypes.c_void_p * max(len(arrays), 1))(*[a.data_ptr() for a in arrays])
+    with torch.cuda.device(lookup.device):
+        changed = torch.empty((1,), dtype=torch.int64, device=lookup.device)
+        _lib.check(_lib.lib().ffi_rewire_f32(lookup.data_ptr(), weights.data_ptr(), ptrs, len(arrays), lookup.numel(),
+                                             int(num_features), threshold.data_ptr(), int(seed) & (2**64 - 1), changed.data_ptr(),
+                                             _stream_handle(lookup.device)))
+    return changed

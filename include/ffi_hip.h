@@ -284,6 +284,26 @@ int ffi_adam_step_f32(float* variable, float* m, float* v, const float* gradient
                       float learning_rate, float beta_1, float beta_2, float epsilon, int64_t step,
                       ffi_stream_t stream);
 
+/*
+ * Rewiring (sparse/layer.py:215-219,236-237; sparse/custom_layer.py:20-43), on the flat per-connection
+ * variables of the layer.
+ * ffi_select_threshold_f32: *threshold (one float on the device) = the k-th smallest |weights[i]|, k counted
+ * from 1 -- the threshold FixedFractionSelector.select (sparse/layer.py:75-86) takes from
+ * tf.nn.top_k(-|w|, k) with k = round(fraction * count); k == 0 gives 0 (an empty selection).
+ * ffi_rewire_f32: every position with |weights[i]| < *threshold (the strict comparison of
+ * sparse/layer.py:57,86; a FixedMagnitudeSelector passes its own threshold) gets a new source drawn
+ * uniformly from [0, num_features) in lookup[i] -- by a counter-based generator keyed on (seed, i); the
+ * reference draws from TensorFlow's stream, which no other implementation reproduces -- and zeros in
+ * arrays[0..n_arrays) (HOST array of up to four device pointers: the optimizer's moments,
+ * sparse/optimizer.py:14-21).  Weights keep their values.  *rewired_count (device, may be NULL)
+ * receives the number of positions changed.  Entry points that cache a plan of `lookup` notice the edit
+ * through its fingerprint; an explicit plan needs ffi_plan_refresh.
+ */
+int ffi_select_threshold_f32(const float* weights, int64_t count, int64_t k, float* threshold, ffi_stream_t stream);
+int ffi_rewire_f32(int32_t* lookup, const float* weights, float* const* arrays, int n_arrays, int64_t count,
+                   int64_t num_features, const float* threshold, uint64_t seed, int64_t* rewired_count,
+                   ffi_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -270,3 +270,19 @@ def adam_step(variable, m, v, gradient, learning_rate=0.001, beta_1=0.9, beta_2=
     v += (g * g - v) * (f(1) - f(beta_2))
     var -= (m * alpha) / (np.sqrt(v, dtype=f) + f(epsilon))
     return var, m, v
+
+
+# ---- rewiring selection (numpy) --------------------------------------------------------------------
+def select_threshold(weights, k):
+    """The threshold of FixedFractionSelector.select (sparse/layer.py:75-86): ``tf.nn.top_k(-|w|, k)`` returns
+    the k smallest magnitudes in ascending order of |w|, its last value is the k-th smallest; k == 0 is
+    taken as 0.0 (nothing has a magnitude below it)."""
+    mags = np.abs(np.asarray(weights, dtype=np.float32).reshape(-1))
+    if k <= 0:
+        return np.float32(0.0)
+    return np.partition(mags, k - 1)[k - 1]
+
+
+def rewire_selection(weights, threshold):
+    """Boolean mask of the connections that are rewired: strictly below the threshold (sparse/layer.py:57,86)."""
+    return np.abs(np.asarray(weights, dtype=np.float32)) < np.float32(threshold)

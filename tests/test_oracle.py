@@ -322,3 +322,19 @@ def test_adam_oracle_against_torch_adam():
         np.testing.assert_allclose(w, p.detach().numpy(), rtol=0, atol=3e-6)
         np.testing.assert_allclose(m, opt.state[p]["exp_avg"].numpy(), rtol=1e-5, atol=1e-7)
         np.testing.assert_allclose(v, opt.state[p]["exp_avg_sq"].numpy(), rtol=1e-4, atol=1e-9)
+
+
+# ---- rewiring selection oracle ------------------------------------------------------------------------
+def test_select_threshold_oracle_is_the_kth_smallest_magnitude():
+    rng = np.random.default_rng(4)
+    w = rng.normal(size=5000).astype(np.float32)
+    w[::7] = 0.25                                       # ties
+    w[::11] *= -1
+    ordered = np.sort(np.abs(w))
+    for k in (1, 2, 50, 2500, 4999, 5000):
+        thr = oracle.select_threshold(w, k)
+        assert thr == ordered[k - 1]
+        sel = oracle.rewire_selection(w, thr)
+        # strict comparison: the threshold value itself (and its ties) stays, so fewer than k are selected
+        assert sel.sum() == (ordered < thr).sum() <= k - 1
+    assert oracle.select_threshold(w, 0) == 0.0 and not oracle.rewire_selection(w, 0.0).any()
