@@ -256,3 +256,39 @@ def test_layer_forward_loss_matches_loss_of_forward(ffi):
     assert rel_err(layer.kernel_weights.grad.cpu().numpy(), gw0.cpu().numpy()) <= GRAD_RTOL
     assert rel_err(layer.bias.grad.cpu().numpy(), gb0.cpu().numpy()) <= GRAD_RTOL
     assert rel_err(scores.cpu().numpy(), layer(x).detach().cpu().numpy()) <= FWD_RTOL
+
+
+def test_dense_stratified_block_trains_end_to_end(ffi):
+    # run.py:63-66 ("dense-stratified"): Dense(intermediate, relu) -> StratifiedRewireLayerV2(num_labels); the sparse
+    # layer's input gradient has to reach the dense layer.  torch supplies the dense layer, the library the sparse one.
+    gen = torch.Generator(device="cuda").manual_seed(31)
+    B, D, H, L = 48, 64, 96, 1500
+    dense = torch.nn.Linear(D, H).cuda()
+    sparse = ffi.StratifiedRewireLayerV2(units=L, input_dim=H, connections=L * 8, generator=gen,
+                                         rewire_selector=ffi.FixedFractionSelector(0.02))
+    opt_dense = torch.optim.Adam(dense.parameters(), lr=0.01)
+    opt_sparse = ffi.SparseAdam(list(sparse.parameters()), learning_rate=0.01)
+    loss_fn = ffi.SparseSquaredHingeLoss()
+    x = torch.rand((B, D), device="cuda", generator=gen)
+    rows = torch.arange(B, device="cuda").repeat_interleave(2)
+    cols = torch.randint(0, L, (B * 2,), device="cuda", generator=gen)
+    y = (torch.stack([rows, cols], dim=1), None)
+    p1 = ffi.PrecisionAtK(k=1)
+    losses = []
+    for it in range(1, 61):
+        opt_dense.zero_grad()
+        opt_sparse.zero_grad()
+        hidden = torch.relu(dense(x))
+        loss, scores = sparse.forward_loss(hidden, y, loss_fn, want_scores=(it == 60))
+        loss.backward()
+        assert dense.weight.grad is not None and torch.isfinite(dense.weight.grad).all() and dense.weight.grad.abs().sum() > 0
+        opt_dense.step()
+        opt_sparse.step()
+        if it % 20 == 1:
+            opt_sparse.update_sparse(sparse)
+        losses.append(float(loss.detach()))
+    p1.update_state(y, scores)
+    assert losses[-1] < 0.3 * losses[0]
+    assert 0.0 <= p1.result() <= 1.0
+    # the listed labels are being pulled apart from the rest
+    assert float(scores[rows, cols].mean()) > float(scores.mean()) + 0.1
