@@ -190,7 +190,7 @@ def main():
     args = parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus above 1 is not supported "
-              "(the layer would shard by label, see DESIGN.md)", file=sys.stderr)
+              "(across GPUs the layer would shard by label: each GPU its own labels, one all-reduce of the input gradient)", file=sys.stderr)
         sys.exit(2)
 
     import importlib
