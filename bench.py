@@ -150,8 +150,9 @@ def train_step(pkg, cfg, x, lookup, w, tp, density, stream, iters):
         check(lib.ffi_backward_bias_f32(ptr(x), ptr(lookup), ptr(w), ptr(g), ptr(gx), ptr(gw), ptr(gb), B, N, L, K, int(tp), sh))
 
     def backward_adam():
-        # learning rate 0: all the memory traffic and arithmetic of the step, and the same scores in every timed pass
-        check(lib.ffi_backward_sparse_adam_f32(ptr(x), ptr(lookup), ptr(w), ptr(g), ptr(masks), 1, ctypes.c_float(0.0), ptr(gx),
+        # learning rate 0: all the memory traffic and arithmetic of the step, and the same scores in every timed pass;
+        # flags: out_grad is valid at the masks' set bits only (1), kernels chosen from the previous call's count (2)
+        check(lib.ffi_backward_sparse_adam_f32(ptr(x), ptr(lookup), ptr(w), ptr(g), ptr(masks), 1 | 2, ctypes.c_float(0.0), ptr(gx),
                                                ptr(mw), ptr(vw), ptr(bias), ptr(mb), ptr(vb), 0.0, 0.9, 0.999, 1e-7, 1,
                                                ctypes.byref(taken), B, N, L, K, int(tp), sh))
 

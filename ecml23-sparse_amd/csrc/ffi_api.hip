@@ -274,19 +274,21 @@ int ffi_forward_loss_f32(const float* features, const int32_t* lookup, const flo
 }
 
 int ffi_backward_sparse_f32(const float* features, const int32_t* lookup, const float* weights, float* out_grad,
-                            const uint32_t* nz_words, int grad_is_partial, float max_density, float* feature_grad, float* weight_grad,
+                            const uint32_t* nz_words, int flags, float max_density, float* feature_grad, float* weight_grad,
                             float* bias_grad, int* sparse_path_taken, int64_t batch, int64_t num_features,
                             int64_t num_units, int64_t fan_in, int transposed, ffi_stream_t stream) {
     if (!features || !lookup || !weights || !out_grad) return FFI_ERR_NULL_POINTER;
     if (!feature_grad && !weight_grad) return FFI_ERR_NULL_POINTER;
     if (bias_grad && !weight_grad) return FFI_ERR_NULL_POINTER;
+    const bool grad_is_partial = (flags & FFI_SPARSE_GRAD_IS_PARTIAL) != 0;
+    if (flags & ~(FFI_SPARSE_GRAD_IS_PARTIAL | FFI_SPARSE_DECIDE_FROM_PREVIOUS)) return FFI_ERR_BAD_ARGUMENT;
     if (grad_is_partial && !nz_words) return FFI_ERR_NULL_POINTER;
     Dims d;
     FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
     hipStream_t s = (hipStream_t)stream;
     const unsigned* words = nullptr;
     unsigned long long set_bits = 0;
-    FFI_TRY(nonzero_count(out_grad, nz_words, d.B, d.L, s, &words, &set_bits));
+    FFI_TRY(nonzero_count(out_grad, nz_words, d.B, d.L, s, (flags & FFI_SPARSE_DECIDE_FROM_PREVIOUS) != 0, &words, &set_bits));
     const double limit = (double)(max_density > 0.f ? max_density : kSparseDefaultMaxDensity) * (double)d.B * (double)d.L;
     const bool sparse = (double)set_bits <= limit && sparse_weight_grad_fits(d.B, d.N);
     if (sparse_path_taken) *sparse_path_taken = sparse ? 1 : 0;
@@ -315,13 +317,15 @@ int ffi_adam_step_f32(float* variable, float* m, float* v, const float* gradient
 }
 
 int ffi_backward_sparse_adam_f32(const float* features, const int32_t* lookup, float* weights, float* out_grad,
-                                 const uint32_t* nz_words, int grad_is_partial, float max_density, float* feature_grad,
+                                 const uint32_t* nz_words, int flags, float max_density, float* feature_grad,
                                  float* weight_m, float* weight_v, float* bias, float* bias_m, float* bias_v,
                                  float learning_rate, float beta_1, float beta_2, float epsilon, int64_t step,
                                  int* sparse_path_taken, int64_t batch, int64_t num_features, int64_t num_units,
                                  int64_t fan_in, int transposed, ffi_stream_t stream) {
     if (!features || !lookup || !weights || !out_grad || !weight_m || !weight_v) return FFI_ERR_NULL_POINTER;
     if (bias && (!bias_m || !bias_v)) return FFI_ERR_NULL_POINTER;
+    const bool grad_is_partial = (flags & FFI_SPARSE_GRAD_IS_PARTIAL) != 0;
+    if (flags & ~(FFI_SPARSE_GRAD_IS_PARTIAL | FFI_SPARSE_DECIDE_FROM_PREVIOUS)) return FFI_ERR_BAD_ARGUMENT;
     if (grad_is_partial && !nz_words) return FFI_ERR_NULL_POINTER;
     if (step < 1) return FFI_ERR_BAD_ARGUMENT;
     Dims d;
@@ -329,7 +333,7 @@ int ffi_backward_sparse_adam_f32(const float* features, const int32_t* lookup, f
     hipStream_t s = (hipStream_t)stream;
     const unsigned* words = nullptr;
     unsigned long long set_bits = 0;
-    FFI_TRY(nonzero_count(out_grad, nz_words, d.B, d.L, s, &words, &set_bits));
+    FFI_TRY(nonzero_count(out_grad, nz_words, d.B, d.L, s, (flags & FFI_SPARSE_DECIDE_FROM_PREVIOUS) != 0, &words, &set_bits));
     const double limit = (double)(max_density > 0.f ? max_density : kSparseDefaultMaxDensity) * (double)d.B * (double)d.L;
     const bool sparse = (double)set_bits <= limit && sparse_weight_grad_fits(d.B, d.N);
     if (sparse_path_taken) *sparse_path_taken = sparse ? 1 : 0;
@@ -464,6 +468,7 @@ int ffi_cache_clear(void) {
         }
     }
     workspace_clear(dev);
+    nonzero_count_forget(dev);
     return FFI_OK;
 }
 

@@ -98,10 +98,13 @@ constexpr int kSparseMaxFeatures = 3072;   // the sparse input gradient keeps 8 
 constexpr float kSparseDefaultMaxDensity = 0.01f;   // above this share of non-zeros the dense kernels are used
 // fills words from g
 int launch_nonzero_scan(const float* g, unsigned* words, int B, int L, hipStream_t s);
-// the masks to use (the caller's, or a scan of g into a workspace) and their number of set bits;
-// synchronises the stream
-int nonzero_count(const float* g, const unsigned* given_words, int B, int L, hipStream_t s, const unsigned** words_out,
-                  unsigned long long* count_out);
+// the masks to use (the caller's, or a scan of g into a workspace) and their number of set bits.  Synchronises the
+// stream, unless `lagged` and an earlier call of the same shape on this stream has left its count: that one is
+// returned then, without waiting (this call's count is left for the next one)
+int nonzero_count(const float* g, const unsigned* given_words, int B, int L, hipStream_t s, bool lagged,
+                  const unsigned** words_out, unsigned long long* count_out);
+// drops the counts remembered for a device (the next lagged call waits again)
+void nonzero_count_forget(int device);
 // active == null: every row of gw is written (zeros for labels without a set bit).  active != null ([L] bytes):
 // only the rows of labels with a set bit are written and active[j] tells which
 int launch_weight_grad_sparse(const float* x, const int32_t* idx, const float* g, const unsigned* words, float* gw,

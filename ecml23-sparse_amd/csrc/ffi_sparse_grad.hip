@@ -22,6 +22,7 @@
 
 #include <algorithm>
 #include <mutex>
+#include <vector>
 
 namespace ffi {
 namespace {
@@ -372,9 +373,16 @@ __global__ __launch_bounds__(256) void igrad_sparse_reduce_kernel(const float* _
     gx[tp ? (size_t)n * B + b : i] = t;
 }
 
-// pinned word the set-bit count is copied to; one per device, calls on a device take turns
+// Pinned words the set-bit counts are written to by the count kernel, one per (device, stream), together with
+// the shape of the call that wrote it: a later call on the same stream may decide from it without waiting.
+struct CountSlot {
+    int device;
+    hipStream_t stream;
+    unsigned long long* host;    // hipHostMalloc'ed, written by nz_count_finish_kernel
+    int B, L;                    // shape of the last call (0: none yet)
+};
 std::mutex g_count_mutex;
-unsigned long long* g_count_host[64] = {nullptr};
+std::vector<CountSlot> g_count_slots;
 
 }  // namespace
 
@@ -393,11 +401,11 @@ int launch_zero_unmasked(float* g, const unsigned* words, int B, int L, hipStrea
     return FFI_OK;
 }
 
-int nonzero_count(const float* g, const unsigned* given_words, int B, int L, hipStream_t s, const unsigned** words_out,
-                  unsigned long long* count_out) {
+int nonzero_count(const float* g, const unsigned* given_words, int B, int L, hipStream_t s, bool lagged,
+                  const unsigned** words_out, unsigned long long* count_out) {
     const int nbt = (B + 31) / 32;
     int dev = -1;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return FFI_ERR_NO_DEVICE;
+    if (hipGetDevice(&dev) != hipSuccess) return FFI_ERR_NO_DEVICE;
     const size_t head = (size_t)kCountBlocks * sizeof(unsigned long long);           // block counts
     const size_t words_bytes = (size_t)nbt * L * sizeof(unsigned);
     unsigned char* ws = nullptr;
@@ -411,15 +419,37 @@ int nonzero_count(const float* g, const unsigned* given_words, int B, int L, hip
     }
     *words_out = words;
     std::lock_guard<std::mutex> lock(g_count_mutex);
-    if (!g_count_host[dev]) {
-        if (hipHostMalloc((void**)&g_count_host[dev], 64) != hipSuccess) { (void)hipGetLastError(); return FFI_ERR_OUT_OF_MEMORY; }
+    CountSlot* slot = nullptr;
+    for (CountSlot& c : g_count_slots)
+        if (c.device == dev && c.stream == s) slot = &c;
+    if (!slot) {
+        CountSlot c{dev, s, nullptr, 0, 0};
+        if (hipHostMalloc((void**)&c.host, 64) != hipSuccess) { (void)hipGetLastError(); return FFI_ERR_OUT_OF_MEMORY; }
+        *c.host = 0;
+        g_count_slots.push_back(c);
+        slot = &g_count_slots.back();
     }
+    // the count of an earlier call of the same shape on this stream, read before this call's kernels can overwrite it
+    const bool use_previous = lagged && slot->B == B && slot->L == L;
+    const unsigned long long previous = *reinterpret_cast<volatile unsigned long long*>(slot->host);
     hipLaunchKernelGGL(nz_count_kernel, dim3(kCountBlocks), dim3(kScanThreads), 0, s, words, (size_t)nbt * L, block_counts);
-    hipLaunchKernelGGL(nz_count_finish_kernel, dim3(1), dim3(64), 0, s, block_counts, kCountBlocks, g_count_host[dev]);
+    hipLaunchKernelGGL(nz_count_finish_kernel, dim3(1), dim3(64), 0, s, block_counts, kCountBlocks, slot->host);
     FFI_HIP_TRY(hipGetLastError());
+    if (use_previous) {
+        *count_out = previous;
+        return FFI_OK;
+    }
     FFI_HIP_TRY(hipStreamSynchronize(s));
-    *count_out = *reinterpret_cast<volatile unsigned long long*>(g_count_host[dev]);
+    *count_out = *reinterpret_cast<volatile unsigned long long*>(slot->host);
+    slot->B = B;
+    slot->L = L;
     return FFI_OK;
+}
+
+void nonzero_count_forget(int device) {
+    std::lock_guard<std::mutex> lock(g_count_mutex);
+    for (CountSlot& c : g_count_slots)
+        if (c.device == device) { c.B = 0; c.L = 0; }
 }
 
 int launch_weight_grad_sparse(const float* x, const int32_t* idx, const float* g, const unsigned* words, float* gw,

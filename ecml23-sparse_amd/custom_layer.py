@@ -162,7 +162,7 @@ class StratifiedRewireLayerV2(torch.nn.Module):
             inputs, indices, weights, out_grad, masks, optimizer._momentums[iw], optimizer._velocities[iw],
             bias, optimizer._momentums[ib] if self.use_bias else None, optimizer._velocities[ib] if self.use_bias else None,
             optimizer.learning_rate, optimizer.beta_1, optimizer.beta_2, optimizer.epsilon, optimizer.iterations + 1,
-            grad_is_partial=True, need_feature_grad=need_input_grad)
+            grad_is_partial=True, need_feature_grad=need_input_grad, decide_from_previous=True)
         return loss_sum[0] / (inputs.shape[0] * self.units), input_grad
 
     # sparse/layer.py:215-219, 236-237 and sparse/custom_layer.py:20-43

@@ -275,7 +275,7 @@ def fan_in_sparse_matmul_tp_bias(features, lookup, weights, bias):
 
 
 def backward_sparse(features, lookup, weights, out_grad, nz_words=None, max_density=None, transposed=False,
-                    need_feature_grad=True, need_bias_grad=False, grad_is_partial=False):
+                    need_feature_grad=True, need_bias_grad=False, grad_is_partial=False, decide_from_previous=False):
     """Backward pass that walks only the non-zero entries of ``out_grad`` (what the reference's GPU
     kernels do entry by entry, tfsparse/cc/kernels/backward.cu.h:73,94,131,151).
 
@@ -283,7 +283,9 @@ def backward_sparse(features, lookup, weights, out_grad, nz_words=None, max_dens
     saves the scan of ``out_grad``.  Above ``max_density`` (share of non-zeros; default: the
     library's) the dense kernels run instead.  ``grad_is_partial``: ``out_grad`` holds values only where
     ``nz_words`` has a bit set (``metrics.forward_loss(..., skip_zero_stores=True)``); the call may then
-    write zeros into the rest of it.  Returns ``(feature_grad or None, weight_grad,
+    write zeros into the rest of it.  ``decide_from_previous``: choose between sparse and dense kernels
+    from the count of non-zeros the previous call of this shape on the stream found, so that the host
+    does not wait (same results; the first call of a shape still waits).  Returns ``(feature_grad or None, weight_grad,
     bias_grad or None, sparse_kernels_ran)``."""
     import ctypes
 
@@ -299,7 +301,8 @@ def backward_sparse(features, lookup, weights, out_grad, nz_words=None, max_dens
         bias_grad = torch.empty((num_units,), dtype=torch.float32, device=features.device) if need_bias_grad else None
         _lib.check(_lib.lib().ffi_backward_sparse_f32(
             features.data_ptr(), lookup.data_ptr(), weights.data_ptr(), out_grad.data_ptr(),
-            nz_words.data_ptr() if nz_words is not None else None, int(bool(grad_is_partial)), float(max_density or 0.0),
+            nz_words.data_ptr() if nz_words is not None else None,
+            int(bool(grad_is_partial)) | (2 if decide_from_previous else 0), float(max_density or 0.0),
             feature_grad.data_ptr() if need_feature_grad else None, weight_grad.data_ptr(),
             bias_grad.data_ptr() if need_bias_grad else None, ctypes.byref(taken),
             batch, num_features, num_units, fan_in, int(transposed), _stream_handle(features.device)))

@@ -143,7 +143,8 @@ class _LayerLossFn(torch.autograd.Function):
         feature_grad, weight_grad, bias_grad, _ = backward_sparse(features, lookup, weights, g, nz_words=masks,
                                                                   transposed=ctx.transposed,
                                                                   need_feature_grad=ctx.needs_input_grad[0],
-                                                                  need_bias_grad=ctx.has_bias, grad_is_partial=True)
+                                                                  need_bias_grad=ctx.has_bias, grad_is_partial=True,
+                                                                  decide_from_previous=True)
         return feature_grad, None, weight_grad, bias_grad, None, None, None, None, None
 
 

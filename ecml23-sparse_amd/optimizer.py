@@ -70,7 +70,7 @@ class SparseAdam:
 
 def backward_sparse_adam(features, lookup, weights, out_grad, nz_words, weight_m, weight_v, bias, bias_m, bias_v,
                          learning_rate, beta_1, beta_2, epsilon, step, transposed=False, grad_is_partial=False,
-                         max_density=None, need_feature_grad=True):
+                         max_density=None, need_feature_grad=True, decide_from_previous=False):
     """Backward pass of the layer and the Adam step on its weights (and bias, unless ``None``) in one call:
     ``weights``, ``bias`` and their moments are updated in place; the weight/bias gradients stay inside the
     library (gradient rows of labels without a non-zero entry of ``out_grad`` are neither written nor read).  Returns ``(feature_grad or None, sparse_kernels_ran)``;
@@ -96,7 +96,8 @@ def backward_sparse_adam(features, lookup, weights, out_grad, nz_words, weight_m
         feature_grad = torch.empty_like(features) if need_feature_grad else None
         _lib.check(_lib.lib().ffi_backward_sparse_adam_f32(
             features.data_ptr(), lookup.data_ptr(), weights.data_ptr(), out_grad.data_ptr(),
-            nz_words.data_ptr() if nz_words is not None else None, int(bool(grad_is_partial)), float(max_density or 0.0),
+            nz_words.data_ptr() if nz_words is not None else None,
+            int(bool(grad_is_partial)) | (2 if decide_from_previous else 0), float(max_density or 0.0),
             feature_grad.data_ptr() if need_feature_grad else None, weight_m.data_ptr(), weight_v.data_ptr(),
             bias.data_ptr() if bias is not None else None, bias_m.data_ptr() if bias is not None else None,
             bias_v.data_ptr() if bias is not None else None,

@@ -236,18 +236,27 @@ int ffi_forward_loss_f32(const float* features, const int32_t* lookup, const flo
  *   nz_words      the masks of the non-zero entries as ffi_forward_loss_f32 / ffi_loss_grad_f32 write
  *                 them (a set bit over a zero entry is allowed, a clear bit over a non-zero entry is
  *                 not), or NULL: out_grad is then scanned first (one read of the matrix);
- *   grad_is_partial  != 0: out_grad holds values only where nz_words (required then) has a bit set, as
- *                 ffi_forward_loss_f32 leaves it with FFI_LOSS_SKIP_ZERO_STORES; if the dense kernels have
- *                 to run, the call first writes zeros into out_grad wherever the bit is clear;
+ *   flags         FFI_SPARSE_GRAD_IS_PARTIAL: out_grad holds values only where nz_words (required then) has a
+ *                 bit set, as ffi_forward_loss_f32 leaves it with FFI_LOSS_SKIP_ZERO_STORES; if the dense
+ *                 kernels have to run, the call first writes zeros into out_grad wherever the bit is clear.
+ *                 FFI_SPARSE_DECIDE_FROM_PREVIOUS: choose the kernels from the number of set bits that the
+ *                 previous call of the same shape on this stream found, without waiting for this call's
+ *                 number (the first call of a shape still waits).  Results are the same either way -- the
+ *                 sparse kernels are correct at any density -- only a sudden jump in density costs one slow
+ *                 call; sparse_path_taken then reports the choice made;
  *   max_density   share of set bits up to which the sparse kernels are used (<= 0: library default);
  *                 above it the call runs the dense kernels of ffi_backward_bias_f32;
  *   sparse_path_taken  HOST int, may be NULL: 1 if the sparse kernels ran, 0 if the dense ones did.
- * Synchronises `stream` once (the host reads the number of set bits).  The sparse input gradient
+ * Synchronises `stream` once (the host reads the number of set bits), except as described under flags.  The sparse input gradient
  * covers num_features <= 3072; wider inputs take the dense input-gradient kernels.  It accumulates
  * with LDS float adds issued in a fixed order, no global atomics.
  */
+enum ffi_sparse_flags {
+    FFI_SPARSE_GRAD_IS_PARTIAL = 1,
+    FFI_SPARSE_DECIDE_FROM_PREVIOUS = 2
+};
 int ffi_backward_sparse_f32(const float* features, const int32_t* lookup, const float* weights,
-                            float* out_grad, const uint32_t* nz_words, int grad_is_partial, float max_density,
+                            float* out_grad, const uint32_t* nz_words, int flags, float max_density,
                             float* feature_grad, float* weight_grad, float* bias_grad, int* sparse_path_taken,
                             int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in,
                             int transposed, ffi_stream_t stream);
@@ -262,7 +271,7 @@ int ffi_backward_sparse_f32(const float* features, const int32_t* lookup, const 
  * No counterpart in the reference, where the optimizer is a separate TensorFlow op.
  */
 int ffi_backward_sparse_adam_f32(const float* features, const int32_t* lookup, float* weights, float* out_grad,
-                                 const uint32_t* nz_words, int grad_is_partial, float max_density,
+                                 const uint32_t* nz_words, int flags, float max_density,
                                  float* feature_grad, float* weight_m, float* weight_v,
                                  float* bias, float* bias_m, float* bias_v,
                                  float learning_rate, float beta_1, float beta_2, float epsilon, int64_t step,

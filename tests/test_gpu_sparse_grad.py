@@ -209,3 +209,21 @@ def test_gradient_stored_only_where_it_is_not_zero(ffi, force_dense):
     assert sparse == (not force_dense)
     assert rel_err(gw.cpu().numpy(), ref_gw) <= GRAD_RTOL and rel_err(gx.cpu().numpy(), ref_gx) <= GRAD_RTOL
     assert rel_err(gb.cpu().numpy(), g_full.cpu().numpy().astype(np.float64).sum(axis=0)) <= GRAD_RTOL
+
+
+def test_deciding_from_the_previous_call_gives_the_same_results(ffi):
+    # the first call of a shape waits for its own count; later ones use the count left behind: a dense gradient
+    # after sparse ones is still computed correctly (by the sparse kernels, once), then the dense kernels take over
+    shape = (64, 256, 1500, 24, True)
+    dev = lambda a: torch.from_numpy(a).cuda()  # noqa: E731
+    taken = []
+    for density in (0.002, 0.003, 0.4, 0.4, 0.002):
+        feats, lookup, w, g = make_case(shape, density, seed=int(density * 1e4))
+        ref_gx, ref_gw = oracle.backward(feats, lookup, w, g, transposed=True)
+        gx, gw, gb, sparse = ffi.backward_sparse(dev(feats), dev(lookup), dev(w), dev(g), transposed=True, need_bias_grad=True,
+                                                 max_density=0.05, decide_from_previous=True)
+        torch.cuda.synchronize()
+        taken.append(sparse)
+        assert rel_err(gw.cpu().numpy(), ref_gw) <= GRAD_RTOL and rel_err(gx.cpu().numpy(), ref_gx) <= GRAD_RTOL
+        assert rel_err(gb.cpu().numpy(), g.astype(np.float64).sum(axis=0)) <= GRAD_RTOL
+    assert taken == [True, True, True, False, False]
