@@ -94,7 +94,7 @@ int launch_forward_loss(const float* x, const int32_t* idx, const float* w, cons
 
 // ---- backward pass over the non-zero entries of out_grad only (ffi_sparse_grad.hip) -------------
 // words[t][j]: bit i set <=> out_grad[32 t + i, j] may be non-zero
-constexpr int kSparseMaxFeatures = 3072;   // the sparse input gradient keeps 8 x N floats in LDS
+constexpr int kSparseMaxFeatures = 4096;   // the sparse input gradient keeps 8 x N floats in LDS
 constexpr float kSparseDefaultMaxDensity = 0.01f;   // above this share of non-zeros the dense kernels are used
 // fills words from g
 int launch_nonzero_scan(const float* g, unsigned* words, int B, int L, hipStream_t s);

@@ -13,8 +13,8 @@
 //                           (one chunk of connections) in registers; labels with many set bits are done by
 //                           the whole wavefront afterwards, lane <-> connection; rows of labels without a
 //                           set bit come out as zeros
-//   igrad_sparse_kernel     one workgroup per (sample, label segment): expands the sample's set bits to a list
-//                           of labels, then lanes <-> (label, connection) add g * w into per-wavefront
+//   igrad_sparse_kernel     one workgroup per (sample, label segment): every lane takes labels from its own word of
+//                           the sample's bit row and adds g * w of the label's connections into per-wavefront
 //                           accumulators gx[n] in LDS (LDS float adds issued in a fixed order)
 //   igrad_sparse_reduce_kernel  sums the segments in ascending order into feature_grad
 #include "ffi_internal.h"
@@ -191,13 +191,28 @@ __global__ __launch_bounds__(256, 4) void wgrad_sparse_kernel(const float* __res
             float acc[32];
 #pragma unroll
             for (int k = 0; k < 32; ++k) acc[k] = 0.f;
-            for (int t = 0; t < nbt; ++t) {
-                unsigned m = light ? words[(size_t)t * L + j] : 0u;
-                if (t == nbt - 1) m &= tail;
-                while (__ballot(m != 0)) {
-                    if (m) {
-                        const int b = 32 * t + __ffs((int)m) - 1;
-                        m &= m - 1;
+            // the label's mask words, eight batch tiles at a time in registers; every step each lane takes the
+            // next set bit of its own label (g and the 32 gathered x values are requested together)
+            for (int tb = 0; tb < nbt; tb += 8) {
+                unsigned mw[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int t = tb + u;
+                    mw[u] = (light && cnt && t < nbt) ? words[(size_t)t * L + j] : 0u;
+                    if (t == nbt - 1) mw[u] &= tail;
+                }
+                for (;;) {
+                    int usel = -1;
+                    unsigned msel = 0;
+#pragma unroll
+                    for (int u = 7; u >= 0; --u)
+                        if (mw[u]) { usel = u; msel = mw[u]; }
+                    if (!__ballot(usel >= 0)) break;
+                    if (usel >= 0) {
+                        const int b = 32 * (tb + usel) + __ffs((int)msel) - 1;
+#pragma unroll
+                        for (int u = 0; u < 8; ++u)
+                            if (u == usel) mw[u] = msel & (msel - 1);
                         const float gv = g[(size_t)b * L + j];
                         const unsigned xrow = (unsigned)b * xsb;
                         // 16 gathers in flight at a time
@@ -274,82 +289,61 @@ __global__ __launch_bounds__(256, 4) void wgrad_sparse_kernel(const float* __res
 
 constexpr int kSgThreads = 512;
 constexpr int kSgWaves = kSgThreads / 64;
-constexpr int kSgChunkWords = 256;                     // 64-bit words expanded per round (one per thread of the first 256)
-constexpr int kSgListCap = kSgChunkWords * 64;         // labels of one round
-constexpr int kSgUnroll = 4;                           // entries a lane has in flight
 
+// One workgroup per (sample, label segment).  Every wavefront walks its own share of the sample's bit row, 64 words
+// (4096 labels) at a time, one word per lane; at every step each lane with a bit left takes its next label, loads
+// that label's row of idx / w (a 32-connection chunk at a time) and adds g * w into the wavefront's own
+// accumulators gx[n] in LDS.  No barriers inside the walk; the order of the adds is fixed by the lane
+// assignment.  The wavefronts' accumulators are summed in ascending order at the end.
+template <bool VEC4>
 __global__ __launch_bounds__(kSgThreads) void igrad_sparse_kernel(const unsigned long long* __restrict__ bits, int nwords,
                                                                   const int32_t* __restrict__ idx,
                                                                   const float* __restrict__ w, const float* __restrict__ g,
                                                                   float* __restrict__ partial, int B, int N, int L, int K,
-                                                                  int S, int words_per_seg, int kp) {
+                                                                  int S, int words_per_seg) {
     extern __shared__ __align__(16) unsigned char sg_lds[];
     float* acc = reinterpret_cast<float*>(sg_lds);                                        // [kSgWaves][N]
-    unsigned short* list = reinterpret_cast<unsigned short*>(acc + (size_t)kSgWaves * N);   // [kSgListCap]
-    __shared__ int wave_total[kSgWaves];
     const int b = blockIdx.x / S, seg = blockIdx.x % S;
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     for (int i = threadIdx.x; i < kSgWaves * N; i += kSgThreads) acc[i] = 0.f;
+    __syncthreads();
     const int w_begin = seg * words_per_seg;
     const int w_end = min(w_begin + words_per_seg, nwords);
     const unsigned long long* row = bits + (size_t)b * nwords;
     const float* grow = g + (size_t)b * L;
     float* myacc = acc + (size_t)wv * N;
-    // kp = fan-in rounded up to a power of two (at most 64): kp lanes per entry, 64 / kp entries per step
-    const int sub = lane / kp, kl = lane % kp, per = 64 / kp;
-    for (int w0 = w_begin; w0 < w_end; w0 += kSgChunkWords) {
-        const int wi = w0 + (int)threadIdx.x;
-        unsigned long long m = (threadIdx.x < kSgChunkWords && wi < w_end) ? row[wi] : 0ull;
-        const int c = __popcll(m);
-        // exclusive prefix of c over the workgroup
-        int incl = c;
+    for (int w0 = w_begin + wv * 64; w0 < w_end; w0 += kSgWaves * 64) {
+        const int wi = w0 + lane;
+        unsigned long long m = wi < w_end ? row[wi] : 0ull;
+        while (__ballot(m != 0)) {
+            if (m) {
+                const int j = wi * 64 + __ffsll((long long)m) - 1;
+                m &= m - 1;
+                const float gv = grow[j];
+                const size_t at = (size_t)j * K;
+                for (int k0 = 0; k0 < K; k0 += 32) {
+                    unsigned n[32];
+                    float wk[32];
+                    if (VEC4 && k0 + 32 <= K) {
 #pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            const int up = __shfl_up(incl, off, 64);
-            if (lane >= off) incl += up;
-        }
-        __syncthreads();                                   // the previous round's list and totals are no longer read
-        if (lane == 63) wave_total[wv] = incl;
-        __syncthreads();
-        int before = 0, total = 0;
+                        for (int q = 0; q < 8; ++q) {
+                            const int4 v = *reinterpret_cast<const int4*>(idx + at + k0 + 4 * q);
+                            const float4 f = *reinterpret_cast<const float4*>(w + at + k0 + 4 * q);
+                            n[4 * q] = (unsigned)v.x; n[4 * q + 1] = (unsigned)v.y; n[4 * q + 2] = (unsigned)v.z; n[4 * q + 3] = (unsigned)v.w;
+                            wk[4 * q] = f.x; wk[4 * q + 1] = f.y; wk[4 * q + 2] = f.z; wk[4 * q + 3] = f.w;
+                        }
+                    } else {
 #pragma unroll
-        for (int i = 0; i < kSgWaves; ++i) {
-            if (i < wv) before += wave_total[i];
-            total += wave_total[i];
-        }
-        int pos = before + incl - c;
-        const unsigned short rel = (unsigned short)(threadIdx.x * 64);
-        while (m) {
-            list[pos++] = (unsigned short)(rel + (__ffsll((long long)m) - 1));
-            m &= m - 1;
-        }
-        __syncthreads();
-        // wavefront wv takes a contiguous share of the listed labels
-        const int e_begin = (int)((long long)total * wv / kSgWaves);
-        const int e_end = (int)((long long)total * (wv + 1) / kSgWaves);
-        const int jbase = w0 * 64;
-        for (int e0 = e_begin + sub; e0 < e_end; e0 += per * kSgUnroll) {
-            int jj[kSgUnroll];
-            float gv[kSgUnroll];
+                        for (int k = 0; k < 32; ++k) {
+                            const bool in = k0 + k < K;
+                            n[k] = in ? (unsigned)idx[at + k0 + k] : 0xffffffffu;
+                            wk[k] = in ? w[at + k0 + k] : 0.f;
+                        }
+                    }
 #pragma unroll
-            for (int u = 0; u < kSgUnroll; ++u) {
-                const int e = e0 + u * per;
-                jj[u] = e < e_end ? jbase + list[e] : -1;
-            }
-#pragma unroll
-            for (int u = 0; u < kSgUnroll; ++u) gv[u] = jj[u] >= 0 ? grow[jj[u]] : 0.f;
-            for (int k = kl; k < K; k += kp) {
-                unsigned n[kSgUnroll];
-                float wk[kSgUnroll];
-#pragma unroll
-                for (int u = 0; u < kSgUnroll; ++u) {
-                    const size_t at = (size_t)(jj[u] >= 0 ? jj[u] : 0) * K + k;
-                    n[u] = (unsigned)idx[at];
-                    wk[u] = w[at];
+                    for (int k = 0; k < 32; ++k)
+                        if (n[k] < (unsigned)N) atomicAdd(&myacc[n[k]], gv * wk[k]);
                 }
-#pragma unroll
-                for (int u = 0; u < kSgUnroll; ++u)
-                    if (jj[u] >= 0 && n[u] < (unsigned)N) atomicAdd(&myacc[n[u]], gv[u] * wk[u]);
             }
         }
     }
@@ -480,7 +474,7 @@ int launch_input_grad_sparse(const int32_t* idx, const float* w, const float* g,
     const int nwords = (d.L + 63) / 64;
     // label segments per sample: enough workgroups to fill the GPU, each with at least one round of words
     int S = std::max(1, (4 * device_cu_count() + d.B - 1) / d.B);
-    S = std::max(1, std::min(S, (nwords + kSgChunkWords - 1) / kSgChunkWords));
+    S = std::max(1, std::min(S, (nwords + kSgWaves * 64 - 1) / (kSgWaves * 64)));
     const int words_per_seg = (nwords + S - 1) / S;
     S = (nwords + words_per_seg - 1) / words_per_seg;
     const size_t bits_bytes = (size_t)d.B * nwords * sizeof(unsigned long long);
@@ -491,12 +485,17 @@ int launch_input_grad_sparse(const int32_t* idx, const float* w, const float* g,
     float* partial = reinterpret_cast<float*>(ws + bits_bytes);
     hipLaunchKernelGGL(nz_transpose_kernel, dim3((nwords + 3) / 4, nbt), dim3(kScanThreads), 0, s, words, bits, d.B, d.L, nwords);
     FFI_HIP_TRY(hipGetLastError());
-    int kp = 1;
-    while (kp < d.K && kp < 64) kp *= 2;
-    const size_t lds = (size_t)kSgWaves * d.N * sizeof(float) + (size_t)kSgListCap * sizeof(unsigned short);
-    FFI_HIP_TRY(hipFuncSetAttribute((const void*)igrad_sparse_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(igrad_sparse_kernel, dim3(d.B * S), dim3(kSgThreads), lds, s, bits, nwords, idx, w, g, partial, d.B, d.N,
-                       d.L, d.K, S, words_per_seg, kp);
+    const size_t lds = (size_t)kSgWaves * d.N * sizeof(float);
+    const bool vec4 = (d.K % 4 == 0) && (((uintptr_t)w | (uintptr_t)idx) % 16 == 0);
+    if (vec4) {
+        FFI_HIP_TRY(hipFuncSetAttribute((const void*)igrad_sparse_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        hipLaunchKernelGGL(igrad_sparse_kernel<true>, dim3(d.B * S), dim3(kSgThreads), lds, s, bits, nwords, idx, w, g, partial, d.B,
+                           d.N, d.L, d.K, S, words_per_seg);
+    } else {
+        FFI_HIP_TRY(hipFuncSetAttribute((const void*)igrad_sparse_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        hipLaunchKernelGGL(igrad_sparse_kernel<false>, dim3(d.B * S), dim3(kSgThreads), lds, s, bits, nwords, idx, w, g, partial, d.B,
+                           d.N, d.L, d.K, S, words_per_seg);
+    }
     FFI_HIP_TRY(hipGetLastError());
     const size_t total = (size_t)d.B * d.N;
     hipLaunchKernelGGL(igrad_sparse_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, partial, S, d.B, d.N,

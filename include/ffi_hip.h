@@ -248,7 +248,7 @@ int ffi_forward_loss_f32(const float* features, const int32_t* lookup, const flo
  *                 above it the call runs the dense kernels of ffi_backward_bias_f32;
  *   sparse_path_taken  HOST int, may be NULL: 1 if the sparse kernels ran, 0 if the dense ones did.
  * Synchronises `stream` once (the host reads the number of set bits), except as described under flags.  The sparse input gradient
- * covers num_features <= 3072; wider inputs take the dense input-gradient kernels.  It accumulates
+ * covers num_features <= 4096; wider inputs take the dense input-gradient kernels.  It accumulates
  * with LDS float adds issued in a fixed order, no global atomics.
  */
 enum ffi_sparse_flags {
