@@ -121,7 +121,8 @@ template <int MAXT, int LPT>
 __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* __restrict__ lab16, const float* __restrict__ wp,
                                   const unsigned* __restrict__ slice_off,
                                   const float* __restrict__ g, float* __restrict__ partial, int B, int L,
-                                  int tile_labels, int tiles, int tiles_per_stream, int nbt, unsigned total_rows) {
+                                  int tile_labels, int tiles, int tiles_per_stream, int nbt, unsigned total_rows,
+                                  const unsigned short* __restrict__ rowpos, int zero_row) {
     extern __shared__ __align__(16) float gs[];
     char* gs_bytes = reinterpret_cast<char*>(gs);
     const int nthreads = blockDim.x;
@@ -154,8 +155,8 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
             if (jl < nl) load_rows32(g, L, b0, B, (unsigned)(j0 + jl), gbn[p]);
         }
         __syncthreads();                       // the previous tile is no longer being read
-        // rows `tile_labels` (even) and `tile_labels + 1` (odd) are all zero: the targets of padding slots
-        if (t == t_begin && threadIdx.x < 64) gs[tile_labels * kTileBatch + threadIdx.x] = 0.f;
+        // rows `zero_row` (even) and `zero_row + 1` (odd) are all zero: the targets of padding slots
+        if (t == t_begin && threadIdx.x < 64) gs[zero_row * kTileBatch + threadIdx.x] = 0.f;
         // gs[jl][c] = g[b0+c][j0+jl]: the rows were loaded coalesced along labels; 16-byte LDS writes
         // whose chunk order is skewed by the label id (no bank conflicts)
 #pragma unroll
@@ -164,7 +165,8 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
             if (jl < nl) {
                 const int r = jl & 7;
                 xor_permute_groups(gbn[p], r);
-                char* rowp = gs_bytes + ((unsigned)jl << 7);
+                // the label's row in LDS is the plan's choice (it balances the bank halves of every column)
+                char* rowp = gs_bytes + ((unsigned)rowpos[j0 + jl] << 7);
 #pragma unroll
                 for (int c = 0; c < 8; ++c)
                     *reinterpret_cast<float4*>(rowp + ((c ^ r) << 4)) =
@@ -210,7 +212,7 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
 #pragma unroll
             for (int q = 0; q < kAhead; ++q) {
                 const bool in = i + q < rows;                       // wave-uniform
-                const unsigned e = in ? e4[q] : (unsigned)tile_labels;
+                const unsigned e = in ? e4[q] : (unsigned)zero_row;
                 const float wv = in ? w4[q] : 0.f;
                 float4 xv[8];
                 igrad_reads(e, skewbase, xv);
@@ -258,14 +260,14 @@ int launch_tiled(const ffi_plan* p, const float* w, const float* g, float* gx, i
     FFI_HIP_TRY(hipFuncSetAttribute((const void*)igrad_permute_weights_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, chunk * 4));
     hipLaunchKernelGGL(igrad_permute_weights_kernel, dim3(p->tiles), dim3(p->threads), chunk * sizeof(float), s, p->pos16,
                        p->slice_off, w, wp, p->L, p->K, p->tile_labels, chunk);
-    const size_t lds = tile_lds_bytes(p->tile_labels + 2);      // + the two all-zero rows
+    const size_t lds = tile_lds_bytes(p->zero_row + 2);         // the tile's rows + the two all-zero rows
     const dim3 grid(streams * nbt), block(p->threads);
 #define FFI_LAUNCH_TILE(MAXT, LPT)                                                                                      \
     do {                                                                                                                \
         FFI_HIP_TRY(hipFuncSetAttribute((const void*)igrad_tile_kernel<MAXT, LPT>,                                      \
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));                        \
         hipLaunchKernelGGL((igrad_tile_kernel<MAXT, LPT>), grid, block, lds, s, p->lab16, wp, p->slice_off, g, \
-                           partial, B, p->L, p->tile_labels, p->tiles, tps, nbt, (unsigned)p->total_rows);                                       \
+                           partial, B, p->L, p->tile_labels, p->tiles, tps, nbt, (unsigned)p->total_rows, p->rowpos, p->zero_row);                                       \
     } while (0)
     // the plan sizes its tiles so that one of these fits: tile_labels <= LPT * threads
     if (p->threads <= 768) {

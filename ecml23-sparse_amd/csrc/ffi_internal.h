@@ -162,8 +162,10 @@ struct ffi_plan {
     int tiles = 0;            // ceil(L / tile_labels)
     long long total_rows = 0; // rows of 64 entries over all slices
     unsigned* slice_off = nullptr;       // [tiles*slices + 1] first row of each slice
-    unsigned short* lab16 = nullptr;     // [total_rows*64] label (inside the tile) of each slot; padding slots hold
-                                         // tile_labels + parity (two all-zero rows of the walking kernel)
+    unsigned short* lab16 = nullptr;     // [total_rows*64] LDS row (of the walking kernel's tile) of each slot's label;
+                                         // padding slots hold zero_row + parity (two all-zero rows)
+    unsigned short* rowpos = nullptr;    // [L] LDS row each label is staged into, inside its tile (see ffi_plan.hip)
+    int zero_row = 0;                    // first of the two all-zero rows = rows of the tile in LDS before them
     unsigned short* pos16 = nullptr;     // [total_rows*64] position (inside the tile's rows of lookup) of each slot;
                                          // kPadPos in padding slots
     // arranged copy of the column ids for the weight gradient (narrow inputs only, else null):

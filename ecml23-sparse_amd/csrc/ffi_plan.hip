@@ -88,12 +88,67 @@ __device__ __forceinline__ unsigned column_slots(unsigned thread, unsigned even,
     return max(first ? 2u * first - 1u : 0u, 2u * second);
 }
 
+// Which LDS row of the walking kernel's tile each label is staged into (rowpos[j], inside the label's tile).
+// The bank half a row lies in is the parity of its row number, and a column is walked fastest when its labels
+// split evenly between the halves (see above: every hole costs a slot).  The label's own parity would split a
+// column's labels like coin flips (about sqrt(n) excess); here the labels of a tile are taken in ascending order
+// and each goes to the half that the columns it feeds have used less so far (weighted sum over its connections
+// of even-count minus odd-count of the column), which keeps the columns that matter close to an even split.
+// Rows of a half are handed out in ascending order, at most `cap` per half.  One workgroup per tile; the tile's
+// column ids are staged in LDS, one wavefront then decides label after label (lane <-> connection).
+__global__ __launch_bounds__(256) void tile_color_kernel(const int32_t* __restrict__ idx, int L, int K, int tile_labels, int cap,
+                                                         int ncols, unsigned short* __restrict__ rowpos) {
+    extern __shared__ int color_lds[];
+    int* imb = color_lds;                                                        // [ncols] even minus odd labels per column
+    int* wt = color_lds + ncols;                                                 // [ncols] weight of the column's balance
+    unsigned short* ids = reinterpret_cast<unsigned short*>(color_lds + 2 * ncols);  // [tile_labels * K] column ids
+    const int t = blockIdx.x;
+    const int j0 = t * tile_labels;
+    const int nl = min(tile_labels, L - j0);
+    const int* src = idx + (size_t)j0 * K;
+    for (int i = threadIdx.x; i < ncols; i += 256) { imb[i] = 0; wt[i] = 0; }
+    __syncthreads();
+    for (int e = threadIdx.x; e < nl * K; e += 256) {
+        const int c = src[e];
+        ids[e] = (unsigned short)c;
+        atomicAdd(&wt[c], 1);                                                    // column lengths first
+    }
+    __syncthreads();
+    // Only the longest columns of a slice (64 columns, one wavefront of the walking kernel) set its number of slot
+    // rows, so their balance counts most: weight = 256 * (length / longest of the slice)^8.
+    for (int c = threadIdx.x; c < ncols; c += 256) {
+        const int len = wt[c];
+        int longest = len;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) longest = max(longest, __shfl_xor(longest, off, 64));
+        float r = longest > 0 ? (float)len / (float)longest : 0.f;
+        r *= r; r *= r; r *= r;
+        wt[c] = (int)(256.f * r);
+    }
+    __syncthreads();
+    if (threadIdx.x >= 64) return;
+    const int lane = threadIdx.x;
+    int placed[2] = {0, 0};
+    for (int jl = 0; jl < nl; ++jl) {
+        int sum = 0;
+        for (int k = lane; k < K; k += 64) { const int c = ids[jl * K + k]; sum += wt[c] * imb[c]; }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+        int color = sum > 0 ? 1 : (sum < 0 ? 0 : (placed[1] < placed[0] ? 1 : 0));
+        if (placed[color] >= cap) color ^= 1;
+        const int delta = color ? -1 : 1;
+        for (int k = lane; k < K; k += 64) atomicAdd(&imb[ids[jl * K + k]], delta);     // a column may occur twice in a label
+        if (lane == 0) rowpos[j0 + jl] = (unsigned short)(2 * placed[color] + color);
+        ++placed[color];
+    }
+}
+
 // One workgroup per label tile, one thread per column.  Counts the tile's connections per column
-// and label parity (integer LDS atomics: order-independent), stores the slot count of the longest
-// column of each slice.
-__global__ void tile_count_kernel(const int32_t* __restrict__ idx, int L, int K, int tile_labels,
-                                  unsigned* __restrict__ slice_len) {
-    extern __shared__ unsigned cnt[];          // [2][threads]: even labels, odd labels
+// and bank half of the label's row (integer LDS atomics: order-independent), stores the slot count of the
+// longest column of each slice.
+__global__ void tile_count_kernel(const int32_t* __restrict__ idx, const unsigned short* __restrict__ rowpos, int L, int K,
+                                  int tile_labels, unsigned* __restrict__ slice_len) {
+    extern __shared__ unsigned cnt[];          // [2][threads]: labels in even rows, labels in odd rows
     const int t = blockIdx.x, nthreads = blockDim.x;
     cnt[threadIdx.x] = 0;
     cnt[nthreads + threadIdx.x] = 0;
@@ -102,7 +157,8 @@ __global__ void tile_count_kernel(const int32_t* __restrict__ idx, int L, int K,
     const int nl = min(tile_labels, L - j0);
     const int* src = idx + (size_t)j0 * K;
     const int total = nl * K;
-    for (int e = threadIdx.x; e < total; e += nthreads) atomicAdd(&cnt[((e / K) & 1) * nthreads + (unsigned)src[e]], 1u);
+    for (int e = threadIdx.x; e < total; e += nthreads)
+        atomicAdd(&cnt[(rowpos[j0 + e / K] & 1u) * nthreads + (unsigned)src[e]], 1u);
     __syncthreads();
     const unsigned even = cnt[threadIdx.x], odd = cnt[nthreads + threadIdx.x];
     unsigned c = column_slots(threadIdx.x, even, odd);
@@ -135,14 +191,15 @@ __global__ __launch_bounds__(1024) void slice_scan_kernel(const unsigned* __rest
 // One workgroup per label tile, one thread per column n.  The tile's column ids pass through LDS
 // in chunks; every thread scans them in flat-position order and places the ones equal to its
 // column (see column_slots for the order), so the result is deterministic without any sort.
-// Per slot: lab16 = label inside the tile, pos16 = position inside the tile's rows of lookup; the
+// Per slot: lab16 = LDS row of the label (rowpos), pos16 = position inside the tile's rows of lookup; the
 // slots a column leaves empty up to the slice's length become padding: pos16 = kPadPos, lab16 =
-// tile_labels + parity (all-zero rows).
+// zero_row + parity (all-zero rows).
 constexpr int kFillChunk = 8192;
-__global__ void tile_fill_kernel(const int32_t* __restrict__ idx, int L, int K, int tile_labels,
-                                 const unsigned* __restrict__ slice_off, unsigned short* __restrict__ lab16,
-                                 unsigned short* __restrict__ pos16) {
+__global__ void tile_fill_kernel(const int32_t* __restrict__ idx, const unsigned short* __restrict__ rowpos, int L, int K,
+                                 int tile_labels, int zero_row, const unsigned* __restrict__ slice_off,
+                                 unsigned short* __restrict__ lab16, unsigned short* __restrict__ pos16) {
     __shared__ __align__(16) int keys[kFillChunk];
+    __shared__ unsigned short rows_of[kPlanTileLabels];     // LDS row of each label of the tile
     const int t = blockIdx.x, nthreads = blockDim.x;
     const int j0 = t * tile_labels;
     const int nl = min(tile_labels, L - j0);
@@ -155,9 +212,10 @@ __global__ void tile_fill_kernel(const int32_t* __restrict__ idx, int L, int K, 
     unsigned short* dlab = lab16 + row0 * 64 + (threadIdx.x & 63);
     unsigned short* dpos = pos16 + row0 * 64 + (threadIdx.x & 63);
     const unsigned first = parity_first(threadIdx.x);
+    for (int i = threadIdx.x; i < nl; i += nthreads) rows_of[i] = rowpos[j0 + i];
     // padding everywhere first; the thread's own slots are then overwritten (same thread: ordered)
     for (unsigned r = 0; r < rows; ++r) {
-        dlab[(size_t)r * 64] = (unsigned short)((unsigned)tile_labels + ((r & 1u) ^ first));
+        dlab[(size_t)r * 64] = (unsigned short)((unsigned)zero_row + ((r & 1u) ^ first));
         dpos[(size_t)r * 64] = (unsigned short)kPadPos;
     }
     unsigned seen[2] = {0u, 0u};  // labels of each parity placed so far
@@ -169,10 +227,11 @@ __global__ void tile_fill_kernel(const int32_t* __restrict__ idx, int L, int K, 
         __syncthreads();
         for (int e = 0; e < n; ++e) {
             if (keys[e] == mine) {
-                const unsigned par = (unsigned)label & 1u;
+                const unsigned row = rows_of[label];
+                const unsigned par = row & 1u;
                 const unsigned t2 = par ? seen[1]++ : seen[0]++;
                 const unsigned slot = 2u * t2 + (par ^ first);
-                dlab[(size_t)slot * 64] = (unsigned short)label;
+                dlab[(size_t)slot * 64] = (unsigned short)row;
                 dpos[(size_t)slot * 64] = (unsigned short)(c0 + e);
             }
             if (++kk == K) { kk = 0; ++label; }
@@ -208,6 +267,8 @@ void free_arrays(ffi_plan* p) {
     if (p->lab16) (void)hipFree(p->lab16);
     if (p->pos16) (void)hipFree(p->pos16);
     if (p->idx16) (void)hipFree(p->idx16);
+    if (p->rowpos) (void)hipFree(p->rowpos);
+    p->rowpos = nullptr;
     p->perm = nullptr; p->col_ptr = nullptr; p->slice_off = nullptr; p->lab16 = nullptr; p->pos16 = nullptr; p->idx16 = nullptr;
     p->tiled = false; p->total_rows = 0; p->bytes = 0;
 }
@@ -241,8 +302,17 @@ int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
         if (slice_len) (void)hipFree(slice_len);
         return FFI_ERR_OUT_OF_MEMORY;
     }
-    hipLaunchKernelGGL(tile_count_kernel, dim3(tiles), dim3(threads), 2 * threads * sizeof(unsigned), s, lookup, p->L, p->K,
-                       TL, slice_len);
+    // rows per bank half: half the tile plus some room for the balancing, within the LDS the walking kernel can have
+    const int cap = TL / 2 + std::min(TL / 16, 64);
+    if (!dev_alloc(&p->rowpos, (size_t)p->L)) { (void)hipFree(slice_len); return FFI_ERR_OUT_OF_MEMORY; }
+    {
+        const size_t lds = 2 * (size_t)threads * sizeof(int) + (size_t)TL * p->K * sizeof(unsigned short);
+        hipError_t ea = hipFuncSetAttribute((const void*)tile_color_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (ea != hipSuccess) { (void)hipFree(slice_len); return hip_fail(ea); }
+        hipLaunchKernelGGL(tile_color_kernel, dim3(tiles), dim3(256), lds, s, lookup, p->L, p->K, TL, cap, threads, p->rowpos);
+    }
+    hipLaunchKernelGGL(tile_count_kernel, dim3(tiles), dim3(threads), 2 * threads * sizeof(unsigned), s, lookup, p->rowpos, p->L,
+                       p->K, TL, slice_len);
     hipLaunchKernelGGL(slice_scan_kernel, dim3(1), dim3(1024), 0, s, slice_len, p->slice_off, (int)nslices,
                        p->d_scratch + 2);
     hipError_t e = hipGetLastError();
@@ -255,15 +325,15 @@ int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     // too skewed, or beyond what the walking kernel's 32-bit buffer offsets reach (256 bytes per row)
     if (rows * 64ull > 3ull * connections + 64ull * nslices || rows >= (1ull << 24)) return FFI_OK;
     if (!dev_alloc(&p->lab16, (size_t)rows * 64) || !dev_alloc(&p->pos16, (size_t)rows * 64)) return FFI_ERR_OUT_OF_MEMORY;
-    hipLaunchKernelGGL(tile_fill_kernel, dim3(tiles), dim3(threads), 0, s, lookup, p->L, p->K, TL, p->slice_off, p->lab16,
-                       p->pos16);
+    hipLaunchKernelGGL(tile_fill_kernel, dim3(tiles), dim3(threads), 0, s, lookup, p->rowpos, p->L, p->K, TL, 2 * cap, p->slice_off,
+                       p->lab16, p->pos16);
     e = hipGetLastError();
     if (e == hipSuccess) e = hipStreamSynchronize(s);
     if (e != hipSuccess) return hip_fail(e);
     p->tiled = true;
-    p->tile_labels = TL; p->threads = threads; p->slices = slices; p->tiles = tiles;
+    p->tile_labels = TL; p->threads = threads; p->slices = slices; p->tiles = tiles; p->zero_row = 2 * cap;
     p->total_rows = (long long)rows;
-    p->bytes = (size_t)rows * 64 * 2 * sizeof(unsigned short) + (nslices + 1) * sizeof(unsigned);
+    p->bytes = (size_t)rows * 64 * 2 * sizeof(unsigned short) + (nslices + 1) * sizeof(unsigned) + (size_t)p->L * sizeof(unsigned short);
     return FFI_OK;
 }
 
