@@ -205,7 +205,7 @@ enum ffi_loss_kind {
     FFI_LOSS_BCE = 3,             /* SparseBinaryCrossEntropyLoss  sparse/metrics.py:167-173 */
     /* flag for ffi_forward_loss_f32, OR-ed into loss_kind: gradients that are exactly zero are not stored
        (out_grad keeps what it held there); needs nz_words, which then says which entries were written.
-       Such an out_grad goes to ffi_backward_sparse_f32 with grad_is_partial != 0. */
+       Such an out_grad goes to ffi_backward_sparse_f32 with FFI_SPARSE_GRAD_IS_PARTIAL. */
     FFI_LOSS_SKIP_ZERO_STORES = 0x100
 };
 int ffi_loss_grad_f32(const float* scores, const int64_t* label_indices, const float* label_values, int64_t nnz,
