@@ -227,3 +227,49 @@ def test_deciding_from_the_previous_call_gives_the_same_results(ffi):
         assert rel_err(gw.cpu().numpy(), ref_gw) <= GRAD_RTOL and rel_err(gx.cpu().numpy(), ref_gx) <= GRAD_RTOL
         assert rel_err(gb.cpu().numpy(), g.astype(np.float64).sum(axis=0)) <= GRAD_RTOL
     assert taken == [True, True, True, False, False]
+
+
+def test_headline_config_full_size_training_step(ffi):
+    # 670,091 labels x fan-in 32 x 768 inputs x batch 128, gradient about 0.2 % non-zero: size-independent checks.
+    #   the fused loss forward (zero gradients not stored) agrees with forward + loss pass at every mask bit,
+    #   the masks cover exactly the non-zero gradients (plus listed positions), the loss sums agree;
+    #   the sparse backward agrees with the dense kernels on the same gradient, and with the adjoint identity
+    #   <out_grad, W x> = <gW, W> = <gx, x> (the layer is linear in x and in W)
+    from ecml23_sparse_amd import synth
+    cfg = synth.CONFIGS["c2"]
+    t = synth.make_inputs(cfg, seed=42, device="cuda", transposed=True)
+    x, lookup, w = t["features"], t["lookup"], t["weights"]
+    B, L = cfg.batch, cfg.num_units
+    scores0 = ffi.fan_in_sparse_matmul_tp(x, lookup, w)
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    sample = scores0.flatten()[torch.randint(0, B * L, (1 << 20,), device="cuda", generator=gen)]
+    bias = torch.full((L,), -1.0 - float(torch.quantile(sample, 0.998)), device="cuda")
+    rows = torch.arange(B, device="cuda").repeat_interleave(5)
+    y = (torch.stack([rows, torch.randint(0, L, (B * 5,), device="cuda", generator=gen)], dim=1), None)
+    kind = oracle.LOSS_SQUARED_HINGE
+    scores = ffi.fan_in_sparse_matmul_tp_bias(x, lookup, w, bias)
+    g_ref, loss_ref = ffi.metrics.sparse_loss_grad(scores, y, kind)
+    _, g, loss, masks = ffi.metrics.forward_loss(x, lookup, w, bias, y, kind, transposed=True, want_masks=True,
+                                                 skip_zero_stores=True)
+    torch.cuda.synchronize()
+    bit = (masks.view(B // 32, 1, L) >> torch.arange(32, device="cuda", dtype=torch.int32).view(1, 32, 1)) & 1
+    written = bit.reshape(B, L).bool()
+    density = float(written.float().mean())
+    assert 0.001 < density < 0.004
+    assert bool((written | (g_ref == 0)).all())                                  # every non-zero gradient is covered
+    scale = float(g_ref.abs().max())
+    assert float((g[written] - g_ref[written]).abs().max()) <= 4e-5 * scale       # scores differ by rounding only
+    assert abs(float(loss) - float(loss_ref)) <= 1e-5 * abs(float(loss_ref))
+    gx_s, gw_s, gb_s, sparse = ffi.backward_sparse(x, lookup, w, g, nz_words=masks, transposed=True, need_bias_grad=True,
+                                                   grad_is_partial=True)
+    assert sparse
+    g_full = torch.where(written, g, torch.zeros_like(g))
+    gx_d, gw_d = ffi.fan_in_sparse_matmul_grad_tp(x, lookup, w, g_full)
+    torch.cuda.synchronize()
+    assert rel_err(gw_s.cpu().numpy(), gw_d.cpu().numpy()) <= GRAD_RTOL
+    assert rel_err(gx_s.cpu().numpy(), gx_d.cpu().numpy()) <= GRAD_RTOL
+    assert rel_err(gb_s.cpu().numpy(), g_full.double().sum(dim=0).cpu().numpy()) <= GRAD_RTOL
+    a = float((scores0.double() * g_full.double()).sum())
+    b = float((x.double() * gx_s.double()).sum())
+    c = float((w.double() * gw_s.double()).sum())
+    assert abs(a - b) <= 1e-4 * abs(a) and abs(a - c) <= 1e-4 * abs(a)
