@@ -34,6 +34,8 @@ from .metrics import (  # noqa: E402
     SparseSquaredHingeLoss,
     SparseBinaryCrossEntropyLoss,
     PrecisionAtK,
+    SparsePrecision,
+    SparseRecall,
 )
 from .custom_layer import StratifiedRewireLayerV2, FixedFractionSelector, FixedMagnitudeSelector  # noqa: E402
 
@@ -58,5 +60,7 @@ __all__ = [
     "SparseSquaredHingeLoss",
     "SparseBinaryCrossEntropyLoss",
     "PrecisionAtK",
+    "SparsePrecision",
+    "SparseRecall",
     "SparseAdam",
 ]

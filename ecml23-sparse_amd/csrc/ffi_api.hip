@@ -256,6 +256,14 @@ int ffi_loss_grad_f32(const float* scores, const int64_t* label_indices, const f
     return launch_loss_grad(la, scores, out_grad, (int)batch, (int)num_units, (hipStream_t)stream);
 }
 
+int ffi_threshold_metrics_f32(const float* scores, const int64_t* label_indices, const float* label_values, int64_t nnz,
+                              float threshold, double* counts, int64_t batch, int64_t num_units, ffi_stream_t stream) {
+    if (!scores || !counts) return FFI_ERR_NULL_POINTER;
+    FFI_TRY(check_loss_args(label_indices, nnz, FFI_LOSS_HINGE, batch, num_units));
+    return launch_threshold_metrics(scores, label_indices, label_values, (int)nnz, threshold, (int)batch, (int)num_units, counts,
+                                    (hipStream_t)stream);
+}
+
 int ffi_forward_loss_f32(const float* features, const int32_t* lookup, const float* weights, const float* bias,
                          const int64_t* label_indices, const float* label_values, int64_t nnz, int loss_kind,
                          float grad_scale, float* scores, float* out_grad, float* loss_sum, uint32_t* nz_words,

@@ -88,6 +88,9 @@ int launch_loss_positives(const LossArgs& la, const float* saved, const float* s
                           double* corr, hipStream_t s);
 // g = scale * dloss/dscore for a whole score matrix (g may be the score buffer itself)
 int launch_loss_grad(const LossArgs& la, const float* scores, float* g, int B, int L, hipStream_t s);
+// out[3] (device doubles): scores above the threshold, sum of label values at such positions, sum of label values
+int launch_threshold_metrics(const float* scores, const int64_t* indices, const float* values, int nnz, float threshold, int B,
+                             int L, double* out, hipStream_t s);
 // forward pass whose epilogue turns the scores into loss gradients (scores may be null)
 int launch_forward_loss(const float* x, const int32_t* idx, const float* w, const float* bias, const LossArgs& la,
                         float* scores, float* g, const Dims& d, hipStream_t s);

@@ -130,7 +130,87 @@ __global__ __launch_bounds__(kFinishThreads) void loss_finish_kernel(const doubl
     }
 }
 
+// ---- thresholded precision / recall counts (SparsePrecision, SparseRecall: sparse/metrics.py:73-129) ----------
+// per wavefront: how many scores exceed the threshold
+__global__ __launch_bounds__(kLossThreads) void threshold_count_kernel(const float* __restrict__ scores, size_t total,
+                                                                       float threshold, unsigned long long* __restrict__ partial) {
+    const size_t nvec = total / 4;
+    const size_t stride = (size_t)gridDim.x * kLossThreads;
+    unsigned c = 0;
+    for (size_t v0 = (size_t)blockIdx.x * kLossThreads + threadIdx.x; v0 < nvec; v0 += stride * kLossVecPerThread) {
+        float4 s[kLossVecPerThread];
+#pragma unroll
+        for (int i = 0; i < kLossVecPerThread; ++i) {
+            const size_t v = v0 + (size_t)i * stride;
+            s[i] = v < nvec ? reinterpret_cast<const float4*>(scores)[v] : make_float4(threshold, threshold, threshold, threshold);
+        }
+#pragma unroll
+        for (int i = 0; i < kLossVecPerThread; ++i)
+            c += (s[i].x > threshold) + (s[i].y > threshold) + (s[i].z > threshold) + (s[i].w > threshold);
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (total & 3)) c += scores[nvec * 4 + threadIdx.x] > threshold;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) c += __shfl_xor(c, off, 64);
+    if ((threadIdx.x & 63) == 0) partial[blockIdx.x * (kLossThreads / 64) + (threadIdx.x >> 6)] = c;
+}
+
+// per listed label position: value * [score > threshold] and value
+__global__ __launch_bounds__(kLossThreads) void threshold_labels_kernel(const int64_t* __restrict__ label_indices,
+                                                                        const float* __restrict__ label_values, int nnz,
+                                                                        const float* __restrict__ scores, float threshold, int B,
+                                                                        int L, double* __restrict__ hit, double* __restrict__ val) {
+    const int p = blockIdx.x * kLossThreads + threadIdx.x;
+    if (p >= nnz) return;
+    const int64_t b = label_indices[2 * (size_t)p], j = label_indices[2 * (size_t)p + 1];
+    double h = 0.0, v = 0.0;
+    if (b >= 0 && b < B && j >= 0 && j < L) {
+        v = label_values ? (double)label_values[p] : 1.0;
+        h = scores[(size_t)b * L + j] > threshold ? v : 0.0;
+    }
+    hit[p] = h;
+    val[p] = v;
+}
+
+// out[0] = number of scores above the threshold, out[1] = sum of label values at such positions, out[2] = sum of label values
+__global__ __launch_bounds__(kFinishThreads) void threshold_finish_kernel(const unsigned long long* __restrict__ partial, int npartial,
+                                                                          const double* __restrict__ hit, const double* __restrict__ val,
+                                                                          int nnz, double* __restrict__ out) {
+    __shared__ double red[3][kFinishThreads / 64];
+    double a = 0.0, h = 0.0, v = 0.0;
+    for (int i = threadIdx.x; i < npartial; i += kFinishThreads) a += (double)partial[i];
+    for (int i = threadIdx.x; i < nnz; i += kFinishThreads) { h += hit[i]; v += val[i]; }
+    a = wave_sum(a); h = wave_sum(h); v = wave_sum(v);
+    if ((threadIdx.x & 63) == 0) { red[0][threadIdx.x >> 6] = a; red[1][threadIdx.x >> 6] = h; red[2][threadIdx.x >> 6] = v; }
+    __syncthreads();
+    if (threadIdx.x < 3) {
+        double t = 0.0;
+        for (int i = 0; i < kFinishThreads / 64; ++i) t += red[threadIdx.x][i];
+        out[threadIdx.x] = t;
+    }
+}
+
 }  // namespace
+
+int launch_threshold_metrics(const float* scores, const int64_t* indices, const float* values, int nnz, float threshold, int B,
+                             int L, double* out, hipStream_t s) {
+    const size_t total = (size_t)B * (size_t)L;
+    const size_t nvec = total / 4;
+    const size_t per_block = (size_t)kLossThreads * kLossVecPerThread;
+    const int blocks = (int)std::max<size_t>(1, std::min<size_t>((nvec + per_block - 1) / per_block, (size_t)device_cu_count() * 16));
+    const int npartial = blocks * (kLossThreads / 64);
+    unsigned char* ws = nullptr;
+    FFI_TRY(workspace_get(s, kWsLoss, ((size_t)npartial + 2 * (size_t)nnz + 2) * sizeof(double), (void**)&ws));
+    unsigned long long* partial = reinterpret_cast<unsigned long long*>(ws);
+    double* hit = reinterpret_cast<double*>(ws) + npartial;
+    double* val = hit + nnz;
+    hipLaunchKernelGGL(threshold_count_kernel, dim3(blocks), dim3(kLossThreads), 0, s, scores, total, threshold, partial);
+    if (nnz > 0)
+        hipLaunchKernelGGL(threshold_labels_kernel, dim3((nnz + kLossThreads - 1) / kLossThreads), dim3(kLossThreads), 0, s, indices,
+                           values, nnz, scores, threshold, B, L, hit, val);
+    hipLaunchKernelGGL(threshold_finish_kernel, dim3(1), dim3(kFinishThreads), 0, s, partial, npartial, hit, val, nnz, out);
+    FFI_HIP_TRY(hipGetLastError());
+    return FFI_OK;
+}
 
 int loss_partial_buffer(hipStream_t s, int npartial, int nnz, double** partial, double** corr, float** saved) {
     double* buf = nullptr;

@@ -228,3 +228,61 @@ class PrecisionAtK:
 
     def result(self):
         return self._correct / self._total if self._total else 0.0
+
+
+def threshold_counts(scores, y_true, threshold):
+    """Device tensor of three doubles: number of scores above ``threshold``, sum of the label values at
+    listed positions whose score is above it, sum of all label values (one pass over the scores)."""
+    if scores.dim() != 2 or scores.dtype != torch.float32 or not scores.is_cuda:
+        raise TypeError("scores must be a float32 [batch, num_units] device matrix")
+    scores = scores.contiguous()
+    batch, num_units = scores.shape
+    indices, values = _labels(y_true, scores.device)
+    with torch.cuda.device(scores.device):
+        counts = torch.empty((3,), dtype=torch.float64, device=scores.device)
+        _lib.check(_lib.lib().ffi_threshold_metrics_f32(
+            scores.data_ptr(), indices.data_ptr() if indices.numel() else None,
+            values.data_ptr() if values is not None and values.numel() else None, indices.shape[0], float(threshold),
+            counts.data_ptr(), batch, num_units, _stream_handle(scores.device)))
+    return counts
+
+
+class _ThresholdMetric:
+    def __init__(self, threshold, name):
+        self.name = name
+        self._threshold = float(threshold)
+        self.reset_state()
+
+    def reset_state(self):
+        self._correct = 0.0
+        self._total = 0.0
+
+    def result(self):
+        return self._correct / self._total if self._total else 0.0     # divide_no_nan
+
+
+class SparsePrecision(_ThresholdMetric):
+    """Label values at predicted positions (score > threshold) over the number of predicted positions,
+    accumulated over ``update_state`` calls (sparse/metrics.py:73-98)."""
+
+    def __init__(self, threshold, name=None):
+        super().__init__(threshold, name or "Precision")
+
+    def update_state(self, y_true, y_pred, sample_weight=None):
+        assert sample_weight is None
+        predicted, correct, _ = threshold_counts(y_pred, y_true, self._threshold).tolist()
+        self._correct += correct
+        self._total += predicted
+
+
+class SparseRecall(_ThresholdMetric):
+    """Label values at predicted positions over the sum of all label values (sparse/metrics.py:101-129)."""
+
+    def __init__(self, threshold, name=None):
+        super().__init__(threshold, name or "Recall")
+
+    def update_state(self, y_true, y_pred, sample_weight=None):
+        assert sample_weight is None
+        _, correct, total = threshold_counts(y_pred, y_true, self._threshold).tolist()
+        self._correct += correct
+        self._total += total

@@ -213,6 +213,17 @@ int ffi_loss_grad_f32(const float* scores, const int64_t* label_indices, const f
                       int64_t batch, int64_t num_units, ffi_stream_t stream);
 
 /*
+ * The counts behind the reference's thresholded metrics (SparsePrecision.update_state, sparse/metrics.py:88-96;
+ * SparseRecall.update_state, :119-126), from one pass over the scores.  counts (three doubles on the device):
+ *   counts[0]  number of scores > threshold                        (precision's denominator)
+ *   counts[1]  sum of label values at listed positions whose score > threshold   (the numerator of both)
+ *   counts[2]  sum of all label values                             (recall's denominator)
+ * label_indices / label_values / nnz as for ffi_loss_grad_f32.
+ */
+int ffi_threshold_metrics_f32(const float* scores, const int64_t* label_indices, const float* label_values, int64_t nnz,
+                              float threshold, double* counts, int64_t batch, int64_t num_units, ffi_stream_t stream);
+
+/*
  * Forward pass, bias add and loss gradient in one pass (no counterpart in the reference, where they
  * are three TensorFlow ops and the [batch, num_units] score matrix makes two more trips through
  * memory): the forward kernel turns each finished score into its loss gradient before storing it.

@@ -286,3 +286,15 @@ def select_threshold(weights, k):
 def rewire_selection(weights, threshold):
     """Boolean mask of the connections that are rewired: strictly below the threshold (sparse/layer.py:57,86)."""
     return np.abs(np.asarray(weights, dtype=np.float32)) < np.float32(threshold)
+
+
+def threshold_counts(scores, label_indices, label_values, threshold):
+    """(predicted, correct, total_true) as SparsePrecision / SparseRecall accumulate them (sparse/metrics.py:88-96,
+    113-126): predicted = count(scores > threshold); correct = sum of label values at listed positions whose score
+    is above the threshold; total_true = sum of all label values."""
+    s = np.asarray(scores)
+    idx = np.asarray(label_indices, dtype=np.int64).reshape(-1, 2)
+    vals = np.ones(len(idx)) if label_values is None else np.asarray(label_values, dtype=np.float64)
+    predicted = float(np.count_nonzero(s > np.float32(threshold)))
+    hit = s[idx[:, 0], idx[:, 1]] > np.float32(threshold) if len(idx) else np.zeros(0, bool)
+    return predicted, float((vals * hit).sum()), float(vals.sum())

@@ -229,3 +229,25 @@ def test_precision_at_k(ffi, k):
     assert abs(metric.result() - expected) < 1e-12
     metric.update_state((torch.from_numpy(indices).cuda(), None), torch.from_numpy(scores).cuda())
     assert abs(metric.result() - expected) < 1e-12          # accumulates numerator and denominator
+
+
+@pytest.mark.parametrize("shape", [(128, 5000), (37, 1001), (1, 3)])
+@pytest.mark.parametrize("threshold", [0.0, 0.7])
+def test_threshold_metrics_against_oracle(ffi, shape, threshold):
+    # SparsePrecision / SparseRecall (sparse/metrics.py:73-129): exact counts, so exact equality
+    B, L = shape
+    rng = np.random.default_rng(B + L)
+    scores = rng.normal(0, 1, (B, L)).astype(np.float32)
+    scores[0, 0] = threshold                                   # on the threshold is not above it
+    indices, values = label_list(rng, B, L, per_sample=min(4, L))
+    values = np.round(values * 4) / 4                          # exactly representable sums
+    predicted, correct, total = oracle.threshold_counts(scores, indices, values, threshold)
+    y = (torch.from_numpy(indices).cuda(), torch.from_numpy(values).cuda())
+    got = ffi.metrics.threshold_counts(torch.from_numpy(scores).cuda(), y, threshold).cpu().numpy()
+    assert tuple(got) == (predicted, correct, total)
+    prec, rec = ffi.SparsePrecision(threshold), ffi.SparseRecall(threshold)
+    for _ in range(2):
+        prec.update_state(y, torch.from_numpy(scores).cuda())
+        rec.update_state(y, torch.from_numpy(scores).cuda())
+    assert abs(prec.result() - (correct / predicted if predicted else 0.0)) < 1e-12
+    assert abs(rec.result() - correct / total) < 1e-12

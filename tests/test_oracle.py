@@ -338,3 +338,12 @@ def test_select_threshold_oracle_is_the_kth_smallest_magnitude():
         # strict comparison: the threshold value itself (and its ties) stays, so fewer than k are selected
         assert sel.sum() == (ordered < thr).sum() <= k - 1
     assert oracle.select_threshold(w, 0) == 0.0 and not oracle.rewire_selection(w, 0.0).any()
+
+
+def test_threshold_counts_oracle_on_a_hand_made_case():
+    # 2 x 4 scores, threshold 0: predicted = {(0,1), (0,3), (1,0)}; labels (0,1) value 1, (1,2) value 2, (1,0) value 0.5
+    scores = np.array([[-1.0, 0.5, 0.0, 2.0], [0.1, -0.2, -3.0, 0.0]], np.float32)
+    idx = np.array([[0, 1], [1, 2], [1, 0]])
+    predicted, correct, total = oracle.threshold_counts(scores, idx, np.array([1.0, 2.0, 0.5]), 0.0)
+    assert (predicted, correct, total) == (3.0, 1.5, 3.5)        # precision 1.5 / 3, recall 1.5 / 3.5
+    assert oracle.threshold_counts(scores, np.zeros((0, 2), int), None, 0.0) == (3.0, 0.0, 0.0)
