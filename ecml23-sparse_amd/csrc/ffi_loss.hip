@@ -22,7 +22,9 @@ constexpr int kLossVecPerThread = 4;    // float4 loads in flight per thread and
 __global__ __launch_bounds__(kLossThreads) void loss_dense_kernel(const float* scores, float* g, size_t total, float scale,
                                                                   int kind, double* __restrict__ partial) {
     // `scores` and `g` may be the same buffer: every element is read before it is written, by the same thread
-    const size_t nvec = total / 4;
+    // 16-byte accesses when both buffers allow them; whatever is left goes element by element
+    const bool vec = (((uintptr_t)scores | (uintptr_t)g) & 15) == 0;
+    const size_t nvec = vec ? total / 4 : 0;
     const size_t stride = (size_t)gridDim.x * kLossThreads;
     float lsum = 0.f;
     for (size_t v0 = (size_t)blockIdx.x * kLossThreads + threadIdx.x; v0 < nvec; v0 += stride * kLossVecPerThread) {
@@ -47,11 +49,11 @@ __global__ __launch_bounds__(kLossThreads) void loss_dense_kernel(const float* s
             }
         }
     }
-    if (blockIdx.x == 0 && threadIdx.x < (total & 3)) {       // the last 1..3 elements
-        const size_t e = nvec * 4 + threadIdx.x;
-        const float sv = scores[e];
-        lsum += cwise_loss(kind, sv, 0.f);
-        g[e] = scale * cwise_loss_grad(kind, sv, 0.f);
+    for (size_t e = nvec * 4 + (size_t)blockIdx.x * kLossThreads + threadIdx.x; e < total; e += stride) {
+        float l, d;
+        cwise_loss_and_grad(kind, scores[e], 0.f, l, d);
+        lsum += l;
+        g[e] = scale * d;
     }
     const double w = wave_sum((double)lsum);
     if ((threadIdx.x & 63) == 0) partial[blockIdx.x * (kLossThreads / 64) + (threadIdx.x >> 6)] = w;
@@ -134,7 +136,7 @@ __global__ __launch_bounds__(kFinishThreads) void loss_finish_kernel(const doubl
 // per wavefront: how many scores exceed the threshold
 __global__ __launch_bounds__(kLossThreads) void threshold_count_kernel(const float* __restrict__ scores, size_t total,
                                                                        float threshold, unsigned long long* __restrict__ partial) {
-    const size_t nvec = total / 4;
+    const size_t nvec = (((uintptr_t)scores) & 15) == 0 ? total / 4 : 0;
     const size_t stride = (size_t)gridDim.x * kLossThreads;
     unsigned c = 0;
     for (size_t v0 = (size_t)blockIdx.x * kLossThreads + threadIdx.x; v0 < nvec; v0 += stride * kLossVecPerThread) {
@@ -148,7 +150,7 @@ __global__ __launch_bounds__(kLossThreads) void threshold_count_kernel(const flo
         for (int i = 0; i < kLossVecPerThread; ++i)
             c += (s[i].x > threshold) + (s[i].y > threshold) + (s[i].z > threshold) + (s[i].w > threshold);
     }
-    if (blockIdx.x == 0 && threadIdx.x < (total & 3)) c += scores[nvec * 4 + threadIdx.x] > threshold;
+    for (size_t e = nvec * 4 + (size_t)blockIdx.x * kLossThreads + threadIdx.x; e < total; e += stride) c += scores[e] > threshold;
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) c += __shfl_xor(c, off, 64);
     if ((threadIdx.x & 63) == 0) partial[blockIdx.x * (kLossThreads / 64) + (threadIdx.x >> 6)] = c;
@@ -194,9 +196,8 @@ __global__ __launch_bounds__(kFinishThreads) void threshold_finish_kernel(const 
 int launch_threshold_metrics(const float* scores, const int64_t* indices, const float* values, int nnz, float threshold, int B,
                              int L, double* out, hipStream_t s) {
     const size_t total = (size_t)B * (size_t)L;
-    const size_t nvec = total / 4;
-    const size_t per_block = (size_t)kLossThreads * kLossVecPerThread;
-    const int blocks = (int)std::max<size_t>(1, std::min<size_t>((nvec + per_block - 1) / per_block, (size_t)device_cu_count() * 16));
+    const size_t per_block = (size_t)kLossThreads * kLossVecPerThread * 4;
+    const int blocks = (int)std::max<size_t>(1, std::min<size_t>((total + per_block - 1) / per_block, (size_t)device_cu_count() * 16));
     const int npartial = blocks * (kLossThreads / 64);
     unsigned char* ws = nullptr;
     FFI_TRY(workspace_get(s, kWsLoss, ((size_t)npartial + 2 * (size_t)nnz + 2) * sizeof(double), (void**)&ws));
@@ -240,9 +241,8 @@ int launch_loss_positives(const LossArgs& la, const float* saved, const float* s
 
 int launch_loss_grad(const LossArgs& la, const float* scores, float* g, int B, int L, hipStream_t s) {
     const size_t total = (size_t)B * (size_t)L;
-    const size_t nvec = total / 4;
-    const size_t per_block = (size_t)kLossThreads * kLossVecPerThread;
-    const int blocks = (int)std::max<size_t>(1, std::min<size_t>((nvec + per_block - 1) / per_block, (size_t)device_cu_count() * 16));
+    const size_t per_block = (size_t)kLossThreads * kLossVecPerThread * 4;
+    const int blocks = (int)std::max<size_t>(1, std::min<size_t>((total + per_block - 1) / per_block, (size_t)device_cu_count() * 16));
     const int npartial = blocks * (kLossThreads / 64);
     double *partial = nullptr, *corr = nullptr;
     float* saved = nullptr;

@@ -251,3 +251,25 @@ def test_threshold_metrics_against_oracle(ffi, shape, threshold):
         rec.update_state(y, torch.from_numpy(scores).cuda())
     assert abs(prec.result() - (correct / predicted if predicted else 0.0)) < 1e-12
     assert abs(rec.result() - correct / total) < 1e-12
+
+
+def test_unaligned_score_buffers(ffi):
+    # scores / out_grad that start 4 bytes into an allocation (a view): no 16-byte accesses may be assumed
+    B, L = 19, 1003
+    rng = np.random.default_rng(77)
+    scores = rng.normal(0, 1, (B, L)).astype(np.float32)
+    indices, values = label_list(rng, B, L)
+    y = (torch.from_numpy(indices).cuda(), torch.from_numpy(values).cuda())
+    base = torch.empty(B * L + 1, device="cuda")
+    view = base[1:].view(B, L)
+    view.copy_(torch.from_numpy(scores))
+    assert view.data_ptr() % 16 == 4
+    losses, grad = oracle.sparse_loss(scores, indices, values, oracle.LOSS_SQUARED_HINGE)
+    g, loss_sum = ffi.metrics.sparse_loss_grad(view, y, oracle.LOSS_SQUARED_HINGE, grad_scale=1.0)
+    torch.cuda.synchronize()
+    assert rel_err(g.cpu().numpy(), grad) <= RTOL and abs(float(loss_sum) - losses.sum()) <= RTOL * losses.sum()
+    got = ffi.metrics.threshold_counts(view, y, 0.0).cpu().numpy()
+    assert tuple(got) == oracle.threshold_counts(scores, indices, values, 0.0)
+    g2, _ = ffi.metrics.sparse_loss_grad(view, y, oracle.LOSS_SQUARED_HINGE, grad_scale=1.0, in_place=True)
+    torch.cuda.synchronize()
+    assert g2.data_ptr() == view.data_ptr() and rel_err(view.cpu().numpy(), grad) <= RTOL
