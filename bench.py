@@ -134,6 +134,13 @@ def train_step(pkg, cfg, x, lookup, w, tp, density, stream, iters):
         check(lib.ffi_forward_loss_f32(ptr(x), ptr(lookup), ptr(w), ptr(bias), ptr(labels), None, labels.shape[0], SQH | SKIP, scale,
                                        None, ptr(g), ptr(loss), ptr(masks), B, N, L, K, int(tp), sh))
 
+    tv, ti = torch.empty((B, 5), device="cuda"), torch.empty((B, 5), dtype=torch.int32, device="cuda")
+
+    def fused_forward_loss_topk():
+        # the same pass with the top-5 of the scores as a by-product (what P@1/3/5 need), still without the score matrix
+        check(lib.ffi_forward_loss_topk_f32(ptr(x), ptr(lookup), ptr(w), ptr(bias), ptr(labels), None, labels.shape[0], SQH | SKIP,
+                                            scale, None, ptr(g), ptr(loss), ptr(masks), ptr(tv), ptr(ti), 5, B, N, L, K, int(tp), sh))
+
     def backward_sparse():
         check(lib.ffi_backward_sparse_f32(ptr(x), ptr(lookup), ptr(w), ptr(g), ptr(masks), 1, ctypes.c_float(0.0), ptr(gx), ptr(gw),
                                           ptr(gb), ctypes.byref(taken), B, N, L, K, int(tp), sh))
@@ -164,6 +171,7 @@ def train_step(pkg, cfg, x, lookup, w, tp, density, stream, iters):
     out["forward_loss_ms"] = round(time_kernel(fused_forward_loss, stream, iters), 4)
     g.zero_()
     fused_forward_loss()
+    out["forward_loss_top5_ms"] = round(time_kernel(fused_forward_loss_topk, stream, iters), 4)
     out["gradient_density"] = round(float((g != 0).float().mean()), 6)
     out["backward_sparse_ms"] = round(time_kernel(backward_sparse, stream, iters), 4)
     out["sparse_kernels_ran"] = bool(taken.value)

@@ -26,6 +26,7 @@ from .fixed_fan_in_ops import (  # noqa: E402
     fan_in_sparse_matmul_tp_bias,
     arrange_connections,
     backward_sparse,
+    fan_in_sparse_topk,
 )
 from . import custom_layer, metrics, optimizer  # noqa: E402
 from .optimizer import SparseAdam  # noqa: E402
@@ -53,6 +54,7 @@ __all__ = [
     "fan_in_sparse_matmul_tp_bias",
     "arrange_connections",
     "backward_sparse",
+    "fan_in_sparse_topk",
     "StratifiedRewireLayerV2",
     "FixedFractionSelector",
     "FixedMagnitudeSelector",

@@ -37,6 +37,9 @@ SIGNATURES = {
     "ffi_forward_topk_bf16": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "ffi_topk_f32": (_int, [_vp, _i64, _i64, _int, _vp, _vp, _vp]),
     "ffi_loss_grad_f32": (_int, [_vp, _vp, _vp, _i64, _int, _f32, _vp, _vp, _vp, _i64, _i64, _vp]),
+    "ffi_forward_topk_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),
+    "ffi_forward_loss_topk_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _int, _f32, _vp, _vp, _vp, _vp, _vp, _vp, _int,
+                                         _i64, _i64, _i64, _i64, _int, _vp]),
     "ffi_threshold_metrics_f32": (_int, [_vp, _vp, _vp, _i64, _f32, _vp, _i64, _i64, _vp]),
     "ffi_forward_loss_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _int, _f32, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "ffi_backward_sparse_adam_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _f32, _vp, _vp, _vp, _vp, _vp, _vp, _f32, _f32, _f32, _f32,

@@ -256,6 +256,36 @@ int ffi_loss_grad_f32(const float* scores, const int64_t* label_indices, const f
     return launch_loss_grad(la, scores, out_grad, (int)batch, (int)num_units, (hipStream_t)stream);
 }
 
+int ffi_forward_topk_f32(const float* features, const int32_t* lookup, const float* weights, const float* bias, float* scores,
+                         float* topk_values, int32_t* topk_indices, int64_t batch, int64_t num_features, int64_t num_units,
+                         int64_t fan_in, int k, int transposed, ffi_stream_t stream) {
+    if (!features || !lookup || !weights || !topk_values || !topk_indices) return FFI_ERR_NULL_POINTER;
+    if (k < 1 || k > 8) return FFI_ERR_BAD_ARGUMENT;
+    Dims d;
+    FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
+    const TopkArgs tk{k, topk_values, topk_indices};
+    return launch_forward_topk(features, lookup, weights, bias, scores, tk, d, (hipStream_t)stream);
+}
+
+int ffi_forward_loss_topk_f32(const float* features, const int32_t* lookup, const float* weights, const float* bias,
+                              const int64_t* label_indices, const float* label_values, int64_t nnz, int loss_kind,
+                              float grad_scale, float* scores, float* out_grad, float* loss_sum, uint32_t* nz_words,
+                              float* topk_values, int32_t* topk_indices, int k, int64_t batch, int64_t num_features,
+                              int64_t num_units, int64_t fan_in, int transposed, ffi_stream_t stream) {
+    if (!features || !lookup || !weights || !out_grad || !topk_values || !topk_indices) return FFI_ERR_NULL_POINTER;
+    if (scores == out_grad) return FFI_ERR_BAD_ARGUMENT;
+    if (k < 1 || k > 8) return FFI_ERR_BAD_ARGUMENT;
+    Dims d;
+    FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
+    const bool skip = (loss_kind & FFI_LOSS_SKIP_ZERO_STORES) != 0;
+    loss_kind &= ~FFI_LOSS_SKIP_ZERO_STORES;
+    if (skip && !nz_words) return FFI_ERR_NULL_POINTER;
+    FFI_TRY(check_loss_args(label_indices, nnz, loss_kind, batch, num_units));
+    const LossArgs la{label_indices, label_values, (int)nnz, loss_kind, grad_scale, loss_sum, nz_words, skip};
+    const TopkArgs tk{k, topk_values, topk_indices};
+    return launch_forward_loss(features, lookup, weights, bias, la, scores, out_grad, &tk, d, (hipStream_t)stream);
+}
+
 int ffi_threshold_metrics_f32(const float* scores, const int64_t* label_indices, const float* label_values, int64_t nnz,
                               float threshold, double* counts, int64_t batch, int64_t num_units, ffi_stream_t stream) {
     if (!scores || !counts) return FFI_ERR_NULL_POINTER;
@@ -278,7 +308,7 @@ int ffi_forward_loss_f32(const float* features, const int32_t* lookup, const flo
     if (skip && !nz_words) return FFI_ERR_NULL_POINTER;
     FFI_TRY(check_loss_args(label_indices, nnz, loss_kind, batch, num_units));
     const LossArgs la{label_indices, label_values, (int)nnz, loss_kind, grad_scale, loss_sum, nz_words, skip};
-    return launch_forward_loss(features, lookup, weights, bias, la, scores, out_grad, d, (hipStream_t)stream);
+    return launch_forward_loss(features, lookup, weights, bias, la, scores, out_grad, nullptr, d, (hipStream_t)stream);
 }
 
 int ffi_backward_sparse_f32(const float* features, const int32_t* lookup, const float* weights, float* out_grad,

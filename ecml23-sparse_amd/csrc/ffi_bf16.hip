@@ -184,46 +184,85 @@ __device__ __forceinline__ void topk_insert_ordered(float (&vals)[kTopMax], int 
 }
 
 // One wavefront per sample merges its `nlists` lists of 8 (empty slots have label -1): every lane
-// reduces a strided share of the candidates, lane 0 merges the 64 lane lists.
+// reduces a strided share of the candidates to a sorted list of its own; then k rounds in which the
+// best head among the 64 lane lists (found with shuffles) is emitted and popped.
 __global__ __launch_bounds__(64) void topk_merge_kernel(const float* __restrict__ part_val, const int* __restrict__ part_idx,
                                                         int B, int nlists, int k, float* __restrict__ values,
                                                         int* __restrict__ indices) {
-    __shared__ float lv[64 * kTopMax];
-    __shared__ int li[64 * kTopMax];
     const int b = blockIdx.x;
+    const int lane = threadIdx.x;
     float vals[kTopMax];
     int ids[kTopMax];
 #pragma unroll
     for (int s = 0; s < kTopMax; ++s) { vals[s] = -__builtin_inff(); ids[s] = 0x7fffffff; }
     const float* pv = part_val + (size_t)b * nlists * kTopMax;
     const int* pi = part_idx + (size_t)b * nlists * kTopMax;
-    for (int c = threadIdx.x; c < nlists * kTopMax; c += 64) {
-        const float v = pv[c];
-        const int id = pi[c];
-        if (id >= 0 && better(v, id, vals[kTopMax - 1], ids[kTopMax - 1])) topk_insert_ordered(vals, ids, v, id);
-    }
+    const int total = nlists * kTopMax;
+    for (int c0 = lane; c0 < total; c0 += 64 * 8) {           // eight candidates per lane in flight
+        float v8[8];
+        int i8[8];
 #pragma unroll
-    for (int s = 0; s < kTopMax; ++s) { lv[threadIdx.x * kTopMax + s] = vals[s]; li[threadIdx.x * kTopMax + s] = ids[s]; }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        for (int c = kTopMax; c < 64 * kTopMax; ++c) {
-            const float v = lv[c];
-            const int id = li[c];
-            if (id != 0x7fffffff && better(v, id, vals[kTopMax - 1], ids[kTopMax - 1])) topk_insert_ordered(vals, ids, v, id);
+        for (int u = 0; u < 8; ++u) {
+            const int c = min(c0 + 64 * u, total - 1);    // clamped, not predicated: the loads issue back to back
+            i8[u] = c0 + 64 * u < total ? pi[c] : -1;
+            v8[u] = pv[c];
         }
 #pragma unroll
-        for (int s = 0; s < kTopMax; ++s) {
-            if (s < k) {
-                const bool filled = ids[s] != 0x7fffffff;
-                values[(size_t)b * k + s] = vals[s];
-                indices[(size_t)b * k + s] = filled ? ids[s] : -1;
-            }
+        for (int u = 0; u < 8; ++u)
+            if (i8[u] >= 0 && better(v8[u], i8[u], vals[kTopMax - 1], ids[kTopMax - 1])) topk_insert_ordered(vals, ids, v8[u], i8[u]);
+    }
+    for (int s = 0; s < k; ++s) {
+        // the best head of all lanes (empty lists carry (-inf, 0x7fffffff) and lose every comparison)
+        float bv = vals[0];
+        int bi = ids[0];
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const float ov = __shfl_xor(bv, off, 64);
+            const int oi = __shfl_xor(bi, off, 64);
+            if (better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
+        }
+        if (lane == 0) {
+            values[(size_t)b * k + s] = bv;
+            indices[(size_t)b * k + s] = bi != 0x7fffffff ? bi : -1;
+        }
+        // the lane that owned it moves its list up (labels are unique, so exactly one lane matches a real winner)
+        if (bi != 0x7fffffff && ids[0] == bi && vals[0] == bv) {
+#pragma unroll
+            for (int t = 0; t + 1 < kTopMax; ++t) { vals[t] = vals[t + 1]; ids[t] = ids[t + 1]; }
+            vals[kTopMax - 1] = -__builtin_inff();
+            ids[kTopMax - 1] = 0x7fffffff;
         }
     }
 }
 
-// top-8 lists of a score matrix scores[B,L]: grid (splits, B); each thread scans a strided share of
-// the split (coalesced), then the workgroup's lists go out as they are (256 lists per split).
+// Wave-level selection: the 64 lanes hold sorted lists of 8; kTopMax rounds in which the best head (found with
+// shuffles) is taken by lane `round` and popped by its owner.  Afterwards lane s < 8 holds the s-th best in out_*.
+__device__ __forceinline__ void wave_topk(float (&vals)[kTopMax], int (&ids)[kTopMax], float& out_v, int& out_i) {
+    const int lane = threadIdx.x & 63;
+    out_v = -__builtin_inff();
+    out_i = 0x7fffffff;
+#pragma unroll
+    for (int s = 0; s < kTopMax; ++s) {
+        float bv = vals[0];
+        int bi = ids[0];
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const float ov = __shfl_xor(bv, off, 64);
+            const int oi = __shfl_xor(bi, off, 64);
+            if (better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
+        }
+        if (lane == s) { out_v = bv; out_i = bi; }
+        if (bi != 0x7fffffff && ids[0] == bi && vals[0] == bv) {
+#pragma unroll
+            for (int t = 0; t + 1 < kTopMax; ++t) { vals[t] = vals[t + 1]; ids[t] = ids[t + 1]; }
+            vals[kTopMax - 1] = -__builtin_inff();
+            ids[kTopMax - 1] = 0x7fffffff;
+        }
+    }
+}
+
+// top-8 lists of a score matrix scores[B,L]: grid (splits, B); each thread scans a strided share of the split
+// (coalesced, eight scores in flight), each wavefront then reduces its 64 lists to one: 4 lists per split.
 __global__ __launch_bounds__(256) void topk_scan_kernel(const float* __restrict__ scores, int L, int labels_per_split,
                                                         float* __restrict__ part_val, int* __restrict__ part_idx, int nlists) {
     const int b = blockIdx.y;
@@ -231,17 +270,32 @@ __global__ __launch_bounds__(256) void topk_scan_kernel(const float* __restrict_
     float vals[kTopMax];
     int ids[kTopMax];
 #pragma unroll
-    for (int s = 0; s < kTopMax; ++s) { vals[s] = -__builtin_inff(); ids[s] = -1; }
+    for (int s = 0; s < kTopMax; ++s) { vals[s] = -__builtin_inff(); ids[s] = 0x7fffffff; }
     const float* row = scores + (size_t)b * L;
-    for (int j = begin + (int)threadIdx.x; j < end; j += 256) {
-        const float v = row[j];
-        if (v > vals[kTopMax - 1]) topk_insert(vals, ids, v, j);
-    }
-    const int list = blockIdx.x * 256 + threadIdx.x;
-    float* pv = part_val + ((size_t)b * nlists + list) * kTopMax;
-    int* pi = part_idx + ((size_t)b * nlists + list) * kTopMax;
+    for (int j0 = begin + (int)threadIdx.x; j0 < end; j0 += 256 * 8) {      // eight scores per thread in flight
+        float v8[8];
 #pragma unroll
-    for (int s = 0; s < kTopMax; ++s) { pv[s] = vals[s]; pi[s] = ids[s]; }
+        for (int u = 0; u < 8; ++u) {
+            const int j = j0 + 256 * u;
+            v8[u] = row[min(j, end - 1)];                 // clamped, not predicated: the eight loads issue back to back
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int j = j0 + 256 * u;
+            // (ascending labels per thread, so `>` keeps the lower label among equal scores; -inf scores still enter
+            // an empty slot through the label comparison)
+            if (j < end && better(v8[u], j, vals[kTopMax - 1], ids[kTopMax - 1])) topk_insert_ordered(vals, ids, v8[u], j);
+        }
+    }
+    float ov;
+    int oi;
+    wave_topk(vals, ids, ov, oi);
+    const int lane = threadIdx.x & 63;
+    if (lane < kTopMax) {
+        const int list = blockIdx.x * 4 + (threadIdx.x >> 6);
+        part_val[((size_t)b * nlists + list) * kTopMax + lane] = ov;
+        part_idx[((size_t)b * nlists + list) * kTopMax + lane] = oi != 0x7fffffff ? oi : -1;
+    }
 }
 
 int prepare_bf16_features(const unsigned short* features, int B, int N, bool tp, hipStream_t s, const unsigned short** xT,
@@ -302,13 +356,101 @@ int launch_forward_topk_bf16(const unsigned short* features, const int32_t* idx,
     return FFI_OK;
 }
 
-int launch_topk_f32(const float* scores, int B, int L, int k, float* values, int32_t* indices, hipStream_t s) {
+int launch_topk_merge(const float* part_val, const int* part_idx, int B, int nlists, int k, float* values, int32_t* indices,
+                      hipStream_t s) {
     if (k < 1 || k > kTopMax) return FFI_ERR_BAD_ARGUMENT;
-    if (B > 65535) return FFI_ERR_TOO_LARGE;
-    int splits = std::max(1, std::min((L + 4095) / 4096, 2 * device_cu_count() / std::max(1, B) + 1));
+    hipLaunchKernelGGL(topk_merge_kernel, dim3(B), dim3(64), 0, s, part_val, part_idx, B, nlists, k, values, indices);
+    FFI_HIP_TRY(hipGetLastError());
+    return FFI_OK;
+}
+
+namespace {
+
+__global__ __launch_bounds__(256) void topk_init_kernel(int* __restrict__ count, int B, int* __restrict__ cand_idx, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < (size_t)B) count[i] = 0;
+    for (size_t e = i; e < n; e += (size_t)gridDim.x * 256) cand_idx[e] = -1;
+}
+
+// a sample whose candidates did not fit its list gets no answer: labels -2, scores NaN
+__global__ __launch_bounds__(256) void topk_overflow_kernel(const int* __restrict__ count, int cap, int B, int k,
+                                                            float* __restrict__ values, int* __restrict__ indices) {
+    const int b = blockIdx.x * 256 + threadIdx.x;
+    if (b >= B || count[b] <= cap) return;
+    for (int s = 0; s < k; ++s) { values[(size_t)b * k + s] = __builtin_nanf(""); indices[(size_t)b * k + s] = -2; }
+}
+
+// sample[b][i] = scores[b][(i * L) / S]: evenly spaced labels whose k-th best score is a threshold that at least k
+// labels of the row reach
+__global__ __launch_bounds__(256) void topk_sample_kernel(const float* __restrict__ scores, int L, int S, float* __restrict__ sample) {
+    const int b = blockIdx.y;
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < S) sample[(size_t)b * S + i] = scores[(size_t)b * L + (int)(((long long)i * L) / S)];
+}
+
+// Every score at or above its row's threshold goes to the row's candidate list.  Such scores are a tiny share of the
+// row, so the scan is a plain stream: eight loads in flight per thread, one wave-wide test, the appends on the side.
+__global__ __launch_bounds__(256) void topk_filter_kernel(const float* __restrict__ scores, int L, int labels_per_split,
+                                                          const float* __restrict__ tau, int tau_stride, int* __restrict__ count,
+                                                          float* __restrict__ cand_val, int* __restrict__ cand_idx, int cap) {
+    constexpr int kPark = 1024;                       // hits a workgroup parks in LDS before it appends them to the row's list
+    __shared__ int park_count;
+    __shared__ float park_val[kPark];
+    __shared__ int park_idx[kPark];
+    const int b = blockIdx.y;
+    const int begin = blockIdx.x * labels_per_split, end = min(begin + labels_per_split, L);
+    const float t = tau[(size_t)b * tau_stride];
+    const float* row = scores + (size_t)b * L;
+    if (threadIdx.x == 0) park_count = 0;
+    __syncthreads();
+    for (int j0 = begin + (int)threadIdx.x; j0 < end; j0 += 256 * 8) {
+        float v8[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v8[u] = row[min(j0 + 256 * u, end - 1)];
+        bool hit = false;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) hit |= (j0 + 256 * u < end) && v8[u] >= t;
+        if (__ballot(hit)) {
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int j = j0 + 256 * u;
+                if (j < end && v8[u] >= t) {
+                    const int p = atomicAdd(&park_count, 1);          // an LDS counter: no round trip to memory
+                    if (p < kPark) {
+                        park_val[p] = v8[u];
+                        park_idx[p] = j;
+                    } else {
+                        const int slot = atomicAdd(&count[b], 1);
+                        if (slot < cap) {
+                            cand_val[(size_t)b * cap + slot] = v8[u];
+                            cand_idx[(size_t)b * cap + slot] = j;
+                        }
+                    }
+                }
+            }
+        }
+    }
+    __syncthreads();
+    const int n = min(park_count, kPark);
+    __shared__ int first_slot;
+    if (threadIdx.x == 0) first_slot = n ? atomicAdd(&count[b], n) : 0;      // one reservation for the whole workgroup
+    __syncthreads();
+    for (int e = threadIdx.x; e < n; e += 256) {
+        const int slot = first_slot + e;
+        if (slot < cap) {
+            cand_val[(size_t)b * cap + slot] = park_val[e];
+            cand_idx[(size_t)b * cap + slot] = park_idx[e];
+        }
+    }
+}
+
+// the old way, for rows too short to be worth a threshold: every thread keeps a list, the wavefronts reduce them
+int topk_by_lists(const float* scores, int B, int L, int k, float* values, int32_t* indices, hipStream_t s) {
+    // enough workgroups to fill the GPU (8 per CU), each with at least 2048 scores to scan
+    int splits = std::max(1, std::min((L + 2047) / 2048, (8 * device_cu_count() + B - 1) / std::max(1, B)));
     const int per = (L + splits - 1) / splits;
     splits = (L + per - 1) / per;
-    const int nlists = splits * 256;
+    const int nlists = splits * 4;
     char* part = nullptr;
     const size_t list_bytes = (size_t)B * nlists * kTopMax * 4;
     FFI_TRY(workspace_get(s, kWsPartials, 2 * list_bytes, (void**)&part));
@@ -318,6 +460,54 @@ int launch_topk_f32(const float* scores, int B, int L, int k, float* values, int
     hipLaunchKernelGGL(topk_merge_kernel, dim3(B), dim3(64), 0, s, pv, pi, B, nlists, k, values, indices);
     FFI_HIP_TRY(hipGetLastError());
     return FFI_OK;
+}
+
+constexpr int kTopkRowSample = 4096;
+
+}  // namespace
+
+int launch_topk_candidates_init(int* count, int* cand_idx, int B, int cap, hipStream_t s) {
+    hipLaunchKernelGGL(topk_init_kernel, dim3(1024), dim3(256), 0, s, count, B, cand_idx, (size_t)B * cap);
+    FFI_HIP_TRY(hipGetLastError());
+    return FFI_OK;
+}
+
+int launch_topk_candidates_select(const float* cand_val, const int* cand_idx, const int* count, int B, int cap, int k,
+                                  float* values, int32_t* indices, hipStream_t s) {
+    FFI_TRY(launch_topk_merge(cand_val, cand_idx, B, cap / 8, k, values, indices, s));
+    hipLaunchKernelGGL(topk_overflow_kernel, dim3((B + 255) / 256), dim3(256), 0, s, count, cap, B, k, values, indices);
+    FFI_HIP_TRY(hipGetLastError());
+    return FFI_OK;
+}
+
+int launch_topk_f32(const float* scores, int B, int L, int k, float* values, int32_t* indices, hipStream_t s) {
+    if (k < 1 || k > kTopMax) return FFI_ERR_BAD_ARGUMENT;
+    if (B > 65535) return FFI_ERR_TOO_LARGE;
+    if (L <= 16 * kTopkRowSample) return topk_by_lists(scores, B, L, k, values, indices, s);
+    // Long rows: a sample of every row fixes a threshold that k of its labels reach (the k-th best of the sample), one
+    // streaming pass collects the few scores at or above it, and the k best of those are the answer.  Exact; a row
+    // with more than kTopkCap scores at or above its threshold (thousands of ties) gets labels -2 instead.
+    const int S = kTopkRowSample;
+    const size_t cand = (size_t)B * kTopkCap;
+    unsigned char* ws = nullptr;
+    FFI_TRY(workspace_get(s, kWsTopk, ((size_t)B * S + 2 * (size_t)B * kTopMax + (size_t)B + 2 * cand) * 4, (void**)&ws));
+    float* sample = reinterpret_cast<float*>(ws);
+    float* tau_val = sample + (size_t)B * S;
+    int* tau_idx = reinterpret_cast<int*>(tau_val + (size_t)B * kTopMax);
+    int* count = tau_idx + (size_t)B * kTopMax;
+    float* cand_val = reinterpret_cast<float*>(count + B);
+    int* cand_idx = reinterpret_cast<int*>(cand_val + cand);
+    hipLaunchKernelGGL(topk_sample_kernel, dim3((S + 255) / 256, B), dim3(256), 0, s, scores, L, S, sample);
+    FFI_HIP_TRY(hipGetLastError());
+    FFI_TRY(topk_by_lists(sample, B, S, k, tau_val, tau_idx, s));
+    FFI_TRY(launch_topk_candidates_init(count, cand_idx, B, kTopkCap, s));
+    int splits = std::max(1, std::min((L + 2047) / 2048, (8 * device_cu_count() + B - 1) / std::max(1, B)));
+    const int per = (L + splits - 1) / splits;
+    splits = (L + per - 1) / per;
+    hipLaunchKernelGGL(topk_filter_kernel, dim3(splits, B), dim3(256), 0, s, scores, L, per, tau_val + (k - 1), k, count, cand_val,
+                       cand_idx, kTopkCap);
+    FFI_HIP_TRY(hipGetLastError());
+    return launch_topk_candidates_select(cand_val, cand_idx, count, B, kTopkCap, k, values, indices, s);
 }
 
 }  // namespace ffi

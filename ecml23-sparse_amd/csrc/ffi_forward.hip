@@ -38,7 +38,23 @@ __device__ __forceinline__ void fwd_lane_step(const char* __restrict__ xs_bytes,
 //   kEpiLossGrad     out = scale * dloss(s, 0)/ds, the loss gradient of a position that is not a listed label
 //                    (listed positions are patched afterwards), and the loss(s, 0) summed per wavefront
 //   kEpiLossGradAndScores  both: scores to `out`, gradients to `gout`
-enum FwdEpilogue { kEpiScores = 0, kEpiLossGrad = 1, kEpiLossGradAndScores = 2 };
+//   kEpiNone         nothing is stored (only the top-k candidates below are wanted)
+enum FwdEpilogue { kEpiScores = 0, kEpiLossGrad = 1, kEpiLossGradAndScores = 2, kEpiNone = 3 };
+
+constexpr int kTopkPark = 24;           // candidates per (workgroup, batch row) parked in LDS: 32 x 24 x 8 bytes = 6 KB
+
+// Per-sample top-k without the score matrix (TOPK): tau[b] is a score that at least k labels of sample b are
+// known to reach (the k-th best of a sample of the labels, found beforehand), so the k best scores are among
+// those >= tau[b]; every such (label, score) is appended to the sample's candidate list, a few hundred to a
+// few thousand entries out of all labels, and a small kernel selects the k best afterwards.
+struct FwdTopk {
+    const float* tau;     // tau[b * tau_stride]
+    int tau_stride;
+    int* count;           // [B] candidates appended so far (may run past cap: the list is then incomplete)
+    float* cand_val;      // [B][cap]
+    int* cand_idx;        // [B][cap]
+    int cap;
+};
 
 struct FwdLoss {
     float* gout;        // [B,L] gradients (kEpiLossGradAndScores), else unused
@@ -78,20 +94,27 @@ __device__ __forceinline__ void loss_epilogue(float (&acc)[32], int nrows, float
     mask = m;
 }
 
-template <bool VEC4, int EPI>
+template <bool VEC4, int EPI, bool TOPK>
 __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* __restrict__ xT,
                                                                   const int32_t* __restrict__ idx,
                                                                   const float* __restrict__ w,
                                                                   const float* __restrict__ bias,
                                                                   float* __restrict__ out, int B, int N,
                                                                   int L, int K, int nbt, int labels_per_stream,
-                                                                  FwdLoss fl) {
+                                                                  FwdLoss fl, FwdTopk ft) {
     extern __shared__ __align__(16) float xs[];
+    __shared__ __align__(16) float tau_s[kTileBatch];
+    __shared__ int local_count[kTileBatch];      // candidates parked per batch row (may run past kTopkPark)
+    __shared__ int local_base[kTileBatch];
+    int2* local_cand = reinterpret_cast<int2*>(xs + (size_t)N * kTileBatch);      // behind the tile (TOPK launches only)
     const char* xs_bytes = reinterpret_cast<const char*>(xs);
     const int u = xcd_contiguous_block(blockIdx.x, gridDim.x);
     const int bt = u % nbt, stream = u / nbt;
     const int b0 = bt * kTileBatch;
     stage_rows32<kTileThreads>(xs, xT, N, B, b0);
+    if (TOPK && threadIdx.x < kTileBatch) local_count[threadIdx.x] = 0;
+    if (TOPK && threadIdx.x < kTileBatch)          // rows past the batch never qualify
+        tau_s[threadIdx.x] = b0 + (int)threadIdx.x < B ? ft.tau[(size_t)(b0 + threadIdx.x) * ft.tau_stride] : __builtin_inff();
     __syncthreads();
     const int lane = threadIdx.x & 63;
     const unsigned skew = (unsigned)(lane & 7) * 16u;
@@ -159,14 +182,54 @@ __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* _
 #pragma unroll
             for (int i = 0; i < 32; ++i) acc[i] += bj;
         }
+        if (TOPK) {
+            // Scores that reach their sample's threshold are rare (about one in a thousand), but a wavefront holds 2048 of
+            // them: the tests are wave-uniform and hierarchical (four groups of eight batch rows, then the rows of a group
+            // that has a hit), so that a row without a hit costs one compare.
+            float tv[32];
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                const float4 t4 = *reinterpret_cast<const float4*>(tau_s + 4 * c);
+                tv[4 * c] = t4.x; tv[4 * c + 1] = t4.y; tv[4 * c + 2] = t4.z; tv[4 * c + 3] = t4.w;
+            }
+#pragma unroll
+            for (int grp = 0; grp < 4; ++grp) {
+                bool hit = false;
+#pragma unroll
+                for (int b = 8 * grp; b < 8 * grp + 8; ++b) hit |= acc[b] >= tv[b];
+                hit &= valid;
+                if (__ballot(hit)) {
+#pragma unroll
+                    for (int b = 8 * grp; b < 8 * grp + 8; ++b) {
+                        const bool h = valid && acc[b] >= tv[b];
+                        if (__ballot(h)) {
+                            if (h) {
+                                // parked in the workgroup's LDS segment of the sample (an LDS counter answers in a few dozen
+                                // clocks, a global one in microseconds); a full segment sends the entry to memory directly
+                                const int lslot = atomicAdd(&local_count[b], 1);
+                                if (lslot < kTopkPark) {
+                                    local_cand[b * kTopkPark + lslot] = make_int2(j, __float_as_int(acc[b]));
+                                } else {
+                                    const int slot = atomicAdd(&ft.count[b0 + b], 1);
+                                    if (slot < ft.cap) {
+                                        ft.cand_val[(size_t)(b0 + b) * ft.cap + slot] = acc[b];
+                                        ft.cand_idx[(size_t)(b0 + b) * ft.cap + slot] = j;
+                                    }
+                                }
+                            }
+                        }
+                    }
+                }
+            }
+        }
         const unsigned lane_off = (unsigned)j * 4u;
         const unsigned stride = (unsigned)L * 4u;
-        if (EPI != kEpiLossGrad && valid) {
+        if ((EPI == kEpiScores || EPI == kEpiLossGradAndScores) && valid) {
 #pragma unroll
             for (int b = 0; b < 32; ++b)
                 __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, acc[b]), orsrc, lane_off, (unsigned)b * stride, 0);
         }
-        if (EPI != kEpiScores) {
+        if (EPI == kEpiLossGrad || EPI == kEpiLossGradAndScores) {
             float l = 0.f;
             unsigned m = 0;
             // the loss kind is the same for the whole launch: one straight-line epilogue per kind
@@ -189,7 +252,27 @@ __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* _
             }
         }
     }
-    if (EPI != kEpiScores) {
+    if (TOPK) {
+        // the parked candidates go to their samples' lists: one reservation per (workgroup, sample)
+        __syncthreads();
+        if (threadIdx.x < kTileBatch) {
+            const int n = min(local_count[threadIdx.x], kTopkPark);
+            local_base[threadIdx.x] = n ? atomicAdd(&ft.count[b0 + threadIdx.x], n) : 0;
+        }
+        __syncthreads();
+        for (int e = threadIdx.x; e < kTileBatch * kTopkPark; e += kTileThreads) {
+            const int b = e / kTopkPark, i = e % kTopkPark;
+            if (i < min(local_count[b], kTopkPark)) {
+                const int2 c = local_cand[e];
+                const int slot = local_base[b] + i;
+                if (slot < ft.cap) {
+                    ft.cand_val[(size_t)(b0 + b) * ft.cap + slot] = __int_as_float(c.y);
+                    ft.cand_idx[(size_t)(b0 + b) * ft.cap + slot] = c.x;
+                }
+            }
+        }
+    }
+    if (EPI == kEpiLossGrad || EPI == kEpiLossGradAndScores) {
         const double t = wave_sum((double)lsum);
         if (lane == 0) fl.partial[(size_t)blockIdx.x * (kTileThreads / 64) + (threadIdx.x >> 6)] = t;
     }
@@ -199,19 +282,58 @@ __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* _
 
 namespace {
 
-template <bool VEC4, int EPI>
+constexpr int kTopkSample = 4096;      // labels whose scores set the per-sample thresholds
+
+// scores of every (L / S)-th label for all samples: sample_scores[b][i] (the thresholds' raw material)
+__global__ __launch_bounds__(256) void fwd_sample_kernel(const float* __restrict__ xT, const int32_t* __restrict__ idx,
+                                                         const float* __restrict__ w, const float* __restrict__ bias, int B, int N,
+                                                         int L, int K, int S, float* __restrict__ sample_scores) {
+    const int i = blockIdx.x;
+    const int j = (int)(((long long)i * L) / S);
+    const int32_t* irow = idx + (size_t)j * K;
+    const float* wrow = w + (size_t)j * K;
+    for (int b = threadIdx.x; b < B; b += 256) {
+        float acc = 0.f, mag = 0.f;
+        for (int k = 0; k < K; ++k) {
+            const unsigned id = (unsigned)irow[k];
+            const float xv = xT[(size_t)(id < (unsigned)N ? id : 0u) * B + b];
+            acc = fmaf(wrow[k], xv, acc);
+            mag = fmaf(fabsf(wrow[k]), fabsf(xv), mag);
+        }
+        if (bias != nullptr) { acc += bias[j]; mag += fabsf(bias[j]); }
+        // The main kernel sums the same products in another order; its score of this label differs from `acc` by at
+        // most a few rounding errors of the largest partial sum (K * 2^-24 * mag).  The threshold must not exceed the
+        // main kernel's value, so the sampled score is lowered by a bound on that difference.
+        sample_scores[(size_t)b * S + i] = acc - (float)(K + 2) * 1.2e-7f * mag;
+    }
+}
+
+template <bool VEC4, int EPI, bool TOPK>
 int launch_lane32(const float* xT, const int32_t* idx, const float* w, const float* bias, float* out, const Dims& d, int nbt,
-                  int per_stream, int blocks, size_t lds, const FwdLoss& fl, hipStream_t s) {
-    FFI_HIP_TRY(hipFuncSetAttribute((const void*)fwd_lane32_kernel<VEC4, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL((fwd_lane32_kernel<VEC4, EPI>), dim3(blocks), dim3(kTileThreads), lds, s, xT, idx, w, bias, out, d.B, d.N,
-                       d.L, d.K, nbt, per_stream, fl);
+                  int per_stream, int blocks, size_t lds, const FwdLoss& fl, const FwdTopk& ft, hipStream_t s) {
+    FFI_HIP_TRY(hipFuncSetAttribute((const void*)fwd_lane32_kernel<VEC4, EPI, TOPK>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL((fwd_lane32_kernel<VEC4, EPI, TOPK>), dim3(blocks), dim3(kTileThreads), lds, s, xT, idx, w, bias, out, d.B, d.N,
+                       d.L, d.K, nbt, per_stream, fl, ft);
     FFI_HIP_TRY(hipGetLastError());
     return FFI_OK;
 }
 
-// Narrow-input forward pass with the given epilogue; `la` is needed for the loss epilogues only.
+template <int EPI>
+int launch_lane32_any(bool vec4, bool topk, const float* xT, const int32_t* idx, const float* w, const float* bias, float* out,
+                      const Dims& d, int nbt, int per_stream, int blocks, size_t lds, const FwdLoss& fl, const FwdTopk& ft,
+                      hipStream_t s) {
+    if (topk)
+        return vec4 ? launch_lane32<true, EPI, true>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, ft, s)
+                    : launch_lane32<false, EPI, true>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, ft, s);
+    if (EPI == kEpiNone) return FFI_OK;                     // nothing to compute
+    return vec4 ? launch_lane32<true, EPI == kEpiNone ? kEpiScores : EPI, false>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, ft, s)
+                : launch_lane32<false, EPI == kEpiNone ? kEpiScores : EPI, false>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, ft, s);
+}
+
+// Narrow-input forward pass with the given epilogue; `la` is needed for the loss epilogues only, `tk` (may be
+// null) asks for the per-sample top-k without the score matrix.
 int forward_tiles(const float* x, const int32_t* idx, const float* w, const float* bias, float* out, float* gout, int epi,
-                  const LossArgs* la, const Dims& d, hipStream_t s) {
+                  const LossArgs* la, const TopkArgs* tk, const Dims& d, hipStream_t s) {
     const float* xT = x;
     if (!d.tp) {
         float* ws = nullptr;
@@ -228,23 +350,49 @@ int forward_tiles(const float* x, const int32_t* idx, const float* w, const floa
     streams = (d.L + per_stream - 1) / per_stream;
     const int blocks = streams * nbt;
     FwdLoss fl{gout, nullptr, nullptr, 0.f, 0, 0};
-    if (epi == kEpiScores)
-        return vec4 ? launch_lane32<true, kEpiScores>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, s)
-                    : launch_lane32<false, kEpiScores>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, s);
-    const int npartial = blocks * (kTileThreads / 64);
-    double* corr = nullptr;
-    FFI_TRY(loss_partial_buffer(s, npartial, la->nnz, &fl.partial, &corr, nullptr));
-    fl.scale = la->scale;
-    fl.kind = la->kind;
-    fl.words = la->nz_words;
-    fl.skip_zero_stores = la->skip_zero_stores ? 1 : 0;
-    if (epi == kEpiLossGrad) {
-        FFI_TRY(vec4 ? (launch_lane32<true, kEpiLossGrad>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, s))
-                     : (launch_lane32<false, kEpiLossGrad>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, s)));
-    } else {
-        FFI_TRY(vec4 ? (launch_lane32<true, kEpiLossGradAndScores>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, s))
-                     : (launch_lane32<false, kEpiLossGradAndScores>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, s)));
+    FwdTopk ft{};
+    const bool topk = tk != nullptr;
+    int* count = nullptr;
+    size_t lds_topk = lds;
+    if (topk) {
+        // thresholds: the k-th best score of every sample among kTopkSample evenly spaced labels
+        const int S = std::min(kTopkSample, d.L);
+        const size_t cand = (size_t)d.B * kTopkCap;
+        unsigned char* ws = nullptr;
+        const size_t bytes = ((size_t)d.B * S + 2 * (size_t)d.B * 8 + (size_t)d.B + 2 * cand) * 4;
+        FFI_TRY(workspace_get(s, kWsTopk, bytes, (void**)&ws));
+        float* sample_scores = reinterpret_cast<float*>(ws);
+        float* tau_val = sample_scores + (size_t)d.B * S;
+        int* tau_idx = reinterpret_cast<int*>(tau_val + (size_t)d.B * 8);
+        count = tau_idx + (size_t)d.B * 8;
+        float* cand_val = reinterpret_cast<float*>(count + d.B);
+        int* cand_idx = reinterpret_cast<int*>(cand_val + cand);
+        hipLaunchKernelGGL(fwd_sample_kernel, dim3(S), dim3(256), 0, s, xT, idx, w, bias, d.B, d.N, d.L, d.K, S, sample_scores);
+        FFI_HIP_TRY(hipGetLastError());
+        FFI_TRY(launch_topk_f32(sample_scores, d.B, S, tk->k, tau_val, tau_idx, s));
+        FFI_TRY(launch_topk_candidates_init(count, cand_idx, d.B, kTopkCap, s));
+        // LDS behind the tile of x holds the workgroup's candidates until the end of the kernel
+        ft = FwdTopk{tau_val + (tk->k - 1), tk->k, count, cand_val, cand_idx, kTopkCap};
+        lds_topk = lds + (size_t)kTileBatch * kTopkPark * sizeof(int2);
     }
+    int npartial = 0;
+    double* corr = nullptr;
+    if (epi == kEpiLossGrad || epi == kEpiLossGradAndScores) {
+        npartial = blocks * (kTileThreads / 64);
+        FFI_TRY(loss_partial_buffer(s, npartial, la->nnz, &fl.partial, &corr, nullptr));
+        fl.scale = la->scale;
+        fl.kind = la->kind;
+        fl.words = la->nz_words;
+        fl.skip_zero_stores = la->skip_zero_stores ? 1 : 0;
+    }
+    if (epi == kEpiScores) FFI_TRY(launch_lane32_any<kEpiScores>(vec4, topk, xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds_topk, fl, ft, s));
+    else if (epi == kEpiLossGrad) FFI_TRY(launch_lane32_any<kEpiLossGrad>(vec4, topk, xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds_topk, fl, ft, s));
+    else if (epi == kEpiLossGradAndScores) FFI_TRY(launch_lane32_any<kEpiLossGradAndScores>(vec4, topk, xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds_topk, fl, ft, s));
+    else FFI_TRY(launch_lane32_any<kEpiNone>(vec4, topk, xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds_topk, fl, ft, s));
+    if (topk) {
+        FFI_TRY(launch_topk_candidates_select(ft.cand_val, ft.cand_idx, count, d.B, kTopkCap, tk->k, tk->values, tk->indices, s));
+    }
+    if (epi != kEpiLossGrad && epi != kEpiLossGradAndScores) return FFI_OK;
     // the listed label positions: from the score matrix when it was written, else recomputed from x ([N,B] here)
     Dims dt = d;
     dt.tp = true;
@@ -258,21 +406,33 @@ int forward_tiles(const float* x, const int32_t* idx, const float* w, const floa
 int launch_forward(const float* x, const int32_t* idx, const float* w, const float* bias, float* out, const Dims& d,
                    hipStream_t s) {
     // (the kernel reaches the 32 rows of out of a batch tile through 32-bit byte offsets)
-    if (tile_path_fits(d.N) && d.L < (1 << 25)) return forward_tiles(x, idx, w, bias, out, nullptr, kEpiScores, nullptr, d, s);
+    if (tile_path_fits(d.N) && d.L < (1 << 25)) return forward_tiles(x, idx, w, bias, out, nullptr, kEpiScores, nullptr, nullptr, d, s);
     return launch_forward_wide(x, idx, w, bias, out, d, s);
 }
 
 int launch_forward_loss(const float* x, const int32_t* idx, const float* w, const float* bias, const LossArgs& la,
-                        float* scores, float* g, const Dims& d, hipStream_t s) {
+                        float* scores, float* g, const TopkArgs* tk, const Dims& d, hipStream_t s) {
     if (tile_path_fits(d.N) && d.L < (1 << 25)) {
-        if (scores == nullptr) return forward_tiles(x, idx, w, bias, g, nullptr, kEpiLossGrad, &la, d, s);
-        return forward_tiles(x, idx, w, bias, scores, g, kEpiLossGradAndScores, &la, d, s);
+        if (scores == nullptr) return forward_tiles(x, idx, w, bias, g, nullptr, kEpiLossGrad, &la, tk, d, s);
+        return forward_tiles(x, idx, w, bias, scores, g, kEpiLossGradAndScores, &la, tk, d, s);
     }
-    // wide inputs: scores by the wide kernel (into g itself when the caller wants no scores), then the
-    // loss gradient as a pass of its own
+    // wide inputs: scores by the wide kernel (into g itself when the caller wants no scores), top-k from them, then
+    // the loss gradient as a pass of its own
     float* sc = scores ? scores : g;
     FFI_TRY(launch_forward_wide(x, idx, w, bias, sc, d, s));
+    if (tk != nullptr) FFI_TRY(launch_topk_f32(sc, d.B, d.L, tk->k, tk->values, tk->indices, s));
     return launch_loss_grad(la, sc, g, d.B, d.L, s);
+}
+
+int launch_forward_topk(const float* x, const int32_t* idx, const float* w, const float* bias, float* scores, const TopkArgs& tk,
+                        const Dims& d, hipStream_t s) {
+    if (tile_path_fits(d.N) && d.L < (1 << 25))
+        return forward_tiles(x, idx, w, bias, scores, nullptr, scores ? kEpiScores : kEpiNone, nullptr, &tk, d, s);
+    // wide inputs: the score matrix (the caller's, or a workspace), then its top-k
+    float* sc = scores;
+    if (sc == nullptr) FFI_TRY(workspace_get(s, kWsScores, (size_t)d.B * d.L * sizeof(float), (void**)&sc));
+    FFI_TRY(launch_forward_wide(x, idx, w, bias, sc, d, s));
+    return launch_topk_f32(sc, d.B, d.L, tk.k, tk.values, tk.indices, s);
 }
 
 }  // namespace ffi

@@ -38,7 +38,7 @@ int hip_fail(hipError_t e);
 
 // Library-owned device scratch, one buffer per (device, stream, slot), grown on demand and kept.
 // Work that uses a buffer is ordered by the stream it belongs to.
-enum WorkspaceSlot { kWsFeaturesT = 0, kWsPartials = 1, kWsSlots = 2, kWsLoss = 3, kWsNonzero = 4, kWsGradients = 5, kWsRewire = 6 };
+enum WorkspaceSlot { kWsFeaturesT = 0, kWsPartials = 1, kWsSlots = 2, kWsLoss = 3, kWsNonzero = 4, kWsGradients = 5, kWsRewire = 6, kWsTopk = 7, kWsScores = 8 };
 int workspace_get(hipStream_t s, int slot, size_t bytes, void** out);
 void workspace_clear(int device);
 size_t workspace_bytes(int device);
@@ -91,9 +91,27 @@ int launch_loss_grad(const LossArgs& la, const float* scores, float* g, int B, i
 // out[3] (device doubles): scores above the threshold, sum of label values at such positions, sum of label values
 int launch_threshold_metrics(const float* scores, const int64_t* indices, const float* values, int nnz, float threshold, int B,
                              int L, double* out, hipStream_t s);
-// forward pass whose epilogue turns the scores into loss gradients (scores may be null)
+// per-sample top-k wanted from a forward pass: values / indices are [B, k], 1 <= k <= 8
+struct TopkArgs {
+    int k;
+    float* values;
+    int32_t* indices;
+};
+// forward pass whose epilogue turns the scores into loss gradients (scores may be null; tk may be null)
 int launch_forward_loss(const float* x, const int32_t* idx, const float* w, const float* bias, const LossArgs& la,
-                        float* scores, float* g, const Dims& d, hipStream_t s);
+                        float* scores, float* g, const TopkArgs* tk, const Dims& d, hipStream_t s);
+// forward pass with per-sample top-k; the score matrix is written only if `scores` is given
+int launch_forward_topk(const float* x, const int32_t* idx, const float* w, const float* bias, float* scores, const TopkArgs& tk,
+                        const Dims& d, hipStream_t s);
+// Candidate lists for a threshold-based top-k: count[B] appended entries, cand_val / cand_idx [B][kTopkCap].
+constexpr int kTopkCap = 8192;          // candidate slots per sample (a multiple of 8)
+int launch_topk_candidates_init(int* count, int* cand_idx, int B, int cap, hipStream_t s);
+// the k best candidates of every sample; a sample whose count exceeds cap gets labels -2 and NaN scores
+int launch_topk_candidates_select(const float* cand_val, const int* cand_idx, const int* count, int B, int cap, int k,
+                                  float* values, int32_t* indices, hipStream_t s);
+// the k best of nlists * 8 (score, label) candidates per sample (label -1 = empty slot)
+int launch_topk_merge(const float* part_val, const int* part_idx, int B, int nlists, int k, float* values, int32_t* indices,
+                      hipStream_t s);
 
 // ---- backward pass over the non-zero entries of out_grad only (ffi_sparse_grad.hip) -------------
 // words[t][j]: bit i set <=> out_grad[32 t + i, j] may be non-zero

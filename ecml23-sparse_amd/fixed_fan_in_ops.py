@@ -368,3 +368,24 @@ def rewire_connections(lookup, weights, arrays, num_features, threshold, seed):
                                              int(num_features), threshold.data_ptr(), int(seed) & (2**64 - 1), changed.data_ptr(),
                                              _stream_handle(lookup.device)))
     return changed
+
+
+def fan_in_sparse_topk(features, lookup, weights, bias=None, k=5, transposed=False, want_scores=False):
+    """``(values [B,k], labels [B,k] int32)`` of the k best fp32 scores per sample (best first, equal scores
+    by ascending label), and the score matrix as a third result if ``want_scores``.  Without
+    ``want_scores`` the ``[B,L]`` matrix is never written.  A sample whose candidate list overflows (see
+    the C header) gets labels -2."""
+    batch, num_features, num_units, fan_in = _check_inputs(features, lookup, weights, transposed)
+    if bias is not None:
+        _check_bias(bias, weights, num_units)
+        bias = bias.contiguous()
+    features, lookup, weights = features.contiguous(), lookup.contiguous(), weights.contiguous()
+    with torch.cuda.device(features.device):
+        values = torch.empty((batch, k), dtype=torch.float32, device=features.device)
+        labels = torch.empty((batch, k), dtype=torch.int32, device=features.device)
+        scores = torch.empty((batch, num_units), dtype=torch.float32, device=features.device) if want_scores else None
+        _lib.check(_lib.lib().ffi_forward_topk_f32(
+            features.data_ptr(), lookup.data_ptr(), weights.data_ptr(), bias.data_ptr() if bias is not None else None,
+            scores.data_ptr() if want_scores else None, values.data_ptr(), labels.data_ptr(),
+            batch, num_features, num_units, fan_in, int(k), int(transposed), _stream_handle(features.device)))
+    return (values, labels, scores) if want_scores else (values, labels)

@@ -67,11 +67,13 @@ def sparse_loss_grad(scores, y_true, kind, grad_scale=None, in_place=False, want
 
 
 def forward_loss(features, lookup, weights, bias, y_true, kind, grad_scale=None, transposed=False, want_scores=False,
-                 want_masks=False, skip_zero_stores=False):
+                 want_masks=False, skip_zero_stores=False, topk=0):
     """Forward pass, bias add and loss gradient in one kernel: ``(scores or None, out_grad, loss_sum)``,
     plus the bit masks of the non-zero gradients with ``want_masks``.  With ``skip_zero_stores`` (needs
     ``want_masks``) ``out_grad`` is written only where its mask bit is set and is undefined elsewhere:
-    hand it to ``backward_sparse(..., grad_is_partial=True)``."""
+    hand it to ``backward_sparse(..., grad_is_partial=True)``.  With ``topk`` = k (1..8) the per-sample k best
+    scores and their labels (``[B,k]`` each) are appended to the results as a pair: the P@k metrics of the step
+    without the score matrix."""
     batch, num_features, num_units, fan_in = _check_inputs(features, lookup, weights, transposed)
     if bias is not None:
         _check_bias(bias, weights, num_units)
@@ -86,15 +88,22 @@ def forward_loss(features, lookup, weights, bias, y_true, kind, grad_scale=None,
         scores = torch.empty_like(out_grad) if want_scores else None
         loss_sum = torch.empty((1,), dtype=torch.float32, device=features.device)
         masks = torch.empty(((batch + 31) // 32, num_units), dtype=torch.int32, device=features.device) if want_masks else None
-        _lib.check(_lib.lib().ffi_forward_loss_f32(
-            features.data_ptr(), lookup.data_ptr(), weights.data_ptr(), bias.data_ptr() if bias is not None else None,
-            indices.data_ptr() if indices.numel() else None,
-            values.data_ptr() if values is not None and values.numel() else None, indices.shape[0],
-            int(kind) | (SKIP_ZERO_STORES if skip_zero_stores else 0), scale,
-            scores.data_ptr() if want_scores else None, out_grad.data_ptr(), loss_sum.data_ptr(),
-            masks.data_ptr() if want_masks else None,
-            batch, num_features, num_units, fan_in, int(transposed), _stream_handle(features.device)))
-    return (scores, out_grad, loss_sum, masks) if want_masks else (scores, out_grad, loss_sum)
+        common = (features.data_ptr(), lookup.data_ptr(), weights.data_ptr(), bias.data_ptr() if bias is not None else None,
+                  indices.data_ptr() if indices.numel() else None,
+                  values.data_ptr() if values is not None and values.numel() else None, indices.shape[0],
+                  int(kind) | (SKIP_ZERO_STORES if skip_zero_stores else 0), scale,
+                  scores.data_ptr() if want_scores else None, out_grad.data_ptr(), loss_sum.data_ptr(),
+                  masks.data_ptr() if want_masks else None)
+        shape = (batch, num_features, num_units, fan_in, int(transposed), _stream_handle(features.device))
+        top = None
+        if topk:
+            top = (torch.empty((batch, topk), dtype=torch.float32, device=features.device),
+                   torch.empty((batch, topk), dtype=torch.int32, device=features.device))
+            _lib.check(_lib.lib().ffi_forward_loss_topk_f32(*common, top[0].data_ptr(), top[1].data_ptr(), int(topk), *shape))
+        else:
+            _lib.check(_lib.lib().ffi_forward_loss_f32(*common, *shape))
+    result = (scores, out_grad, loss_sum, masks) if want_masks else (scores, out_grad, loss_sum)
+    return result + (top,) if topk else result
 
 
 def _scaled(out_grad, upstream):

@@ -240,6 +240,29 @@ int ffi_forward_loss_f32(const float* features, const int32_t* lookup, const flo
                          int transposed, ffi_stream_t stream);
 
 /*
+ * Forward pass with a per-sample top-k in fp32 (1 <= k <= 8), same ordering rule as ffi_forward_topk_bf16 (scores
+ * descending, equal scores by ascending label: tf.nn.top_k, sparse/metrics.py:19).  `bias` may be NULL.  The
+ * [batch, num_units] score matrix is written only if `scores` is given.  How: a sample of the labels is scored
+ * first and fixes, per sample, a threshold that k labels are known to reach; the forward kernel then appends
+ * every score at or above its sample's threshold to a candidate list (a tiny share of all labels), and the k
+ * best candidates are selected.  The result is exact.  A sample whose candidates overflow its list (8192 slots;
+ * e.g. thousands of labels tied with the k-th score) gets labels -2 and NaN scores instead.
+ * ffi_forward_loss_topk_f32 is ffi_forward_loss_f32 with the same top-k of the scores as a by-product: what a
+ * training step needs for the loss, the backward pass and the P@k metrics (sparse/metrics.py:31-71) without
+ * the score matrix ever being stored.  No counterpart in the reference.
+ */
+int ffi_forward_topk_f32(const float* features, const int32_t* lookup, const float* weights, const float* bias,
+                         float* scores, float* topk_values, int32_t* topk_indices,
+                         int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in,
+                         int k, int transposed, ffi_stream_t stream);
+int ffi_forward_loss_topk_f32(const float* features, const int32_t* lookup, const float* weights, const float* bias,
+                              const int64_t* label_indices, const float* label_values, int64_t nnz,
+                              int loss_kind, float grad_scale, float* scores, float* out_grad, float* loss_sum,
+                              uint32_t* nz_words, float* topk_values, int32_t* topk_indices, int k,
+                              int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in,
+                              int transposed, ffi_stream_t stream);
+
+/*
  * Backward pass that skips the exact zeros of out_grad, as the reference's GPU kernels do entry by
  * entry (`if(out == 0) continue`, tfsparse/cc/kernels/backward.cu.h:73,94,131,151): with a hinge loss
  * every satisfied margin has gradient 0, and late in training that is nearly all of them.  Same

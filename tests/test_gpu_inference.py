@@ -146,3 +146,81 @@ def test_inference_argument_errors(ffi):
         ops.fan_in_sparse_topk_bf16(x, lookup, w, k=0)
     with pytest.raises(RuntimeError):
         ops.fan_in_sparse_matmul_bf16(x.cpu(), lookup.cpu(), w.cpu())
+
+
+# ---- fp32 forward with fused top-k (no score matrix) ------------------------------------------------------------
+#            B    N     L      K  transposed
+TOPK_F32 = [(128, 768, 20000, 32, True),
+            (37, 300, 9001, 7, False),
+            (64, 512, 12000, 64, True),
+            (5, 96, 700, 40, False),          # fewer labels than the threshold sample
+            (40, 1216, 6000, 16, True),       # the widest input whose tile of x fits in LDS
+            (33, 3000, 5000, 12, True)]       # wide inputs: scores, then their top-k
+
+
+@pytest.mark.parametrize("k", [1, 5, 8])
+@pytest.mark.parametrize("shape", TOPK_F32)
+def test_fp32_topk_without_the_score_matrix(ffi, shape, k):
+    # exact: the labels and scores are those of the top-k (tf.nn.top_k order) of the scores the same kernel writes
+    B, N, L, K, tp = shape
+    rng = np.random.default_rng(sum(shape[:4]) + k)
+    x = np.maximum(rng.standard_normal((B, N)), 0).astype(np.float32)
+    lookup = rng.integers(0, N, size=(L, K)).astype(np.int32)
+    w = rng.standard_normal((L, K)).astype(np.float32)
+    bias = (rng.standard_normal(L) * 0.3).astype(np.float32)
+    feats = np.ascontiguousarray(x.T) if tp else x
+    dev = lambda a: torch.from_numpy(a).cuda()  # noqa: E731
+    v1, i1, scores = ffi.fan_in_sparse_topk(dev(feats), dev(lookup), dev(w), dev(bias), k=k, transposed=tp, want_scores=True)
+    v2, i2 = ffi.fan_in_sparse_topk(dev(feats), dev(lookup), dev(w), dev(bias), k=k, transposed=tp)
+    torch.cuda.synchronize()
+    sc = scores.cpu().numpy()
+    ref_v, ref_i = oracle.topk(sc, k)
+    assert np.array_equal(i1.cpu().numpy(), ref_i) and np.array_equal(v1.cpu().numpy(), ref_v)
+    assert np.array_equal(i2.cpu().numpy(), ref_i) and np.array_equal(v2.cpu().numpy(), ref_v)
+    # and the scores are the layer's
+    assert rel_err(sc, oracle.forward(feats, lookup, w, transposed=tp) + bias[None, :]) <= 1e-5
+
+
+def test_fp32_topk_with_ties_and_cancellation(ffi):
+    # many exactly equal scores (ties broken by label) and scores that are sums of large cancelling terms
+    B, N, L, K = 40, 64, 9000, 4
+    rng = np.random.default_rng(3)
+    x = rng.integers(-3, 4, (B, N)).astype(np.float32) * 1000.0
+    lookup = rng.integers(0, N, size=(L, K)).astype(np.int32)
+    w = rng.integers(-2, 3, (L, K)).astype(np.float32)
+    dev = lambda a: torch.from_numpy(a).cuda()  # noqa: E731
+    v, i, scores = ffi.fan_in_sparse_topk(dev(x), dev(lookup), dev(w), None, k=8, want_scores=True)
+    v2, i2 = ffi.fan_in_sparse_topk(dev(x), dev(lookup), dev(w), None, k=8)
+    torch.cuda.synchronize()
+    ref_v, ref_i = oracle.topk(scores.cpu().numpy(), 8)
+    assert np.array_equal(i.cpu().numpy(), ref_i) and np.array_equal(v.cpu().numpy(), ref_v)
+    assert np.array_equal(i2.cpu().numpy(), ref_i)
+
+
+def test_fp32_topk_with_a_run_of_high_scores(ffi):
+    # 300 neighbouring labels beat every other one: one workgroup meets far more candidates of a sample than it parks
+    B, N, L, K = 6, 128, 30000, 8
+    rng = np.random.default_rng(11)
+    x = np.abs(rng.standard_normal((B, N))).astype(np.float32)
+    lookup = rng.integers(0, N, size=(L, K)).astype(np.int32)
+    w = rng.standard_normal((L, K)).astype(np.float32)
+    w[7000:7300] = np.abs(w[7000:7300]) + 5.0
+    dev = lambda a: torch.from_numpy(a).cuda()  # noqa: E731
+    v, i, scores = ffi.fan_in_sparse_topk(dev(x), dev(lookup), dev(w), None, k=8, want_scores=True)
+    v2, i2 = ffi.fan_in_sparse_topk(dev(x), dev(lookup), dev(w), None, k=8)
+    torch.cuda.synchronize()
+    ref_v, ref_i = oracle.topk(scores.cpu().numpy(), 8)
+    assert (ref_i >= 7000).all() and (ref_i < 7300).all()
+    assert np.array_equal(i.cpu().numpy(), ref_i) and np.array_equal(v.cpu().numpy(), ref_v)
+    assert np.array_equal(i2.cpu().numpy(), ref_i) and np.array_equal(v2.cpu().numpy(), ref_v)
+
+
+def test_fp32_topk_overflow_is_reported(ffi):
+    # every label ties with the best score: no list of 8192 candidates can hold them, the sample gets -2
+    B, N, L, K = 3, 16, 20000, 2
+    x = torch.ones((B, N), device="cuda")
+    lookup = torch.zeros((L, K), dtype=torch.int32, device="cuda")
+    w = torch.ones((L, K), device="cuda")
+    v, i = ffi.fan_in_sparse_topk(x, lookup, w, None, k=3)
+    torch.cuda.synchronize()
+    assert bool((i == -2).all()) and bool(torch.isnan(v).all())

@@ -273,3 +273,33 @@ def test_unaligned_score_buffers(ffi):
     g2, _ = ffi.metrics.sparse_loss_grad(view, y, oracle.LOSS_SQUARED_HINGE, grad_scale=1.0, in_place=True)
     torch.cuda.synchronize()
     assert g2.data_ptr() == view.data_ptr() and rel_err(view.cpu().numpy(), grad) <= RTOL
+
+
+@pytest.mark.parametrize("shape", [(128, 768, 20000, 32, True), (37, 300, 9001, 7, False), (33, 3000, 5000, 12, True)])
+def test_forward_loss_with_topk_by_product(ffi, shape):
+    # loss gradient, masks, loss sum and the top-5 of the scores from one forward pass; the top-5 equals that of the
+    # separately written score matrix, the rest is unchanged by asking for it
+    B, N, L, K, tp = shape
+    rng = np.random.default_rng(sum(shape[:4]))
+    x = np.maximum(rng.standard_normal((B, N)), 0).astype(np.float32)
+    lookup = rng.integers(0, N, size=(L, K)).astype(np.int32)
+    w = (rng.standard_normal((L, K)) * 0.4).astype(np.float32)
+    bias = np.full(L, -1.0, np.float32)
+    indices, values = label_list(rng, B, L)
+    feats = np.ascontiguousarray(x.T) if tp else x
+    dev = lambda a: torch.from_numpy(a).cuda()  # noqa: E731
+    y = (dev(indices), dev(values))
+    args = (dev(feats), dev(lookup), dev(w), dev(bias), y, oracle.LOSS_SQUARED_HINGE)
+    scores, g0, l0, m0 = ffi.metrics.forward_loss(*args, transposed=tp, want_scores=True, want_masks=True)
+    none, g1, l1, m1, (tv, ti) = ffi.metrics.forward_loss(*args, transposed=tp, want_masks=True, topk=5)
+    torch.cuda.synchronize()
+    assert none is None
+    ref_v, ref_i = oracle.topk(scores.cpu().numpy(), 5)
+    assert np.array_equal(ti.cpu().numpy(), ref_i) and np.array_equal(tv.cpu().numpy(), ref_v)
+    assert torch.equal(m0, m1) and float(l0) == float(l1)
+    assert rel_err(g1.cpu().numpy(), g0.cpu().numpy()) <= RTOL
+    p5 = ffi.PrecisionAtK(k=5)
+    p5.update_from_topk(y, ti, L)
+    truth = np.zeros((B, L), np.float32)
+    truth[indices[:, 0], indices[:, 1]] = values
+    assert abs(p5.result() - truth[np.arange(B)[:, None], ref_i].sum() / (B * 5)) < 1e-9
