@@ -224,3 +224,29 @@ def test_fp32_topk_overflow_is_reported(ffi):
     v, i = ffi.fan_in_sparse_topk(x, lookup, w, None, k=3)
     torch.cuda.synchronize()
     assert bool((i == -2).all()) and bool(torch.isnan(v).all())
+
+
+def test_inference_config_full_size(ffi):
+    # c5 at its full size (batch 512, 100,000 inputs, 670,091 labels, fan-in 64, sorted rows, bf16): the fused top-5 equals
+    # the top-5 of the score matrix the unfused kernel writes, and a label slice of those scores meets both oracle gates
+    from ecml23_sparse_amd import synth
+    cfg = synth.CONFIGS["c5"]
+    t = synth.make_inputs(cfg, seed=42, device="cuda", transposed=True)
+    x, lookup, w = t["features"].to(torch.bfloat16), t["lookup"], t["weights"].to(torch.bfloat16)
+    print("case config=c5 full size", flush=True)
+    vals, labels = ffi.fan_in_sparse_topk_bf16(x, lookup, w, k=5, transposed=True)
+    scores = ffi.fan_in_sparse_matmul_bf16(x, lookup, w, transposed=True)
+    ref_v, ref_i = ffi.topk_scores(scores, 5)
+    torch.cuda.synchronize()
+    assert torch.equal(labels, ref_i) and torch.equal(vals, ref_v)
+    # the device top-k itself, on a few samples, against the oracle's
+    rows = scores[:4].cpu().numpy()
+    o_v, o_i = oracle.topk(rows, 5)
+    assert np.array_equal(ref_i[:4].cpu().numpy(), o_i) and np.array_equal(ref_v[:4].cpu().numpy(), o_v)
+    sl = slice(123_000, 123_500)
+    xs = x.float().cpu().numpy()
+    ls, ws = lookup[sl].cpu().numpy(), w[sl].float().cpu().numpy()
+    got = scores[:, sl].cpu().numpy()
+    assert rel_err(got, oracle.forward(xs, ls, ws, transposed=True)) <= SAME_INPUT_RTOL
+    x32 = t["features"].cpu().numpy()
+    assert rel_err(got, oracle.forward(x32, ls, t["weights"][sl].cpu().numpy(), transposed=True)) <= FP32_INPUT_RTOL
