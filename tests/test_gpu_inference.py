@@ -154,6 +154,7 @@ TOPK_F32 = [(128, 768, 20000, 32, True),
             (37, 300, 9001, 7, False),
             (64, 512, 12000, 64, True),
             (5, 96, 700, 40, False),          # fewer labels than the threshold sample
+            (3, 16, 3, 4, False),             # fewer labels than k: the missing places are (-inf, -1) as in the oracle
             (40, 1216, 6000, 16, True),       # the widest input whose tile of x fits in LDS
             (33, 3000, 5000, 12, True)]       # wide inputs: scores, then their top-k
 
@@ -213,6 +214,19 @@ def test_fp32_topk_with_a_run_of_high_scores(ffi):
     assert (ref_i >= 7000).all() and (ref_i < 7300).all()
     assert np.array_equal(i.cpu().numpy(), ref_i) and np.array_equal(v.cpu().numpy(), ref_v)
     assert np.array_equal(i2.cpu().numpy(), ref_i) and np.array_equal(v2.cpu().numpy(), ref_v)
+
+
+def test_fp32_topk_argument_errors(ffi):
+    x = torch.zeros((4, 16), device="cuda")
+    lookup = torch.zeros((5, 2), dtype=torch.int32, device="cuda")
+    w = torch.zeros((5, 2), device="cuda")
+    for k in (0, 9):
+        with pytest.raises(ffi._lib.FfiError):
+            ffi.fan_in_sparse_topk(x, lookup, w, None, k=k)
+    with pytest.raises(ValueError):
+        ffi.fan_in_sparse_topk(x, lookup, w, torch.zeros(4, device="cuda"), k=1)      # bias of the wrong length
+    with pytest.raises(RuntimeError):
+        ffi.fan_in_sparse_topk(x.cpu(), lookup.cpu(), w.cpu(), None, k=1)
 
 
 def test_fp32_topk_overflow_is_reported(ffi):
