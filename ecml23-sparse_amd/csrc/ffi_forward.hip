@@ -24,9 +24,13 @@ namespace {
 // the chunk order skewed by its lane id; the accumulators are brought back to natural batch order
 // before the stores, which are then full 256-byte rows of out per wavefront.
 // ------------------------------------------------------------------------------------------------
+// `base` is a raw LDS address: (address of the tile + (lane & 7) * 16) + row * 128.  The tile is 128-byte aligned, so the
+// chunk bits can be flipped with XOR after the add: one add and seven XORs per row instead of an add per read.
+typedef float lds_v4f __attribute__((ext_vector_type(4)));
+typedef const lds_v4f __attribute__((address_space(3)))* lds_v4f_ptr;
 template <int C>
-__device__ __forceinline__ void fwd_lane_step(const char* __restrict__ xs_bytes, unsigned base, float wv, float (&acc)[32]) {
-    const float4 v = *reinterpret_cast<const float4*>(xs_bytes + skew_addr<C>(base));
+__device__ __forceinline__ void fwd_lane_step(unsigned base, float wv, float (&acc)[32]) {
+    const lds_v4f v = *(lds_v4f_ptr)(size_t)(skew_addr<C>(base));
     acc[4 * C + 0] = fmaf(wv, v.x, acc[4 * C + 0]);
     acc[4 * C + 1] = fmaf(wv, v.y, acc[4 * C + 1]);
     acc[4 * C + 2] = fmaf(wv, v.z, acc[4 * C + 2]);
@@ -102,12 +106,11 @@ __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* _
                                                                   float* __restrict__ out, int B, int N,
                                                                   int L, int K, int nbt, int labels_per_stream,
                                                                   FwdLoss fl, FwdTopk ft) {
-    extern __shared__ __align__(16) float xs[];
+    extern __shared__ __align__(128) float xs[];
     __shared__ __align__(16) float tau_s[kTileBatch];
     __shared__ int local_count[kTileBatch];      // candidates parked per batch row (may run past kTopkPark)
     __shared__ int local_base[kTileBatch];
     int2* local_cand = reinterpret_cast<int2*>(xs + (size_t)N * kTileBatch);      // behind the tile (TOPK launches only)
-    const char* xs_bytes = reinterpret_cast<const char*>(xs);
     const int u = xcd_contiguous_block(blockIdx.x, gridDim.x);
     const int bt = u % nbt, stream = u / nbt;
     const int b0 = bt * kTileBatch;
@@ -117,7 +120,7 @@ __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* _
         tau_s[threadIdx.x] = b0 + (int)threadIdx.x < B ? ft.tau[(size_t)(b0 + threadIdx.x) * ft.tau_stride] : __builtin_inff();
     __syncthreads();
     const int lane = threadIdx.x & 63;
-    const unsigned skew = (unsigned)(lane & 7) * 16u;
+    const unsigned skewbase = (unsigned)(size_t)(__attribute__((address_space(3))) float*)xs + (unsigned)(lane & 7) * 16u;
     const int l_begin = stream * labels_per_stream;
     const int l_end = min(l_begin + labels_per_stream, L);
     const int nchunks = (K + 31) / 32;
@@ -168,11 +171,11 @@ __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* _
             for (int k = 0; k < 32; ++k) {
                 if (full || k < kn) {
                     const unsigned id = (k & 1) ? (idp[k >> 1] >> 16) : (idp[k >> 1] & 0xffffu);
-                    const unsigned rb = (id << 7) | skew;
-                    fwd_lane_step<0>(xs_bytes, rb, wv[k], acc); fwd_lane_step<1>(xs_bytes, rb, wv[k], acc);
-                    fwd_lane_step<2>(xs_bytes, rb, wv[k], acc); fwd_lane_step<3>(xs_bytes, rb, wv[k], acc);
-                    fwd_lane_step<4>(xs_bytes, rb, wv[k], acc); fwd_lane_step<5>(xs_bytes, rb, wv[k], acc);
-                    fwd_lane_step<6>(xs_bytes, rb, wv[k], acc); fwd_lane_step<7>(xs_bytes, rb, wv[k], acc);
+                    const unsigned rb = (id << 7) + skewbase;
+                    fwd_lane_step<0>(rb, wv[k], acc); fwd_lane_step<1>(rb, wv[k], acc);
+                    fwd_lane_step<2>(rb, wv[k], acc); fwd_lane_step<3>(rb, wv[k], acc);
+                    fwd_lane_step<4>(rb, wv[k], acc); fwd_lane_step<5>(rb, wv[k], acc);
+                    fwd_lane_step<6>(rb, wv[k], acc); fwd_lane_step<7>(rb, wv[k], acc);
                 }
             }
         }
