@@ -1,0 +1,282 @@
+// A C++ caller of the C-ABI library with neither Python nor torch in the process: what the reference's own
+// test and benchmark programs are to its kernels (testing/test.cpp, testing/quick-bench.cpp), this program is
+// to libffi_hip.so.  It allocates with hipMalloc, calls the extern "C" entry points on a stream of its own and
+// compares with the CPU oracle (test infrastructure, linked here and nowhere in the library).
+//
+//   cabi_harness test                 known-answer case (testing/test.cpp:13-47), then the reference's shape
+//                                     grid (testing/test.cpp:50-59) with its input law (uniform [-1,1], out_grad
+//                                     clipped at zero, outputs pre-filled with garbage:
+//                                     testing/test_case_templates.h:54-69,110-119) in both feature layouts,
+//                                     against the oracle with the reference's absolute gates (1e-5 forward,
+//                                     1.5e-5 gradients: test_case_templates.h:82,139-140; relative gates where the
+//                                     sums are too long for those).  Exit code = failures.
+//   cabi_harness bench [B N L K]      forward and backward timings in both layouts, 1 warm-up + 5 timed calls
+//                                     (testing/quick-bench.cpp:14-35; default shape {50, 32768, 670000, 32}).
+#include <hip/hip_runtime.h>
+
+#include <chrono>
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <thread>
+#include <vector>
+
+#include "ffi_hip.h"
+
+extern "C" {
+int ffi_oracle_forward_f32(const float* features, const int32_t* lookup, const float* weights, float* output, int64_t B,
+                           int64_t N, int64_t L, int64_t K, int transposed, int threads);
+int ffi_oracle_backward_f32(const float* features, const int32_t* lookup, const float* weights, const float* out_grad,
+                            float* feature_grad, float* weight_grad, int64_t B, int64_t N, int64_t L, int64_t K,
+                            int transposed, int threads);
+}
+
+namespace {
+
+#define HIP_OK(expr)                                                                              \
+    do {                                                                                          \
+        hipError_t e_ = (expr);                                                                   \
+        if (e_ != hipSuccess) {                                                                   \
+            std::fprintf(stderr, "%s:%d: %s: %s\n", __FILE__, __LINE__, #expr, hipGetErrorString(e_)); \
+            std::exit(2);                                                                         \
+        }                                                                                         \
+    } while (0)
+
+#define FFI_OK_OR_DIE(expr)                                                                       \
+    do {                                                                                          \
+        int s_ = (expr);                                                                          \
+        if (s_ != FFI_OK) {                                                                       \
+            std::fprintf(stderr, "%s:%d: %s -> %s\n", __FILE__, __LINE__, #expr, ffi_status_string(s_)); \
+            std::exit(2);                                                                         \
+        }                                                                                         \
+    } while (0)
+
+struct Rng {                       // splitmix64
+    uint64_t s;
+    uint64_t next() {
+        uint64_t z = (s += 0x9e3779b97f4a7c15ull);
+        z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+        z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+        return z ^ (z >> 31);
+    }
+    float uniform() { return (float)((double)(next() >> 11) * (2.0 / 9007199254740992.0) - 1.0); }   // [-1, 1)
+    int32_t below(int64_t n) { return (int32_t)(next() % (uint64_t)n); }
+};
+
+template <typename T>
+struct DeviceBuffer {
+    T* p = nullptr;
+    size_t n = 0;
+    explicit DeviceBuffer(size_t count) : n(count) { HIP_OK(hipMalloc((void**)&p, count * sizeof(T))); }
+    ~DeviceBuffer() { (void)hipFree(p); }
+    DeviceBuffer(const DeviceBuffer&) = delete;
+    DeviceBuffer& operator=(const DeviceBuffer&) = delete;
+    void upload(const std::vector<T>& h) { HIP_OK(hipMemcpy(p, h.data(), h.size() * sizeof(T), hipMemcpyHostToDevice)); }
+    std::vector<T> download() const {
+        std::vector<T> h(n);
+        HIP_OK(hipMemcpy(h.data(), p, n * sizeof(T), hipMemcpyDeviceToHost));
+        return h;
+    }
+};
+
+struct Shape { int64_t B, N, L, K; };
+
+struct Case {
+    Shape s;
+    bool transposed;
+    std::vector<float> features, weights, out_grad;
+    std::vector<int32_t> lookup;
+};
+
+Case make_case(const Shape& s, bool transposed, uint64_t seed) {
+    Case c{s, transposed, {}, {}, {}, {}};
+    Rng rng{seed};
+    std::vector<float> x((size_t)s.B * s.N);
+    for (float& v : x) v = rng.uniform();
+    if (transposed) {                                   // [N,B], the layout of the Tp ops
+        c.features.resize(x.size());
+        for (int64_t b = 0; b < s.B; ++b)
+            for (int64_t n = 0; n < s.N; ++n) c.features[(size_t)n * s.B + b] = x[(size_t)b * s.N + n];
+    } else {
+        c.features = x;
+    }
+    c.lookup.resize((size_t)s.L * s.K);
+    for (int32_t& v : c.lookup) v = rng.below(s.N);     // duplicates inside a row are legal, as in the reference's tests
+    c.weights.resize((size_t)s.L * s.K);
+    for (float& v : c.weights) v = rng.uniform();
+    c.out_grad.resize((size_t)s.B * s.L);
+    for (float& v : c.out_grad) { v = rng.uniform(); if (v < 0.f) v = 0.f; }
+    return c;
+}
+
+double max_abs_diff(const std::vector<float>& a, const std::vector<float>& b) {
+    double m = 0;
+    for (size_t i = 0; i < a.size(); ++i) {
+        const double d = std::fabs((double)a[i] - (double)b[i]);
+        if (!(d <= m)) m = d;                           // a NaN ends up as the maximum
+    }
+    return m;
+}
+
+double max_abs(const std::vector<float>& a) {
+    double m = 0;
+    for (float v : a) m = std::fmax(m, std::fabs((double)v));
+    return m;
+}
+
+int oracle_threads() { return (int)std::max(1u, std::thread::hardware_concurrency()); }
+
+int known_answer(hipStream_t stream) {
+    // testing/test.cpp:13-47: 3 samples x 3 features, 2 units x 2 connections
+    const std::vector<float> x = {1, 2, 3, 4, 5, 6, 0, 1, 1};
+    const std::vector<int32_t> lookup = {1, 2, 0, 2};
+    const std::vector<float> w = {1, 2, 3, 4};
+    const std::vector<float> expected = {8, 15, 17, 36, 3, 4};
+    int failures = 0;
+    for (int transposed = 0; transposed < 2; ++transposed) {
+        std::vector<float> f = x;
+        if (transposed)
+            for (int b = 0; b < 3; ++b)
+                for (int n = 0; n < 3; ++n) f[n * 3 + b] = x[b * 3 + n];
+        DeviceBuffer<float> dx(9), dw(4), dout(6);
+        DeviceBuffer<int32_t> dl(4);
+        dx.upload(f); dw.upload(w); dl.upload(lookup);
+        dout.upload(std::vector<float>(6, -77.f));
+        FFI_OK_OR_DIE(ffi_forward_f32(dx.p, dl.p, dw.p, dout.p, 3, 3, 2, 2, transposed, stream));
+        HIP_OK(hipStreamSynchronize(stream));
+        const bool ok = dout.download() == expected;
+        std::printf("known answer transposed=%d: %s\n", transposed, ok ? "ok" : "FAILED");
+        failures += !ok;
+    }
+    return failures;
+}
+
+int shape_grid(hipStream_t stream) {
+    const Shape grid[] = {{3, 5, 4, 2},       {12, 8, 8, 4},          {127, 254, 513, 4},    {12, 8, 32, 16},
+                          {17, 12, 63, 44},   {127, 254, 513, 73},    {127, 254, 513, 80},   {1, 32, 4000000, 4}};
+    int failures = 0;
+    for (const Shape& s : grid) {
+        for (int transposed = 0; transposed < 2; ++transposed) {
+            const Case c = make_case(s, transposed != 0, 42);
+            DeviceBuffer<float> dx(c.features.size()), dw(c.weights.size()), dg(c.out_grad.size());
+            DeviceBuffer<float> dout(c.out_grad.size()), dgx(c.features.size()), dgw(c.weights.size());
+            DeviceBuffer<int32_t> dl(c.lookup.size());
+            dx.upload(c.features); dw.upload(c.weights); dg.upload(c.out_grad); dl.upload(c.lookup);
+            // outputs start as garbage: the library has to overwrite every element
+            Rng junk{7};
+            std::vector<float> j1(dout.n), j2(dgx.n), j3(dgw.n);
+            for (float& v : j1) v = junk.uniform();
+            for (float& v : j2) v = junk.uniform();
+            for (float& v : j3) v = junk.uniform();
+            dout.upload(j1); dgx.upload(j2); dgw.upload(j3);
+            FFI_OK_OR_DIE(ffi_forward_f32(dx.p, dl.p, dw.p, dout.p, s.B, s.N, s.L, s.K, transposed, stream));
+            FFI_OK_OR_DIE(ffi_backward_f32(dx.p, dl.p, dw.p, dg.p, dgx.p, dgw.p, s.B, s.N, s.L, s.K, transposed, stream));
+            HIP_OK(hipStreamSynchronize(stream));
+            std::vector<float> out(dout.n), gx(dgx.n), gw(dgw.n);
+            const int th = oracle_threads();
+            if (ffi_oracle_forward_f32(c.features.data(), c.lookup.data(), c.weights.data(), out.data(), s.B, s.N, s.L, s.K,
+                                       transposed, th) != 0 ||
+                ffi_oracle_backward_f32(c.features.data(), c.lookup.data(), c.weights.data(), c.out_grad.data(), gx.data(),
+                                        gw.data(), s.B, s.N, s.L, s.K, transposed, th) != 0) {
+                std::fprintf(stderr, "oracle failed\n");
+                std::exit(2);
+            }
+            const double e_out = max_abs_diff(dout.download(), out);
+            const double e_gx = max_abs_diff(dgx.download(), gx);
+            const double e_gw = max_abs_diff(dgw.download(), gw);
+            // The reference's absolute gates; where a result is a long sum (4,000,000 labels feed 32 input columns:
+            // 500,000 terms each) the order of fp32 additions alone moves it by more than that, and the gate is the
+            // relative one of the parity tests (1e-5 forward, 1e-4 gradients, of the largest reference value).
+            const bool ok = (e_out < 1e-5 || e_out <= 1e-5 * max_abs(out)) && (e_gx < 1.5e-5 || e_gx <= 1e-4 * max_abs(gx)) &&
+                            (e_gw < 1.5e-5 || e_gw <= 1e-4 * max_abs(gw));
+            std::printf("shape {%lld, %lld, %lld, %lld} transposed=%d: max |diff| forward %.2e feature_grad %.2e weight_grad %.2e %s\n",
+                        (long long)s.B, (long long)s.N, (long long)s.L, (long long)s.K, transposed, e_out, e_gx, e_gw,
+                        ok ? "ok" : "FAILED");
+            std::fflush(stdout);
+            failures += !ok;
+        }
+    }
+    return failures;
+}
+
+int error_codes(hipStream_t stream) {
+    // the reference aborts on these (gsl_Expects, forward.cu:19-28); the library reports them
+    DeviceBuffer<float> a(16);
+    DeviceBuffer<int32_t> l(16);
+    int failures = 0;
+    failures += ffi_forward_f32(nullptr, l.p, a.p, a.p, 2, 2, 2, 2, 0, stream) != FFI_ERR_NULL_POINTER;
+    failures += ffi_forward_f32(a.p, l.p, a.p, a.p, 0, 2, 2, 2, 0, stream) != FFI_ERR_BAD_SHAPE;
+    failures += ffi_forward_f32(a.p, l.p, a.p, a.p, 2, 2, (int64_t)1 << 31, 2, 0, stream) != FFI_ERR_TOO_LARGE;
+    std::printf("status codes: %s\n", failures ? "FAILED" : "ok");
+    return failures;
+}
+
+template <typename F>
+double time_ms(hipStream_t stream, int iters, F&& call) {
+    call();                                             // warm-up (builds the plan of the lookup on first use)
+    HIP_OK(hipStreamSynchronize(stream));
+    hipEvent_t a, b;
+    HIP_OK(hipEventCreate(&a));
+    HIP_OK(hipEventCreate(&b));
+    HIP_OK(hipEventRecord(a, stream));
+    for (int i = 0; i < iters; ++i) call();
+    HIP_OK(hipEventRecord(b, stream));
+    HIP_OK(hipEventSynchronize(b));
+    float ms = 0;
+    HIP_OK(hipEventElapsedTime(&ms, a, b));
+    HIP_OK(hipEventDestroy(a));
+    HIP_OK(hipEventDestroy(b));
+    return ms / iters;
+}
+
+int bench(hipStream_t stream, const Shape& s) {
+    std::printf("shape {%lld, %lld, %lld, %lld}\n", (long long)s.B, (long long)s.N, (long long)s.L, (long long)s.K);
+    for (int transposed = 0; transposed < 2; ++transposed) {
+        const Case c = make_case(s, transposed != 0, 42);
+        DeviceBuffer<float> dx(c.features.size()), dw(c.weights.size()), dg(c.out_grad.size());
+        DeviceBuffer<float> dout(c.out_grad.size()), dgx(c.features.size()), dgw(c.weights.size());
+        DeviceBuffer<int32_t> dl(c.lookup.size());
+        dx.upload(c.features); dw.upload(c.weights); dg.upload(c.out_grad); dl.upload(c.lookup);
+        const double fwd = time_ms(stream, 5, [&] {
+            FFI_OK_OR_DIE(ffi_forward_f32(dx.p, dl.p, dw.p, dout.p, s.B, s.N, s.L, s.K, transposed, stream));
+        });
+        const double bwd = time_ms(stream, 5, [&] {
+            FFI_OK_OR_DIE(ffi_backward_f32(dx.p, dl.p, dw.p, dg.p, dgx.p, dgw.p, s.B, s.N, s.L, s.K, transposed, stream));
+        });
+        std::printf("%s forward pass %.3f ms, backward pass %.3f ms\n", transposed ? "transposed" : "plain     ", fwd, bwd);
+        std::fflush(stdout);
+    }
+    return 0;
+}
+
+}  // namespace
+
+int main(int argc, char** argv) {
+    const char* mode = argc > 1 ? argv[1] : "test";
+    int ndev = 0;
+    if (hipGetDeviceCount(&ndev) != hipSuccess || ndev == 0) {
+        std::fprintf(stderr, "no GPU\n");
+        return 2;
+    }
+    HIP_OK(hipSetDevice(0));
+    hipStream_t stream;
+    HIP_OK(hipStreamCreate(&stream));
+    std::printf("libffi_hip ABI v%d for %s\n", ffi_abi_version(), ffi_target_arch());
+    int rc = 0;
+    if (std::strcmp(mode, "test") == 0) {
+        rc = known_answer(stream) + error_codes(stream) + shape_grid(stream);
+        std::printf("%d failure(s)\n", rc);
+    } else if (std::strcmp(mode, "bench") == 0) {
+        Shape s{50, 32768, 670000, 32};
+        if (argc == 6) s = Shape{std::atoll(argv[2]), std::atoll(argv[3]), std::atoll(argv[4]), std::atoll(argv[5])};
+        rc = bench(stream, s);
+    } else {
+        std::fprintf(stderr, "usage: %s test | bench [B N L K]\n", argv[0]);
+        rc = 2;
+    }
+    ffi_cache_clear();
+    HIP_OK(hipStreamDestroy(stream));
+    return rc;
+}
