@@ -147,6 +147,7 @@ const char* ffi_status_string(int status) {
 int ffi_forward_f32(const float* features, const int32_t* lookup, const float* weights, float* result,
                     int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in,
                     int transposed, ffi_stream_t stream) {
+    StreamCall call_lock((hipStream_t)stream);
     if (!features || !lookup || !weights || !result) return FFI_ERR_NULL_POINTER;
     Dims d;
     FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
@@ -156,6 +157,7 @@ int ffi_forward_f32(const float* features, const int32_t* lookup, const float* w
 int ffi_forward_bias_f32(const float* features, const int32_t* lookup, const float* weights, const float* bias,
                          float* result, int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in,
                          int transposed, ffi_stream_t stream) {
+    StreamCall call_lock((hipStream_t)stream);
     if (!features || !lookup || !weights || !bias || !result) return FFI_ERR_NULL_POINTER;
     Dims d;
     FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
@@ -165,6 +167,7 @@ int ffi_forward_bias_f32(const float* features, const int32_t* lookup, const flo
 int ffi_weight_grad_f32(const float* features, const int32_t* lookup, const float* out_grad,
                         float* weight_grad, int64_t batch, int64_t num_features, int64_t num_units,
                         int64_t fan_in, int transposed, ffi_stream_t stream) {
+    StreamCall call_lock((hipStream_t)stream);
     if (!features || !lookup || !out_grad || !weight_grad) return FFI_ERR_NULL_POINTER;
     Dims d;
     FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
@@ -174,6 +177,7 @@ int ffi_weight_grad_f32(const float* features, const int32_t* lookup, const floa
 int ffi_input_grad_f32(const int32_t* lookup, const float* weights, const float* out_grad,
                        float* feature_grad, int64_t batch, int64_t num_features, int64_t num_units,
                        int64_t fan_in, int transposed, ffi_stream_t stream) {
+    StreamCall call_lock((hipStream_t)stream);
     if (!lookup || !weights || !out_grad || !feature_grad) return FFI_ERR_NULL_POINTER;
     Dims d;
     FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
@@ -184,6 +188,7 @@ int ffi_backward_f32(const float* features, const int32_t* lookup, const float* 
                      const float* out_grad, float* feature_grad, float* weight_grad, int64_t batch,
                      int64_t num_features, int64_t num_units, int64_t fan_in, int transposed,
                      ffi_stream_t stream) {
+    StreamCall call_lock((hipStream_t)stream);
     if (!features || !lookup || !weights || !out_grad) return FFI_ERR_NULL_POINTER;
     if (!feature_grad && !weight_grad) return FFI_ERR_NULL_POINTER;
     Dims d;
@@ -201,6 +206,7 @@ int ffi_backward_bias_f32(const float* features, const int32_t* lookup, const fl
                           const float* out_grad, float* feature_grad, float* weight_grad, float* bias_grad,
                           int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in, int transposed,
                           ffi_stream_t stream) {
+    StreamCall call_lock((hipStream_t)stream);
     if (!features || !lookup || !weights || !out_grad || !weight_grad || !bias_grad) return FFI_ERR_NULL_POINTER;
     Dims d;
     FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
@@ -214,6 +220,7 @@ int ffi_backward_bias_f32(const float* features, const int32_t* lookup, const fl
 int ffi_forward_bf16_f32(const uint16_t* features, const int32_t* lookup, const uint16_t* weights, float* result,
                          int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in, int transposed,
                          ffi_stream_t stream) {
+    StreamCall call_lock((hipStream_t)stream);
     if (!features || !lookup || !weights || !result) return FFI_ERR_NULL_POINTER;
     Dims d;
     FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
@@ -223,6 +230,7 @@ int ffi_forward_bf16_f32(const uint16_t* features, const int32_t* lookup, const 
 int ffi_forward_topk_bf16(const uint16_t* features, const int32_t* lookup, const uint16_t* weights, float* topk_values,
                           int32_t* topk_indices, int64_t batch, int64_t num_features, int64_t num_units,
                           int64_t fan_in, int k, int transposed, ffi_stream_t stream) {
+    StreamCall call_lock((hipStream_t)stream);
     if (!features || !lookup || !weights || !topk_values || !topk_indices) return FFI_ERR_NULL_POINTER;
     Dims d;
     FFI_TRY(check_dims(batch, num_features, num_units, fan_in, transposed, &d));
@@ -231,6 +239,7 @@ int ffi_forward_topk_bf16(const uint16_t* features, const int32_t* lookup, const
 
 int ffi_topk_f32(const float* scores, int64_t batch, int64_t num_units, int k, float* topk_values, int32_t* topk_indices,
                  ffi_stream_t stream) {
+    StreamCall call_lock((hipStream_t)stream);
     if (!scores || !topk_values || !topk_indices) return FFI_ERR_NULL_POINTER;
     if (batch <= 0 || num_units <= 0) return FFI_ERR_BAD_SHAPE;
     if (batch >= INT32_MAX || num_units >= INT32_MAX) return FFI_ERR_TOO_LARGE;
@@ -250,6 +259,7 @@ static int check_loss_args(const int64_t* label_indices, int64_t nnz, int loss_k
 int ffi_loss_grad_f32(const float* scores, const int64_t* label_indices, const float* label_values, int64_t nnz,
                       int loss_kind, float grad_scale, float* out_grad, float* loss_sum, uint32_t* nz_words, int64_t batch,
                       int64_t num_units, ffi_stream_t stream) {
+    StreamCall call_lock((hipStream_t)stream);
     if (!scores || !out_grad) return FFI_ERR_NULL_POINTER;
     FFI_TRY(check_loss_args(label_indices, nnz, loss_kind, batch, num_units));
     const LossArgs la{label_indices, label_values, (int)nnz, loss_kind, grad_scale, loss_sum, nz_words, false};
@@ -259,6 +269,7 @@ int ffi_loss_grad_f32(const float* scores, const int64_t* label_indices, const f
 int ffi_forward_topk_f32(const float* features, const int32_t* lookup, const float* weights, const float* bias, float* scores,
                          float* topk_values, int32_t* topk_indices, int64_t batch, int64_t num_features, int64_t num_units,
                          int64_t fan_in, int k, int transposed, ffi_stream_t stream) {
+    StreamCall call_lock((hipStream_t)stream);
     if (!features || !lookup || !weights || !topk_values || !topk_indices) return FFI_ERR_NULL_POINTER;
     if (k < 1 || k > 8) return FFI_ERR_BAD_ARGUMENT;
     Dims d;
@@ -272,6 +283,7 @@ int ffi_forward_loss_topk_f32(const float* features, const int32_t* lookup, cons
                               float grad_scale, float* scores, float* out_grad, float* loss_sum, uint32_t* nz_words,
                               float* topk_values, int32_t* topk_indices, int k, int64_t batch, int64_t num_features,
                               int64_t num_units, int64_t fan_in, int transposed, ffi_stream_t stream) {
+    StreamCall call_lock((hipStream_t)stream);
     if (!features || !lookup || !weights || !out_grad || !topk_values || !topk_indices) return FFI_ERR_NULL_POINTER;
     if (scores == out_grad) return FFI_ERR_BAD_ARGUMENT;
     if (k < 1 || k > 8) return FFI_ERR_BAD_ARGUMENT;
@@ -288,6 +300,7 @@ int ffi_forward_loss_topk_f32(const float* features, const int32_t* lookup, cons
 
 int ffi_threshold_metrics_f32(const float* scores, const int64_t* label_indices, const float* label_values, int64_t nnz,
                               float threshold, double* counts, int64_t batch, int64_t num_units, ffi_stream_t stream) {
+    StreamCall call_lock((hipStream_t)stream);
     if (!scores || !counts) return FFI_ERR_NULL_POINTER;
     FFI_TRY(check_loss_args(label_indices, nnz, FFI_LOSS_HINGE, batch, num_units));
     return launch_threshold_metrics(scores, label_indices, label_values, (int)nnz, threshold, (int)batch, (int)num_units, counts,
@@ -299,6 +312,7 @@ int ffi_forward_loss_f32(const float* features, const int32_t* lookup, const flo
                          float grad_scale, float* scores, float* out_grad, float* loss_sum, uint32_t* nz_words,
                          int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in, int transposed,
                          ffi_stream_t stream) {
+    StreamCall call_lock((hipStream_t)stream);
     if (!features || !lookup || !weights || !out_grad) return FFI_ERR_NULL_POINTER;
     if (scores == out_grad) return FFI_ERR_BAD_ARGUMENT;
     Dims d;
@@ -315,6 +329,7 @@ int ffi_backward_sparse_f32(const float* features, const int32_t* lookup, const 
                             const uint32_t* nz_words, int flags, float max_density, float* feature_grad, float* weight_grad,
                             float* bias_grad, int* sparse_path_taken, int64_t batch, int64_t num_features,
                             int64_t num_units, int64_t fan_in, int transposed, ffi_stream_t stream) {
+    StreamCall call_lock((hipStream_t)stream);
     if (!features || !lookup || !weights || !out_grad) return FFI_ERR_NULL_POINTER;
     if (!feature_grad && !weight_grad) return FFI_ERR_NULL_POINTER;
     if (bias_grad && !weight_grad) return FFI_ERR_NULL_POINTER;
@@ -347,6 +362,7 @@ int ffi_backward_sparse_f32(const float* features, const int32_t* lookup, const 
 
 int ffi_adam_step_f32(float* variable, float* m, float* v, const float* gradient, int64_t count, float learning_rate,
                       float beta_1, float beta_2, float epsilon, int64_t step, ffi_stream_t stream) {
+    StreamCall call_lock((hipStream_t)stream);
     if (!variable || !m || !v || !gradient) return FFI_ERR_NULL_POINTER;
     if (count <= 0) return FFI_ERR_BAD_SHAPE;
     if (step < 1) return FFI_ERR_BAD_ARGUMENT;
@@ -360,6 +376,7 @@ int ffi_backward_sparse_adam_f32(const float* features, const int32_t* lookup, f
                                  float learning_rate, float beta_1, float beta_2, float epsilon, int64_t step,
                                  int* sparse_path_taken, int64_t batch, int64_t num_features, int64_t num_units,
                                  int64_t fan_in, int transposed, ffi_stream_t stream) {
+    StreamCall call_lock((hipStream_t)stream);
     if (!features || !lookup || !weights || !out_grad || !weight_m || !weight_v) return FFI_ERR_NULL_POINTER;
     if (bias && (!bias_m || !bias_v)) return FFI_ERR_NULL_POINTER;
     const bool grad_is_partial = (flags & FFI_SPARSE_GRAD_IS_PARTIAL) != 0;
@@ -410,6 +427,7 @@ int ffi_backward_sparse_adam_f32(const float* features, const int32_t* lookup, f
 }
 
 int ffi_select_threshold_f32(const float* weights, int64_t count, int64_t k, float* threshold, ffi_stream_t stream) {
+    StreamCall call_lock((hipStream_t)stream);
     if (!weights || !threshold) return FFI_ERR_NULL_POINTER;
     if (count <= 0) return FFI_ERR_BAD_SHAPE;
     if (k < 0 || k > count) return FFI_ERR_BAD_ARGUMENT;
@@ -418,6 +436,7 @@ int ffi_select_threshold_f32(const float* weights, int64_t count, int64_t k, flo
 
 int ffi_rewire_f32(int32_t* lookup, const float* weights, float* const* arrays, int n_arrays, int64_t count,
                    int64_t num_features, const float* threshold, uint64_t seed, int64_t* rewired_count, ffi_stream_t stream) {
+    StreamCall call_lock((hipStream_t)stream);
     if (!lookup || !weights || !threshold || (n_arrays > 0 && !arrays)) return FFI_ERR_NULL_POINTER;
     if (n_arrays < 0 || n_arrays > 4) return FFI_ERR_BAD_ARGUMENT;
     for (int i = 0; i < n_arrays; ++i)
@@ -430,6 +449,7 @@ int ffi_rewire_f32(int32_t* lookup, const float* weights, float* const* arrays, 
 
 int ffi_plan_create(const int32_t* lookup, int64_t num_units, int64_t fan_in, int64_t num_features,
                     int64_t batch_hint, ffi_stream_t stream, ffi_plan** plan) {
+    StreamCall call_lock((hipStream_t)stream);
     if (!lookup || !plan) return FFI_ERR_NULL_POINTER;
     *plan = nullptr;
     Dims d;
@@ -443,6 +463,7 @@ int ffi_plan_create(const int32_t* lookup, int64_t num_units, int64_t fan_in, in
 }
 
 int ffi_plan_refresh(ffi_plan* plan, const int32_t* lookup, ffi_stream_t stream) {
+    StreamCall call_lock((hipStream_t)stream);
     if (!plan || !lookup) return FFI_ERR_NULL_POINTER;
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess) return FFI_ERR_NO_DEVICE;
@@ -459,6 +480,7 @@ int ffi_plan_destroy(ffi_plan* plan) {
 
 int ffi_input_grad_planned_f32(const ffi_plan* plan, const float* weights, const float* out_grad,
                                float* feature_grad, int64_t batch, int transposed, ffi_stream_t stream) {
+    StreamCall call_lock((hipStream_t)stream);
     if (!plan || !weights || !out_grad || !feature_grad) return FFI_ERR_NULL_POINTER;
     if (batch <= 0) return FFI_ERR_BAD_SHAPE;
     if (batch >= INT32_MAX) return FFI_ERR_TOO_LARGE;
@@ -471,6 +493,7 @@ int ffi_input_grad_planned_f32(const ffi_plan* plan, const float* weights, const
 int ffi_weight_grad_planned_f32(const ffi_plan* plan, const float* features, const int32_t* lookup,
                                 const float* out_grad, float* weight_grad, int64_t batch, int transposed,
                                 ffi_stream_t stream) {
+    StreamCall call_lock((hipStream_t)stream);
     if (!plan || !features || !lookup || !out_grad || !weight_grad) return FFI_ERR_NULL_POINTER;
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess) return FFI_ERR_NO_DEVICE;
@@ -482,6 +505,7 @@ int ffi_weight_grad_planned_f32(const ffi_plan* plan, const float* features, con
 
 int ffi_arrange_connections_f32(int32_t* lookup, float* const* arrays, int n_arrays, int64_t num_units, int64_t fan_in,
                                 ffi_stream_t stream) {
+    StreamCall call_lock((hipStream_t)stream);
     if (!lookup || (n_arrays > 0 && !arrays)) return FFI_ERR_NULL_POINTER;
     if (n_arrays < 0 || n_arrays > 4) return FFI_ERR_BAD_ARGUMENT;
     for (int i = 0; i < n_arrays; ++i)
@@ -522,6 +546,7 @@ size_t ffi_cache_bytes(void) {
 
 int ffi_check_lookup(const int32_t* lookup, int64_t num_units, int64_t fan_in, int64_t num_features,
                      ffi_stream_t stream) {
+    StreamCall call_lock((hipStream_t)stream);
     if (!lookup) return FFI_ERR_NULL_POINTER;
     Dims d;
     FFI_TRY(check_dims(1, num_features, num_units, fan_in, 0, &d));

@@ -36,6 +36,20 @@ int hip_fail(hipError_t e);
         if (s__ != FFI_OK) return s__; \
     } while (0)
 
+// Held by every entry point that enqueues work, from its first launch to its last: calls on one stream share that
+// stream's workspaces, so the kernels of one call must not be interleaved with those of another call made from a
+// second thread on the same stream (TensorFlow enters an op's Compute from several threads at once).  Calls on
+// different streams do not wait for each other.  Recursive: an entry point may be built from others.
+class StreamCall {
+public:
+    explicit StreamCall(hipStream_t s);
+    ~StreamCall();
+    StreamCall(const StreamCall&) = delete;
+    StreamCall& operator=(const StreamCall&) = delete;
+private:
+    void* mutex_;
+};
+
 // Library-owned device scratch, one buffer per (device, stream, slot), grown on demand and kept.
 // Work that uses a buffer is ordered by the stream it belongs to.
 enum WorkspaceSlot { kWsFeaturesT = 0, kWsPartials = 1, kWsSlots = 2, kWsLoss = 3, kWsNonzero = 4, kWsGradients = 5, kWsRewire = 6, kWsTopk = 7, kWsScores = 8 };

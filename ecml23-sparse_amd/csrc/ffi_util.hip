@@ -3,6 +3,7 @@
 #include "ffi_lds_tile.h"
 
 #include <algorithm>
+#include <deque>
 #include <mutex>
 #include <vector>
 
@@ -18,6 +19,15 @@ struct WsEntry {
 };
 std::mutex g_ws_mutex;
 std::vector<WsEntry> g_ws;
+
+struct StreamMutex {
+    int device;
+    hipStream_t stream;
+    std::recursive_mutex mutex;
+    StreamMutex(int d, hipStream_t s) : device(d), stream(s) {}
+};
+std::mutex g_stream_mutexes_guard;
+std::deque<StreamMutex> g_stream_mutexes;      // a deque: entries are never moved or removed
 
 constexpr int kTrTile = 32;
 
@@ -39,6 +49,27 @@ __global__ __launch_bounds__(kTrTile * 8) void transpose_kernel(const float* __r
 }
 
 }  // namespace
+
+StreamCall::StreamCall(hipStream_t s) : mutex_(nullptr) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return; }   // the call itself will report the missing device
+    std::recursive_mutex* m = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g_stream_mutexes_guard);
+        for (StreamMutex& e : g_stream_mutexes)
+            if (e.device == dev && e.stream == s) m = &e.mutex;
+        if (!m) {
+            g_stream_mutexes.emplace_back(dev, s);
+            m = &g_stream_mutexes.back().mutex;
+        }
+    }
+    m->lock();
+    mutex_ = m;
+}
+
+StreamCall::~StreamCall() {
+    if (mutex_) static_cast<std::recursive_mutex*>(mutex_)->unlock();
+}
 
 int device_cu_count() {
     static int cached[64] = {0};

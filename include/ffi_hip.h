@@ -19,8 +19,11 @@
  *   - every function returns FFI_OK (0) or a negative ffi_status instead of aborting, where the
  *     reference fail-fasts through gsl_Expects (forward.cu:19-28, backward.cu:27-40):
  *     null pointers, any dimension <= 0 or > INT32_MAX, num_units*fan_in > INT32_MAX.
- *   - the library is thread-safe; calls that share a plan or the internal plan cache serialise.  Calls that
- *     use the same stream share that stream's internal workspaces: issue them from one thread at a time.
+ *   - the library is thread-safe, as an op kernel that TensorFlow enters from several threads at once has to be
+ *     (the reference's kernels are stateless, register.cpp:18-72): calls that share a plan or the internal plan
+ *     cache serialise, and calls on the same stream serialise for the time it takes to enqueue their work (they
+ *     share that stream's internal workspaces; the stream then runs them one after the other).  Calls on different
+ *     streams do not wait for each other.
  */
 #ifndef FFI_HIP_H
 #define FFI_HIP_H

@@ -414,3 +414,44 @@ def test_other_benchmark_configs_full_size_properties(ffi, name):
     part = (gx.double() - gx2.double()).cpu().numpy()
     o_part = oracle.input_grad(xs, ls, ws, gs, transposed=True)
     assert np.abs(part - o_part).max() <= 1e-4 * np.abs(gx.cpu().numpy()).max()
+
+
+def test_calls_from_two_threads_on_one_stream(ffi):
+    # TensorFlow enters an op's Compute from several threads; both calls here use the stream's transpose workspace
+    # ([B,N] features) and the plan cache (backward).  Each thread checks every result of its own inputs.
+    import threading
+    B, N, L, K = 64, 200, 6000, 16
+    lib = ffi._lib.lib()
+    cases = []
+    for seed in (1, 2):
+        x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=100 + seed)
+        ref_out = oracle.forward(x, lookup, w)
+        ref_gx, ref_gw = oracle.backward(x, lookup, w, g)
+        cases.append((dev(x), dev(lookup), dev(w), dev(g), ref_out, ref_gx, ref_gw))
+    s = stream()
+    errors = []
+
+    def worker(case):
+        dx, dl, dw, dg, ref_out, ref_gx, ref_gw = case
+        out = torch.empty((B, L), device="cuda")
+        gx = torch.empty((B, N), device="cuda")
+        gw = torch.empty((L, K), device="cuda")
+        try:
+            for _ in range(40):
+                ffi._lib.check(lib.ffi_forward_f32(dx.data_ptr(), dl.data_ptr(), dw.data_ptr(), out.data_ptr(), B, N, L, K, 0, s))
+                ffi._lib.check(lib.ffi_backward_f32(dx.data_ptr(), dl.data_ptr(), dw.data_ptr(), dg.data_ptr(), gx.data_ptr(),
+                                                    gw.data_ptr(), B, N, L, K, 0, s))
+                torch.cuda.synchronize()
+                e = (rel_err(out.cpu().numpy(), ref_out), rel_err(gx.cpu().numpy(), ref_gx), rel_err(gw.cpu().numpy(), ref_gw))
+                if not (e[0] <= FWD_RTOL and e[1] <= GRAD_RTOL and e[2] <= GRAD_RTOL):
+                    errors.append(e)
+                    return
+        except Exception as exc:  # noqa: BLE001
+            errors.append(exc)
+
+    threads = [threading.Thread(target=worker, args=(c,)) for c in cases]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
