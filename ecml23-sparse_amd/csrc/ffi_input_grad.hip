@@ -238,7 +238,17 @@ __global__ __launch_bounds__(256) void igrad_reduce_kernel(const float* __restri
     const int n = blockIdx.y;
     if (b >= B) return;
     float v = 0.f;
-    for (int r = 0; r < streams; ++r) v += partial[((size_t)r * nthreads + n) * bpad + b];
+    const size_t step = (size_t)nthreads * bpad;
+    const float* p = partial + (size_t)n * bpad + b;
+    int r = 0;
+    for (; r + 8 <= streams; r += 8) {                 // eight loads in flight, added in ascending order
+        float t[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) t[q] = p[(size_t)(r + q) * step];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) v += t[q];
+    }
+    for (; r < streams; ++r) v += p[(size_t)r * step];
     if (TP) gx[(size_t)n * B + b] = v; else gx[(size_t)b * N + n] = v;
 }
 
