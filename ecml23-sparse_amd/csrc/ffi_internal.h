@@ -66,7 +66,8 @@ int launch_forward_topk_bf16(const unsigned short* features, const int32_t* idx,
 int launch_topk_f32(const float* scores, int B, int L, int k, float* values, int32_t* indices, hipStream_t s);
 
 // dst[c][r] = src[r][c] for a row-major [rows, cols] matrix.
-int launch_transpose(const float* src, float* dst, int rows, int cols, hipStream_t s);
+// dst[c * dst_ld + r] = src[r * src_ld + c] for r < rows, c < cols (leading dimensions default to the dense ones)
+int launch_transpose(const float* src, float* dst, int rows, int cols, hipStream_t s, int src_ld = 0, int dst_ld = 0);
 
 // ---- launchers (each validates nothing; callers pass validated Dims) ---------------------------
 // bias ([L], added to every row of out) and bias_grad ([L], column sums of g) may be null

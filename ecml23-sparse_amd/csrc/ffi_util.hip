@@ -33,18 +33,19 @@ constexpr int kTrTile = 32;
 
 // 32x32 tiles through LDS (padded), coalesced on both sides.
 __global__ __launch_bounds__(kTrTile * 8) void transpose_kernel(const float* __restrict__ src,
-                                                                 float* __restrict__ dst, int rows, int cols) {
+                                                                 float* __restrict__ dst, int rows, int cols, int src_ld,
+                                                                 int dst_ld) {
     __shared__ float tile[kTrTile][kTrTile + 1];
     const int c0 = blockIdx.x * kTrTile, r0 = blockIdx.y * kTrTile;
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
     for (int i = ty; i < kTrTile; i += 8) {
         const int r = r0 + i, c = c0 + tx;
-        tile[i][tx] = (r < rows && c < cols) ? src[(size_t)r * cols + c] : 0.f;
+        tile[i][tx] = (r < rows && c < cols) ? src[(size_t)r * src_ld + c] : 0.f;
     }
     __syncthreads();
     for (int i = ty; i < kTrTile; i += 8) {
         const int c = c0 + i, r = r0 + tx;
-        if (r < rows && c < cols) dst[(size_t)c * rows + r] = tile[tx][i];
+        if (r < rows && c < cols) dst[(size_t)c * dst_ld + r] = tile[tx][i];
     }
 }
 
@@ -130,10 +131,11 @@ size_t workspace_bytes(int device) {
     return total;
 }
 
-int launch_transpose(const float* src, float* dst, int rows, int cols, hipStream_t s) {
+int launch_transpose(const float* src, float* dst, int rows, int cols, hipStream_t s, int src_ld, int dst_ld) {
     dim3 grid((cols + kTrTile - 1) / kTrTile, (rows + kTrTile - 1) / kTrTile);
     if (grid.y > 65535u) return FFI_ERR_TOO_LARGE;
-    hipLaunchKernelGGL(transpose_kernel, grid, dim3(kTrTile * 8), 0, s, src, dst, rows, cols);
+    hipLaunchKernelGGL(transpose_kernel, grid, dim3(kTrTile * 8), 0, s, src, dst, rows, cols, src_ld > 0 ? src_ld : cols,
+                       dst_ld > 0 ? dst_ld : rows);
     FFI_HIP_TRY(hipGetLastError());
     return FFI_OK;
 }

@@ -18,6 +18,7 @@ namespace {
 constexpr int kWideThreads = 256;   // 4 wavefronts per workgroup
 constexpr int kWideLabels = 64;     // labels per workgroup: 16 per wavefront
 constexpr int kWideBatch = 128;     // batch entries per pass: each lane owns b and b+64
+constexpr int kWideInflight = 8;      // connections whose gathers a wavefront has in flight
 constexpr int kWideStride = kWideBatch + 1;   // LDS row stride in floats (odd: conflict-free both ways)
 
 __device__ __forceinline__ float wave_sum(float v) {
@@ -30,18 +31,20 @@ __device__ __forceinline__ float wave_sum(float v) {
 // grid (label blocks, batch passes).  A wavefront walks 16 labels one after the other; per
 // connection it loads one 512-byte piece of row idx[j,k] of xT and does two multiply-adds per lane.
 // Results go through LDS so that out is written in 256-byte rows.
+// TWO == false (batch <= 64): lanes own one batch entry each, the loads and multiply-adds of the second half are left out.
+template <bool TWO>
 __global__ __launch_bounds__(kWideThreads) void fwd_wide_kernel(const float* __restrict__ xT,
                                                                 const int32_t* __restrict__ idx,
                                                                 const float* __restrict__ w,
                                                                 const float* __restrict__ bias, float* __restrict__ out,
-                                                                int B, int N, int L, int K) {
+                                                                int B, int N, int L, int K, int ldb) {
     __shared__ float tile[kWideLabels * kWideStride];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j0 = blockIdx.x * kWideLabels;
     const int bc0 = blockIdx.y * kWideBatch;
-    const buffer_rsrc xr = make_rsrc(xT, (size_t)N * (size_t)B * sizeof(float));
+    const buffer_rsrc xr = make_rsrc(xT, (size_t)N * (size_t)ldb * sizeof(float));
     const unsigned lane_off0 = (unsigned)(bc0 + lane) * 4u, lane_off1 = lane_off0 + 256u;
-    const unsigned row_bytes = (unsigned)B * 4u;
+    const unsigned row_bytes = (unsigned)ldb * 4u;
     for (int q = 0; q < kWideLabels / 4; ++q) {
         const int jl = wave * (kWideLabels / 4) + q;
         const int j = j0 + jl;
@@ -55,23 +58,26 @@ __global__ __launch_bounds__(kWideThreads) void fwd_wide_kernel(const float* __r
                 const unsigned iv = (lane < kn) ? (unsigned)irow[k0 + lane] : 0u;
                 const float wv = (lane < kn) ? wrow[k0 + lane] : 0.f;
                 int k = 0;
-                for (; k + 4 <= kn; k += 4) {
-                    float x0[4], x1[4], ws[4];
+                for (; k + kWideInflight <= kn; k += kWideInflight) {
+                    float x0[kWideInflight], x1[kWideInflight], ws[kWideInflight];
 #pragma unroll
-                    for (int u = 0; u < 4; ++u) {
+                    for (int u = 0; u < kWideInflight; ++u) {
                         const unsigned n = (unsigned)__builtin_amdgcn_readlane((int)iv, k + u);
                         ws[u] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wv), k + u));
                         x0[u] = buffer_load_f32(xr, lane_off0, n * row_bytes);
-                        x1[u] = buffer_load_f32(xr, lane_off1, n * row_bytes);
+                        x1[u] = TWO ? buffer_load_f32(xr, lane_off1, n * row_bytes) : 0.f;
                     }
 #pragma unroll
-                    for (int u = 0; u < 4; ++u) { acc0 = fmaf(ws[u], x0[u], acc0); acc1 = fmaf(ws[u], x1[u], acc1); }
+                    for (int u = 0; u < kWideInflight; ++u) {
+                        acc0 = fmaf(ws[u], x0[u], acc0);
+                        if (TWO) acc1 = fmaf(ws[u], x1[u], acc1);
+                    }
                 }
                 for (; k < kn; ++k) {
                     const unsigned n = (unsigned)__builtin_amdgcn_readlane((int)iv, k);
                     const float wk = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wv), k));
                     acc0 = fmaf(wk, buffer_load_f32(xr, lane_off0, n * row_bytes), acc0);
-                    acc1 = fmaf(wk, buffer_load_f32(xr, lane_off1, n * row_bytes), acc1);
+                    if (TWO) acc1 = fmaf(wk, buffer_load_f32(xr, lane_off1, n * row_bytes), acc1);
                 }
             }
         }
@@ -84,7 +90,7 @@ __global__ __launch_bounds__(kWideThreads) void fwd_wide_kernel(const float* __r
     if (j0 + jl < L) {
         const bool has_bias = bias != nullptr;
         const float bj = has_bias ? bias[j0 + jl] : 0.f;
-        for (int bb = threadIdx.x >> 6; bb < kWideBatch; bb += kWideThreads / 64) {
+        for (int bb = threadIdx.x >> 6; bb < (TWO ? kWideBatch : kWideBatch / 2); bb += kWideThreads / 64) {
             const int b = bc0 + bb;
             const float v = tile[jl * kWideStride + bb];
             if (b < B) out[(size_t)b * L + j0 + jl] = has_bias ? v + bj : v;
@@ -97,11 +103,12 @@ __global__ __launch_bounds__(kWideThreads) void fwd_wide_kernel(const float* __r
 // along labels), then every wavefront handles 16 labels: per connection one 512-byte piece of the
 // xT row times the label's out_grad, summed over the lanes, accumulated over the batch passes in
 // LDS by a single lane (fixed order: reproducible).
+template <bool TWO>
 __global__ __launch_bounds__(kWideThreads) void wgrad_wide_kernel(const float* __restrict__ xT,
                                                                   const int32_t* __restrict__ idx,
                                                                   const float* __restrict__ g, float* __restrict__ gw,
                                                                   float* __restrict__ bias_grad, int B, int N, int L,
-                                                                  int K) {
+                                                                  int K, int ldb) {
     extern __shared__ float smem[];
     float* gt = smem;                                   // [64 labels][129]
     float* res = smem + kWideLabels * kWideStride;      // [64 labels][K]
@@ -109,15 +116,15 @@ __global__ __launch_bounds__(kWideThreads) void wgrad_wide_kernel(const float* _
     if (threadIdx.x < kWideLabels) bres[threadIdx.x] = 0.f;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j0 = blockIdx.x * kWideLabels;
-    const buffer_rsrc xr = make_rsrc(xT, (size_t)N * (size_t)B * sizeof(float));
-    const unsigned row_bytes = (unsigned)B * 4u;
+    const buffer_rsrc xr = make_rsrc(xT, (size_t)N * (size_t)ldb * sizeof(float));
+    const unsigned row_bytes = (unsigned)ldb * 4u;
     for (int t = threadIdx.x; t < kWideLabels * K; t += kWideThreads) res[t] = 0.f;
     for (int bc0 = 0; bc0 < B; bc0 += kWideBatch) {
         __syncthreads();
         {
             const int jl = threadIdx.x & 63;
             const bool in = j0 + jl < L;
-            for (int bb = threadIdx.x >> 6; bb < kWideBatch; bb += kWideThreads / 64) {
+            for (int bb = threadIdx.x >> 6; bb < (TWO ? kWideBatch : kWideBatch / 2); bb += kWideThreads / 64) {
                 const int b = bc0 + bb;
                 gt[jl * kWideStride + bb] = (in && b < B) ? g[(size_t)b * L + j0 + jl] : 0.f;
             }
@@ -131,7 +138,7 @@ __global__ __launch_bounds__(kWideThreads) void wgrad_wide_kernel(const float* _
             const int jl = wave * (kWideLabels / 4) + q;
             const int j = j0 + jl;
             if (j >= L) break;                                  // wave-uniform
-            const float g0 = gt[jl * kWideStride + lane], g1 = gt[jl * kWideStride + 64 + lane];
+            const float g0 = gt[jl * kWideStride + lane], g1 = TWO ? gt[jl * kWideStride + 64 + lane] : 0.f;
             if (bias_grad != nullptr) {                         // wave-uniform
                 const float gs = wave_sum(g0 + g1);
                 if (lane == 0) bres[jl] += gs;
@@ -142,17 +149,17 @@ __global__ __launch_bounds__(kWideThreads) void wgrad_wide_kernel(const float* _
                 const unsigned iv = (lane < kn) ? (unsigned)irow[k0 + lane] : 0u;
                 float mine = 0.f;                               // lane k collects connection k0+k
                 int k = 0;
-                for (; k + 4 <= kn; k += 4) {
-                    float x0[4], x1[4];
+                for (; k + kWideInflight <= kn; k += kWideInflight) {
+                    float x0[kWideInflight], x1[kWideInflight];
 #pragma unroll
-                    for (int u = 0; u < 4; ++u) {
+                    for (int u = 0; u < kWideInflight; ++u) {
                         const unsigned n = (unsigned)__builtin_amdgcn_readlane((int)iv, k + u);
                         x0[u] = buffer_load_f32(xr, lane_off0, n * row_bytes);
-                        x1[u] = buffer_load_f32(xr, lane_off1, n * row_bytes);
+                        x1[u] = TWO ? buffer_load_f32(xr, lane_off1, n * row_bytes) : 0.f;
                     }
 #pragma unroll
-                    for (int u = 0; u < 4; ++u) {
-                        const float p = fmaf(in1 ? x1[u] : 0.f, g1, (in0 ? x0[u] : 0.f) * g0);
+                    for (int u = 0; u < kWideInflight; ++u) {
+                        const float p = TWO ? fmaf(in1 ? x1[u] : 0.f, g1, (in0 ? x0[u] : 0.f) * g0) : (in0 ? x0[u] : 0.f) * g0;
                         const float s = wave_sum(p);
                         if (lane == k + u) mine = s;
                     }
@@ -160,8 +167,8 @@ __global__ __launch_bounds__(kWideThreads) void wgrad_wide_kernel(const float* _
                 for (; k < kn; ++k) {
                     const unsigned n = (unsigned)__builtin_amdgcn_readlane((int)iv, k);
                     const float a = buffer_load_f32(xr, lane_off0, n * row_bytes);
-                    const float b = buffer_load_f32(xr, lane_off1, n * row_bytes);
-                    const float s = wave_sum(fmaf(in1 ? b : 0.f, g1, (in0 ? a : 0.f) * g0));
+                    const float b = TWO ? buffer_load_f32(xr, lane_off1, n * row_bytes) : 0.f;
+                    const float s = wave_sum(TWO ? fmaf(in1 ? b : 0.f, g1, (in0 ? a : 0.f) * g0) : (in0 ? a : 0.f) * g0);
                     if (lane == k) mine = s;
                 }
                 if (lane < kn) res[jl * K + k0 + lane] += mine;
@@ -182,17 +189,18 @@ __global__ __launch_bounds__(kWideThreads) void wgrad_wide_kernel(const float* _
 // per lane, then handed out as scalars), gathering one 512-byte piece of row j of gT per
 // connection.  No atomics, fixed order: reproducible.  Label blocks bound the part of gT that is
 // live at any time, so the gathers are served by the last-level cache.
+template <bool TWO>
 __global__ __launch_bounds__(kWideThreads) void igrad_wide_kernel(const int32_t* __restrict__ perm,
                                                                   const int32_t* __restrict__ col_ptr,
                                                                   const float* __restrict__ w,
                                                                   const float* __restrict__ gT, float* __restrict__ gxT,
                                                                   int B, int N, int L, int K, int nblocks,
-                                                                  unsigned kdiv_mul, unsigned kdiv_shift) {
+                                                                  unsigned kdiv_mul, unsigned kdiv_shift, int ldb) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = blockIdx.x * (kWideThreads / 64) + wave;
     if (n >= N) return;                                         // wave-uniform
     const int bc0 = blockIdx.y * kWideBatch;
-    const buffer_rsrc gr = make_rsrc(gT, (size_t)L * (size_t)B * sizeof(float));
+    const buffer_rsrc gr = make_rsrc(gT, (size_t)L * (size_t)ldb * sizeof(float));
     const unsigned lane_off0 = (unsigned)(bc0 + lane) * 4u, lane_off1 = lane_off0 + 256u;
     float acc0 = 0.f, acc1 = 0.f;
     for (int blk = 0; blk < nblocks; ++blk) {
@@ -205,29 +213,32 @@ __global__ __launch_bounds__(kWideThreads) void igrad_wide_kernel(const int32_t*
             // label of the connection: p / K by multiply-high and shift (exact for p < 2^31)
             const unsigned jv = kdiv_mul ? (__umulhi((unsigned)p, kdiv_mul) >> kdiv_shift) : (unsigned)p;
             int i = 0;
-            for (; i + 4 <= cnt; i += 4) {
-                float a[4], b[4], ws[4];
+            for (; i + kWideInflight <= cnt; i += kWideInflight) {
+                float a[kWideInflight], b[kWideInflight], ws[kWideInflight];
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
+                for (int u = 0; u < kWideInflight; ++u) {
                     const unsigned j = (unsigned)__builtin_amdgcn_readlane((int)jv, i + u);
                     ws[u] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wv), i + u));
-                    // rows of gT are B*4 bytes; L*B*4 < 2^32 is checked by the launcher
-                    a[u] = buffer_load_f32(gr, lane_off0, j * (unsigned)B * 4u);
-                    b[u] = buffer_load_f32(gr, lane_off1, j * (unsigned)B * 4u);
+                    // rows of gT are ldb*4 bytes; L*ldb*4 < 2^32 is checked by the launcher
+                    a[u] = buffer_load_f32(gr, lane_off0, j * (unsigned)ldb * 4u);
+                    b[u] = TWO ? buffer_load_f32(gr, lane_off1, j * (unsigned)ldb * 4u) : 0.f;
                 }
 #pragma unroll
-                for (int u = 0; u < 4; ++u) { acc0 = fmaf(ws[u], a[u], acc0); acc1 = fmaf(ws[u], b[u], acc1); }
+                for (int u = 0; u < kWideInflight; ++u) {
+                    acc0 = fmaf(ws[u], a[u], acc0);
+                    if (TWO) acc1 = fmaf(ws[u], b[u], acc1);
+                }
             }
             for (; i < cnt; ++i) {
                 const unsigned j = (unsigned)__builtin_amdgcn_readlane((int)jv, i);
                 const float wk = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wv), i));
-                acc0 = fmaf(wk, buffer_load_f32(gr, lane_off0, j * (unsigned)B * 4u), acc0);
-                acc1 = fmaf(wk, buffer_load_f32(gr, lane_off1, j * (unsigned)B * 4u), acc1);
+                acc0 = fmaf(wk, buffer_load_f32(gr, lane_off0, j * (unsigned)ldb * 4u), acc0);
+                if (TWO) acc1 = fmaf(wk, buffer_load_f32(gr, lane_off1, j * (unsigned)ldb * 4u), acc1);
             }
         }
     }
     if (bc0 + lane < B) gxT[(size_t)n * B + bc0 + lane] = acc0;
-    if (bc0 + 64 + lane < B) gxT[(size_t)n * B + bc0 + 64 + lane] = acc1;
+    if (TWO && bc0 + 64 + lane < B) gxT[(size_t)n * B + bc0 + 64 + lane] = acc1;
 }
 
 // floor(p / d) for 0 <= p < 2^31 as (p * mul) >> (32 + shift)
@@ -242,21 +253,43 @@ void magic_divisor(unsigned d, unsigned* mul, unsigned* shift) {
 
 }  // namespace
 
-bool wide_offsets_fit(long long rows, long long B) { return rows * B * 4 < (1ll << 32); }
+// Row stride (in floats) of the library's own [rows][batch] copies: a multiple of 32, so that rows start on 128-byte
+// lines and a gathered row piece touches as few lines as it can.
+int wide_row_stride(int B) { return (B + 31) / 32 * 32; }
+
+bool wide_offsets_fit(long long rows, long long B) { return rows * wide_row_stride((int)B) * 4 < (1ll << 32); }
+
+namespace {
+
+// xT[N][ldb] for the wide kernels: the caller's [N,B] buffer itself when its rows are aligned already, else a copy.
+int wide_features(const float* x, const Dims& d, hipStream_t s, const float** xT, int* ldb) {
+    const int ld = wide_row_stride(d.B);
+    if (d.tp && ld == d.B) { *xT = x; *ldb = d.B; return FFI_OK; }
+    float* ws = nullptr;
+    FFI_TRY(workspace_get(s, kWsFeaturesT, (size_t)d.N * ld * sizeof(float), (void**)&ws));
+    if (d.tp) {
+        FFI_HIP_TRY(hipMemcpy2DAsync(ws, (size_t)ld * sizeof(float), x, (size_t)d.B * sizeof(float), (size_t)d.B * sizeof(float),
+                                     (size_t)d.N, hipMemcpyDeviceToDevice, s));
+    } else {
+        FFI_TRY(launch_transpose(x, ws, d.B, d.N, s, d.N, ld));     // [B,N] -> [N,ld]
+    }
+    *xT = ws;
+    *ldb = ld;
+    return FFI_OK;
+}
+
+}  // namespace
 
 int launch_forward_wide(const float* x, const int32_t* idx, const float* w, const float* bias, float* out, const Dims& d,
                         hipStream_t s) {
     if (!wide_offsets_fit(d.N, d.B)) return FFI_ERR_TOO_LARGE;
-    const float* xT = x;
-    if (!d.tp) {
-        float* ws = nullptr;
-        FFI_TRY(workspace_get(s, kWsFeaturesT, (size_t)d.N * d.B * sizeof(float), (void**)&ws));
-        FFI_TRY(launch_transpose(x, ws, d.B, d.N, s));
-        xT = ws;
-    }
+    const float* xT = nullptr;
+    int ldb = 0;
+    FFI_TRY(wide_features(x, d, s, &xT, &ldb));
     dim3 grid((d.L + kWideLabels - 1) / kWideLabels, (d.B + kWideBatch - 1) / kWideBatch);
     if (grid.y > 65535u) return FFI_ERR_TOO_LARGE;
-    hipLaunchKernelGGL(fwd_wide_kernel, grid, dim3(kWideThreads), 0, s, xT, idx, w, bias, out, d.B, d.N, d.L, d.K);
+    if (d.B > 64) hipLaunchKernelGGL(fwd_wide_kernel<true>, grid, dim3(kWideThreads), 0, s, xT, idx, w, bias, out, d.B, d.N, d.L, d.K, ldb);
+    else hipLaunchKernelGGL(fwd_wide_kernel<false>, grid, dim3(kWideThreads), 0, s, xT, idx, w, bias, out, d.B, d.N, d.L, d.K, ldb);
     FFI_HIP_TRY(hipGetLastError());
     return FFI_OK;
 }
@@ -266,33 +299,39 @@ int launch_weight_grad_wide(const float* x, const int32_t* idx, const float* g, 
     if (!wide_offsets_fit(d.N, d.B)) return FFI_ERR_TOO_LARGE;
     const size_t lds = ((size_t)kWideLabels * kWideStride + (size_t)kWideLabels * d.K + kWideLabels) * sizeof(float);
     if (lds > 150 * 1024) return FFI_ERR_TOO_LARGE;               // fan-in beyond ~450
-    const float* xT = x;
-    if (!d.tp) {
-        float* ws = nullptr;
-        FFI_TRY(workspace_get(s, kWsFeaturesT, (size_t)d.N * d.B * sizeof(float), (void**)&ws));
-        FFI_TRY(launch_transpose(x, ws, d.B, d.N, s));
-        xT = ws;
+    const float* xT = nullptr;
+    int ldb = 0;
+    FFI_TRY(wide_features(x, d, s, &xT, &ldb));
+    const dim3 grid((d.L + kWideLabels - 1) / kWideLabels);
+    if (d.B > 64) {
+        FFI_HIP_TRY(hipFuncSetAttribute((const void*)wgrad_wide_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        hipLaunchKernelGGL(wgrad_wide_kernel<true>, grid, dim3(kWideThreads), lds, s, xT, idx, g, gw, bias_grad, d.B, d.N, d.L, d.K, ldb);
+    } else {
+        FFI_HIP_TRY(hipFuncSetAttribute((const void*)wgrad_wide_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        hipLaunchKernelGGL(wgrad_wide_kernel<false>, grid, dim3(kWideThreads), lds, s, xT, idx, g, gw, bias_grad, d.B, d.N, d.L, d.K, ldb);
     }
-    FFI_HIP_TRY(hipFuncSetAttribute((const void*)wgrad_wide_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(wgrad_wide_kernel, dim3((d.L + kWideLabels - 1) / kWideLabels), dim3(kWideThreads), lds, s, xT, idx,
-                       g, gw, bias_grad, d.B, d.N, d.L, d.K);
     FFI_HIP_TRY(hipGetLastError());
     return FFI_OK;
 }
 
 int launch_input_grad_wide(const ffi_plan* p, const float* w, const float* g, float* gx, int B, bool tp, hipStream_t s) {
     if (!wide_offsets_fit(p->L, B)) return FFI_ERR_TOO_LARGE;
+    const int ldb = wide_row_stride(B);
     float* gT = nullptr;
-    FFI_TRY(workspace_get(s, kWsPartials, (size_t)p->L * B * sizeof(float), (void**)&gT));
-    FFI_TRY(launch_transpose(g, gT, B, p->L, s));                 // [B,L] -> [L,B]
+    FFI_TRY(workspace_get(s, kWsPartials, (size_t)p->L * ldb * sizeof(float), (void**)&gT));
+    FFI_TRY(launch_transpose(g, gT, B, p->L, s, p->L, ldb));      // [B,L] -> [L,ldb]
     float* gxT = gx;
     if (!tp) FFI_TRY(workspace_get(s, kWsFeaturesT, (size_t)p->N * B * sizeof(float), (void**)&gxT));
     unsigned mul = 0, shift = 0;
     magic_divisor((unsigned)p->K, &mul, &shift);
     dim3 grid((p->N + kWideThreads / 64 - 1) / (kWideThreads / 64), (B + kWideBatch - 1) / kWideBatch);
     if (grid.y > 65535u) return FFI_ERR_TOO_LARGE;
-    hipLaunchKernelGGL(igrad_wide_kernel, grid, dim3(kWideThreads), 0, s, p->perm, p->col_ptr, w, gT, gxT, B, p->N, p->L,
-                       p->K, p->nblocks, mul, shift);
+    if (B > 64)
+        hipLaunchKernelGGL(igrad_wide_kernel<true>, grid, dim3(kWideThreads), 0, s, p->perm, p->col_ptr, w, gT, gxT, B, p->N, p->L,
+                           p->K, p->nblocks, mul, shift, ldb);
+    else
+        hipLaunchKernelGGL(igrad_wide_kernel<false>, grid, dim3(kWideThreads), 0, s, p->perm, p->col_ptr, w, gT, gxT, B, p->N,
+                           p->L, p->K, p->nblocks, mul, shift, ldb);
     FFI_HIP_TRY(hipGetLastError());
     if (!tp) FFI_TRY(launch_transpose(gxT, gx, p->N, B, s));      // [N,B] -> [B,N]
     return FFI_OK;

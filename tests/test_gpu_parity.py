@@ -140,7 +140,10 @@ PATH_SHAPES = [
     (33, 96, 9, 5),            # fewer labels than lanes, odd fan-in
     (64, 1100, 3000, 12),      # N > 1024: tile forward / weight-grad, global plan
     (40, 1216, 2500, 36),      # largest N that still fits the LDS tile
-    (48, 1300, 2000, 20),      # wide: generic kernels
+    (48, 1300, 2000, 20),      # wide: generic kernels, one batch entry per lane, rows padded to 128 bytes
+    (64, 1400, 700, 16),       # wide, rows already aligned: [N,B] features used in place
+    (70, 1500, 900, 9),        # wide, two batch entries per lane, the second half nearly empty
+    (200, 2000, 600, 33),      # wide, two batch passes
     (7, 64, 70000, 3),         # many tiles of a tiny column set
     (128, 512, 4100, 100),     # four register chunks per label, tail of 4
 ]
