@@ -21,6 +21,7 @@ constexpr int kBfThreads = 256;            // 4 wavefronts
 constexpr int kBfBatch = 512;              // batch entries per pass: 8 per lane
 constexpr int kBfLabels = 32;              // labels per workgroup step when scores are written out
 constexpr int kBfStride = kBfBatch + 1;
+constexpr int kBfInflight = 4;             // connections whose 16-byte gathers a wavefront has in flight
 constexpr int kTopMax = 8;                 // list length kept per sample (k <= 8)
 
 __device__ __forceinline__ float bf16_lo(unsigned u) { return __uint_as_float(u << 16); }
@@ -49,17 +50,17 @@ __device__ __forceinline__ void bf16_label_scores(const buffer_rsrc xr, unsigned
         const unsigned iv = (lane < kn) ? (unsigned)irow[k0 + lane] : 0u;
         const float wv = (lane < kn) ? bf16_lo((unsigned)wrow[k0 + lane]) : 0.f;
         int k = 0;
-        for (; k + 2 <= kn; k += 2) {
-            uint4 x[2];
-            float ws[2];
+        for (; k + kBfInflight <= kn; k += kBfInflight) {
+            uint4 x[kBfInflight];
+            float ws[kBfInflight];
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
+            for (int u = 0; u < kBfInflight; ++u) {
                 const unsigned n = (unsigned)__builtin_amdgcn_readlane((int)iv, k + u);
                 ws[u] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wv), k + u));
                 x[u] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(xr, lane_off, n * row_bytes, 0));
             }
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
+            for (int u = 0; u < kBfInflight; ++u) {
                 acc[0] = fmaf(ws[u], bf16_lo(x[u].x), acc[0]); acc[1] = fmaf(ws[u], bf16_hi(x[u].x), acc[1]);
                 acc[2] = fmaf(ws[u], bf16_lo(x[u].y), acc[2]); acc[3] = fmaf(ws[u], bf16_hi(x[u].y), acc[3]);
                 acc[4] = fmaf(ws[u], bf16_lo(x[u].z), acc[4]); acc[5] = fmaf(ws[u], bf16_hi(x[u].z), acc[5]);
