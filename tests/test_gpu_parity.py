@@ -458,3 +458,31 @@ def test_calls_from_two_threads_on_one_stream(ffi):
     for t in threads:
         t.join()
     assert not errors, errors
+
+
+def _random_shapes(count, seed):
+    rng = np.random.default_rng(seed)
+    shapes = []
+    for _ in range(count):
+        B = int(rng.choice([1, 2, 7, 31, 32, 33, 50, 64, 65, 100, 128, 200, 257]))
+        N = int(rng.choice([1, 3, 17, 64, 100, 255, 512, 768, 1024, 1025, 1216, 1217, 2000, 5000]))
+        L = int(rng.choice([1, 2, 63, 64, 65, 500, 1023, 1024, 1025, 3000, 7001]))
+        K = int(rng.choice([1, 2, 3, 4, 8, 15, 16, 31, 32, 33, 48, 64, 65, 100]))
+        shapes.append((B, N, L, K, bool(rng.integers(0, 2))))
+    return shapes
+
+
+@pytest.mark.parametrize("shape", _random_shapes(36, seed=2024), ids=lambda s: "B%d_N%d_L%d_K%d_%s" % (s[0], s[1], s[2], s[3], "tp" if s[4] else "nt"))
+def test_drawn_shapes(ffi, shape):
+    # sizes drawn around the boundaries of the kernels' regimes (batch tiles of 32, wavefronts of 64, label tiles of 1024,
+    # register chunks of 32 connections, 1216 columns for the LDS tile, 1024 for the tiled plan), either layout
+    B, N, L, K, transposed = shape
+    x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=B + 3 * N + 5 * L + 7 * K)
+    xin = np.ascontiguousarray(x.T) if transposed else x
+    print(f"case shape={shape}", flush=True)
+    out = hip_forward(ffi, xin, lookup, w, transposed)
+    gx, gw = hip_backward(ffi, xin, lookup, w, g, transposed)
+    assert rel_err(out, oracle.forward(xin, lookup, w, transposed=transposed)) <= FWD_RTOL
+    o_gx, o_gw = oracle.backward(xin, lookup, w, g, transposed=transposed)
+    assert rel_err(gw, o_gw) <= GRAD_RTOL
+    assert rel_err(gx, o_gx) <= GRAD_RTOL

@@ -273,3 +273,31 @@ def test_headline_config_full_size_training_step(ffi):
     b = float((x.double() * gx_s.double()).sum())
     c = float((w.double() * gw_s.double()).sum())
     assert abs(a - b) <= 1e-4 * abs(a) and abs(a - c) <= 1e-4 * abs(a)
+
+
+def _drawn_shapes(count, seed):
+    rng = np.random.default_rng(seed)
+    shapes = []
+    for _ in range(count):
+        B = int(rng.choice([1, 7, 31, 32, 33, 64, 65, 100, 128, 200]))
+        N = int(rng.choice([3, 64, 255, 512, 768, 1024, 1217, 3000, 4096, 4097]))
+        L = int(rng.choice([1, 63, 64, 65, 255, 256, 257, 1025, 3000, 7001, 33000]))
+        K = int(rng.choice([1, 3, 4, 15, 16, 32, 33, 64, 65, 100]))
+        shapes.append((B, N, L, K, bool(rng.integers(0, 2))))
+    return shapes
+
+
+@pytest.mark.parametrize("density", [0.003, 0.1])
+@pytest.mark.parametrize("shape", _drawn_shapes(16, seed=77), ids=lambda s: "B%d_N%d_L%d_K%d_%s" % (s[0], s[1], s[2], s[3], "tp" if s[4] else "nt"))
+def test_sparse_backward_drawn_shapes(ffi, shape, density):
+    # sizes drawn around the boundaries of the sparse kernels (blocks of 256 labels per wavefront, chunks of 32,768
+    # labels of a bit row, 4096 columns for the LDS accumulators, 32-connection register chunks), masks given
+    tp = shape[4]
+    feats, lookup, w, g = make_case(shape, density, seed=sum(shape[:4]) + 1)
+    print(f"case shape={shape} density={density}", flush=True)
+    ref_gx, ref_gw = oracle.backward(feats, lookup, w, g, transposed=tp)
+    gx, gw, gb, sparse = run(ffi, feats, lookup, w, g, tp, words=masks_of(g))
+    assert sparse
+    assert rel_err(gw, ref_gw) <= GRAD_RTOL
+    assert rel_err(gx, ref_gx) <= GRAD_RTOL
+    assert rel_err(gb, g.sum(axis=0)) <= GRAD_RTOL
