@@ -133,7 +133,12 @@ FUSED = [(128, 768, 5000, 32, True),
          (37, 300, 1001, 7, False),
          (64, 512, 2100, 64, True),
          (33, 3000, 333, 12, True),        # wide inputs: forward kernel, then the loss as a pass of its own
-         (130, 2048, 260, 72, False)]
+         (130, 2048, 260, 72, False),
+         (1, 17, 65, 3, False),            # one sample
+         (65, 1216, 1025, 33, True),       # the widest LDS tile, three batch tiles with one row in the last
+         (50, 1217, 700, 16, False),       # one column more: the wide kernels
+         (200, 64, 3000, 100, True),       # four register chunks per label
+         (31, 768, 1023, 32, False)]
 
 
 @pytest.mark.parametrize("kind", KINDS)
