@@ -43,7 +43,11 @@ __device__ __forceinline__ void fwd_lane_step(unsigned base, float wv, float (&a
 //                    (listed positions are patched afterwards), and the loss(s, 0) summed per wavefront
 //   kEpiLossGradAndScores  both: scores to `out`, gradients to `gout`
 //   kEpiNone         nothing is stored (only the top-k candidates below are wanted)
-enum FwdEpilogue { kEpiScores = 0, kEpiLossGrad = 1, kEpiLossGradAndScores = 2, kEpiNone = 3 };
+//   kEpiLossGradSkewed  kEpiLossGrad for launches that do not store gradients that are exactly zero (nearly nothing is
+//                    stored then): the accumulators stay in the lane's skewed register order (register q holds batch
+//                    entry q ^ 4 (lane & 7)), the 96 conditional moves back to natural order are left out, the few stores
+//                    address their rows per lane and only the mask's bits are put in order
+enum FwdEpilogue { kEpiScores = 0, kEpiLossGrad = 1, kEpiLossGradAndScores = 2, kEpiNone = 3, kEpiLossGradSkewed = 4 };
 
 constexpr int kTopkPark = 24;           // candidates per (workgroup, batch row) parked in LDS: 32 x 24 x 8 bytes = 6 KB
 
@@ -72,10 +76,13 @@ struct FwdLoss {
 // Scores of one label for the 32 samples of a batch tile -> scaled loss gradients (in place), the sum of the
 // losses of the first `nrows` samples, and the mask of the non-zero gradients among them.
 template <int KIND>
-__device__ __forceinline__ void loss_epilogue(float (&acc)[32], int nrows, float scale, float& loss, unsigned& mask) {
+__device__ __forceinline__ void loss_epilogue(float (&acc)[32], bool all_rows, unsigned valid_bits, float scale, float& loss,
+                                              unsigned& mask) {
+    // `all_rows` (workgroup-uniform): the batch tile is full; else bit q of `valid_bits` says whether register q belongs
+    // to a sample of the batch (rows past it count for nothing)
     float l = 0.f;
     unsigned m = 0;
-    if (nrows == 32) {
+    if (all_rows) {
 #pragma unroll
         for (int b = 0; b < 32; ++b) {
             float lb, gb;
@@ -84,13 +91,14 @@ __device__ __forceinline__ void loss_epilogue(float (&acc)[32], int nrows, float
             m |= (gb != 0.f ? 1u : 0u) << b;
             acc[b] = scale * gb;
         }
-    } else {                               // last batch tile: rows past the batch count for nothing
+    } else {
 #pragma unroll
         for (int b = 0; b < 32; ++b) {
             float lb, gb;
             cwise_loss_and_grad(KIND, acc[b], 0.f, lb, gb);
-            l += b < nrows ? lb : 0.f;
-            m |= (b < nrows && gb != 0.f ? 1u : 0u) << b;
+            const bool in = (valid_bits >> b) & 1u;
+            l += in ? lb : 0.f;
+            m |= (in && gb != 0.f ? 1u : 0u) << b;
             acc[b] = scale * gb;
         }
     }
@@ -131,6 +139,13 @@ __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* _
     buffer_rsrc grsrc = orsrc;
     if (EPI == kEpiLossGradAndScores) grsrc = make_rsrc(fl.gout + (size_t)b0 * (size_t)L, (size_t)nrows * (size_t)L * sizeof(float));
     float lsum = 0.f;
+
+    constexpr bool SKEW = EPI == kEpiLossGradSkewed;
+    constexpr bool LOSS = EPI == kEpiLossGrad || EPI == kEpiLossGradAndScores || SKEW;
+    static_assert(!(SKEW && TOPK), "the top-k tests need the natural order");
+    // registers (in the order the epilogue sees them) that belong to samples of the batch
+    const unsigned rows_valid = nrows >= kTileBatch ? 0xffffffffu : (1u << nrows) - 1u;
+    const unsigned regs_valid = SKEW ? xor_permute_bits(rows_valid, lane & 7) : rows_valid;
 
     for (int base = l_begin; base < l_end; base += kTileThreads) {
         if (base + (int)(threadIdx.x & ~63u) >= l_end) break;     // nothing left for this wavefront
@@ -179,7 +194,7 @@ __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* _
                 }
             }
         }
-        xor_permute_groups(acc, lane & 7);                 // back to natural batch order
+        if (!SKEW) xor_permute_groups(acc, lane & 7);      // back to natural batch order
         if (bias != nullptr) {                             // added after the sum, as a separate bias_add would
             const float bj = bias[jj];
 #pragma unroll
@@ -232,16 +247,27 @@ __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* _
             for (int b = 0; b < 32; ++b)
                 __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, acc[b]), orsrc, lane_off, (unsigned)b * stride, 0);
         }
-        if (EPI == kEpiLossGrad || EPI == kEpiLossGradAndScores) {
+        if (LOSS) {
             float l = 0.f;
             unsigned m = 0;
+            const bool all_rows = nrows >= kTileBatch;
             // the loss kind is the same for the whole launch: one straight-line epilogue per kind
-            if (fl.kind == FFI_LOSS_SQUARED_HINGE) loss_epilogue<FFI_LOSS_SQUARED_HINGE>(acc, nrows, fl.scale, l, m);
-            else if (fl.kind == FFI_LOSS_HINGE) loss_epilogue<FFI_LOSS_HINGE>(acc, nrows, fl.scale, l, m);
-            else loss_epilogue<FFI_LOSS_BCE>(acc, nrows, fl.scale, l, m);
+            if (fl.kind == FFI_LOSS_SQUARED_HINGE) loss_epilogue<FFI_LOSS_SQUARED_HINGE>(acc, all_rows, regs_valid, fl.scale, l, m);
+            else if (fl.kind == FFI_LOSS_HINGE) loss_epilogue<FFI_LOSS_HINGE>(acc, all_rows, regs_valid, fl.scale, l, m);
+            else loss_epilogue<FFI_LOSS_BCE>(acc, all_rows, regs_valid, fl.scale, l, m);
             if (valid) {
                 lsum += l;
-                if (fl.skip_zero_stores) {
+                if (SKEW) {
+                    // register q is the gradient of batch entry q ^ r4: its row of out_grad is the lane's own
+                    unsigned r4 = (unsigned)(lane & 7) << 2;
+                    asm volatile("" : "+v"(r4));           // keeps the 32 row offsets from being hoisted out of the label loop
+#pragma unroll
+                    for (int q = 0; q < 32; ++q)
+                        if ((m >> q) & 1u)
+                            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, acc[q]), orsrc,
+                                                                  lane_off + ((unsigned)q ^ r4) * stride, 0u, 0);
+                    m = xor_permute_bits(m, lane & 7);
+                } else if (fl.skip_zero_stores) {
 #pragma unroll
                     for (int b = 0; b < 32; ++b)
                         if ((m >> b) & 1u)
@@ -275,7 +301,7 @@ __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* _
             }
         }
     }
-    if (EPI == kEpiLossGrad || EPI == kEpiLossGradAndScores) {
+    if (LOSS) {
         const double t = wave_sum((double)lsum);
         if (lane == 0) fl.partial[(size_t)blockIdx.x * (kTileThreads / 64) + (threadIdx.x >> 6)] = t;
     }
@@ -325,9 +351,11 @@ template <int EPI>
 int launch_lane32_any(bool vec4, bool topk, const float* xT, const int32_t* idx, const float* w, const float* bias, float* out,
                       const Dims& d, int nbt, int per_stream, int blocks, size_t lds, const FwdLoss& fl, const FwdTopk& ft,
                       hipStream_t s) {
-    if (topk)
-        return vec4 ? launch_lane32<true, EPI, true>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, ft, s)
-                    : launch_lane32<false, EPI, true>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, ft, s);
+    if constexpr (EPI != kEpiLossGradSkewed) {              // (that epilogue has no top-k form)
+        if (topk)
+            return vec4 ? launch_lane32<true, EPI, true>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, ft, s)
+                        : launch_lane32<false, EPI, true>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, ft, s);
+    }
     if (EPI == kEpiNone) return FFI_OK;                     // nothing to compute
     return vec4 ? launch_lane32<true, EPI == kEpiNone ? kEpiScores : EPI, false>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, ft, s)
                 : launch_lane32<false, EPI == kEpiNone ? kEpiScores : EPI, false>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, ft, s);
@@ -389,6 +417,8 @@ int forward_tiles(const float* x, const int32_t* idx, const float* w, const floa
         fl.skip_zero_stores = la->skip_zero_stores ? 1 : 0;
     }
     if (epi == kEpiScores) FFI_TRY(launch_lane32_any<kEpiScores>(vec4, topk, xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds_topk, fl, ft, s));
+    else if (epi == kEpiLossGrad && !topk && fl.skip_zero_stores)
+        FFI_TRY(launch_lane32_any<kEpiLossGradSkewed>(vec4, false, xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds_topk, fl, ft, s));
     else if (epi == kEpiLossGrad) FFI_TRY(launch_lane32_any<kEpiLossGrad>(vec4, topk, xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds_topk, fl, ft, s));
     else if (epi == kEpiLossGradAndScores) FFI_TRY(launch_lane32_any<kEpiLossGradAndScores>(vec4, topk, xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds_topk, fl, ft, s));
     else FFI_TRY(launch_lane32_any<kEpiNone>(vec4, topk, xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds_topk, fl, ft, s));

@@ -120,6 +120,14 @@ __device__ __forceinline__ void xor_permute_groups(float (&v)[32], int r) {
         if (!(e & 4)) cond_swap(b1, v[e], v[e + 4]);
 }
 
+// The same permutation applied to the 32 bits of a mask (bit e <-> bit e ^ 4r): halves, bytes, nibbles.
+__device__ __forceinline__ unsigned xor_permute_bits(unsigned m, int r) {
+    if (r & 4) m = (m >> 16) | (m << 16);
+    if (r & 2) m = ((m & 0xff00ff00u) >> 8) | ((m & 0x00ff00ffu) << 8);
+    if (r & 1) m = ((m & 0xf0f0f0f0u) >> 4) | ((m & 0x0f0f0f0fu) << 4);
+    return m;
+}
+
 // Byte address (inside the tile) of the chunk read at step C, given base = row*128 | (lane&7)*16.
 template <int C>
 __device__ __forceinline__ unsigned skew_addr(unsigned base) { return C == 0 ? base : (base ^ (unsigned)(C * 16)); }
