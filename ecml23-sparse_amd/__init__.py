@@ -29,7 +29,7 @@ from .fixed_fan_in_ops import (  # noqa: E402
     fan_in_sparse_topk,
 )
 from . import custom_layer, metrics, optimizer  # noqa: E402
-from .optimizer import SparseAdam  # noqa: E402
+from .optimizer import SparseAdam, SparseOptWrapper, RewireCallback  # noqa: E402
 from .metrics import (  # noqa: E402
     SparseHingeLoss,
     SparseSquaredHingeLoss,
@@ -65,4 +65,6 @@ __all__ = [
     "SparsePrecision",
     "SparseRecall",
     "SparseAdam",
+    "SparseOptWrapper",
+    "RewireCallback",
 ]

@@ -117,6 +117,11 @@ class StratifiedRewireLayerV2(torch.nn.Module):
         tp_in = inputs.t().contiguous()
         return ops.fan_in_sparse_matmul_tp(tp_in, indices, weights)
 
+    @property
+    def sparse_weights(self):
+        """The variable an optimizer keeps moments for (sparse/layer.py:160-162)."""
+        return self.kernel_weights
+
     def forward(self, inputs: torch.Tensor) -> torch.Tensor:
         if inputs.dim() != 2 or inputs.shape[1] != self.input_dim:
             raise ValueError(f"inputs must have shape [batch, {self.input_dim}], got {tuple(inputs.shape)}")

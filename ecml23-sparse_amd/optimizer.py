@@ -60,12 +60,85 @@ class SparseAdam:
 
     def update_sparse(self, layer):
         if self.update_moments:
-            i = self._index_of(layer.kernel_weights)
+            i = self._index_of(layer.sparse_weights)
             new_m, new_v = layer.rewire([self._momentums[i], self._velocities[i]])
             self._momentums[i].copy_(new_m)
             self._velocities[i].copy_(new_v)
         else:
             layer.rewire(None)
+
+
+class SparseOptWrapper(torch.nn.Module):
+    """The training loop's model wrapper (sparse/optimizer.py:26-74): ``train_step((x, y))`` runs the base
+    model, the loss, the backward pass and the optimizer step, then lets the optimizer rewire every sparse layer
+    when ``optimizer.iterations % rewire_interval == 1`` (``rewire_interval <= 0``: never).
+
+    ``compile(optimizer, loss, metrics)`` takes an optimizer with ``zero_grad()``, ``step()``, ``iterations`` and
+    ``update_sparse(layer)`` (``SparseAdam``), a loss called as ``loss(y_true, y_pred)`` and metrics with
+    ``update_state(y_true, y_pred)`` / ``result()``.  Several optimizers may be given as a list: they are stepped
+    together and the first one that has ``update_sparse`` does the rewiring (torch models often keep a stock optimizer
+    for their dense layers).
+    """
+
+    def __init__(self, rewire_interval: int, base_model: torch.nn.Module):
+        super().__init__()
+        self.rewire_interval = int(rewire_interval)
+        self.base_model = base_model
+        self.optimizers = []
+        self.loss = None
+        self.metrics = []
+
+    def forward(self, *args, **kwargs):
+        return self.base_model(*args, **kwargs)
+
+    def compile(self, optimizer, loss, metrics=()):
+        self.optimizers = list(optimizer) if isinstance(optimizer, (list, tuple)) else [optimizer]
+        if not any(hasattr(o, "update_sparse") for o in self.optimizers):
+            raise TypeError("one of the optimizers must have update_sparse(layer)")
+        self.loss = loss
+        self.metrics = list(metrics)
+
+    @property
+    def optimizer(self):
+        """The optimizer that rewires (the reference's single optimizer)."""
+        return next(o for o in self.optimizers if hasattr(o, "update_sparse"))
+
+    def sparse_layers(self):
+        return [m for m in self.base_model.modules() if hasattr(m, "sparse_weights")]
+
+    def train_step(self, data):
+        x, y = data
+        for o in self.optimizers:
+            o.zero_grad()
+        y_pred = self.base_model(x)
+        loss = self.loss(y, y_pred)
+        loss.backward()
+        for o in self.optimizers:
+            o.step()
+        self.handle_sparse_layers()
+        results = {"loss": float(loss.detach())}
+        with torch.no_grad():
+            for m in self.metrics:
+                m.update_state(y, y_pred.detach())
+                results[getattr(m, "name", type(m).__name__)] = m.result()
+        return results
+
+    def handle_sparse_layers(self):
+        if self.rewire_interval > 0 and self.optimizer.iterations % self.rewire_interval == 1:
+            for layer in self.sparse_layers():
+                self.optimizer.update_sparse(layer)
+
+
+class RewireCallback:
+    """Rewires every sparse layer at the start of each epoch but the first (sparse/optimizer.py:77-86)."""
+
+    def __init__(self, model: "SparseOptWrapper"):
+        self.model = model
+
+    def on_epoch_begin(self, epoch, logs=None):
+        if epoch != 0:
+            for layer in self.model.sparse_layers():
+                self.model.optimizer.update_sparse(layer)
 
 
 def backward_sparse_adam(features, lookup, weights, out_grad, nz_words, weight_m, weight_v, bias, bias_m, bias_v,

@@ -292,3 +292,56 @@ def test_dense_stratified_block_trains_end_to_end(ffi):
     assert 0.0 <= p1.result() <= 1.0
     # the listed labels are being pulled apart from the rest
     assert float(scores[rows, cols].mean()) > float(scores.mean()) + 0.1
+
+
+def test_training_loop_wrapper_rewires_on_schedule(ffi):
+    # SparseOptWrapper.train_step (sparse/optimizer.py:43-74): forward, loss, backward, optimizer step, and a rewire of
+    # every sparse layer whenever optimizer.iterations % rewire_interval == 1; RewireCallback rewires at epoch starts.
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    B, D, H, L = 32, 48, 64, 800
+
+    class Net(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.dense = torch.nn.Linear(D, H)
+            # (arrange=False: connections keep their places, so a changed index is a redrawn connection)
+            self.sparse = ffi.StratifiedRewireLayerV2(units=L, input_dim=H, connections=L * 8, generator=gen, arrange=False,
+                                                      rewire_selector=ffi.FixedFractionSelector(0.05))
+
+        def forward(self, x):
+            return self.sparse(torch.relu(self.dense(x)))
+
+    net = Net().cuda()
+    model = ffi.SparseOptWrapper(rewire_interval=4, base_model=net)
+    with pytest.raises(TypeError):
+        model.compile(torch.optim.Adam(net.dense.parameters(), lr=0.01), ffi.SparseSquaredHingeLoss())
+    sparse_opt = ffi.SparseAdam(list(net.sparse.parameters()), learning_rate=0.01)
+    model.compile([torch.optim.Adam(net.dense.parameters(), lr=0.01), sparse_opt], ffi.SparseSquaredHingeLoss(),
+                  metrics=[ffi.PrecisionAtK(k=1)])
+    assert model.optimizer is sparse_opt and model.sparse_layers() == [net.sparse]
+    x = torch.rand((B, D), device="cuda", generator=gen)
+    rows = torch.arange(B, device="cuda").repeat_interleave(2)
+    cols = torch.randint(0, L, (B * 2,), device="cuda", generator=gen)
+    y = (torch.stack([rows, cols], dim=1), None)
+    rewired_at, losses = [], []
+    for it in range(1, 13):
+        before = net.sparse.kernel_indices.clone()
+        out = model.train_step((x, y))
+        assert sparse_opt.iterations == it
+        if not torch.equal(before, net.sparse.kernel_indices):
+            rewired_at.append(it)
+            # the optimizer's moments are cleared where connections were redrawn
+            changed = before != net.sparse.kernel_indices
+            i = sparse_opt._index_of(net.sparse.sparse_weights)
+            assert float(sparse_opt._momentums[i][changed].abs().max()) == 0.0
+            assert float(sparse_opt._velocities[i][changed].abs().max()) == 0.0
+        losses.append(out["loss"])
+        assert 0.0 <= out["P_at_1"] <= 1.0
+    assert rewired_at == [1, 5, 9]
+    assert losses[-1] < losses[0]
+    cb = ffi.RewireCallback(model)
+    before = net.sparse.kernel_indices.clone()
+    cb.on_epoch_begin(0)
+    assert torch.equal(before, net.sparse.kernel_indices)
+    cb.on_epoch_begin(1)
+    assert not torch.equal(before, net.sparse.kernel_indices)
