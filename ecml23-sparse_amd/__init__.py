@@ -38,7 +38,7 @@ from .metrics import (  # noqa: E402
     SparsePrecision,
     SparseRecall,
 )
-from .custom_layer import StratifiedRewireLayerV2, FixedFractionSelector, FixedMagnitudeSelector  # noqa: E402
+from .custom_layer import StratifiedRewireLayerV2, RewireSelector, FixedFractionSelector, FixedMagnitudeSelector  # noqa: E402
 
 __all__ = [
     "fan_in_sparse_matmul",
@@ -56,6 +56,7 @@ __all__ = [
     "backward_sparse",
     "fan_in_sparse_topk",
     "StratifiedRewireLayerV2",
+    "RewireSelector",
     "FixedFractionSelector",
     "FixedMagnitudeSelector",
     "SparseHingeLoss",

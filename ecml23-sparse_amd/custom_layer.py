@@ -16,7 +16,20 @@ import torch
 from . import fixed_fan_in_ops as ops
 
 
-class FixedMagnitudeSelector:
+class RewireSelector:
+    """Decides which connections a rewiring step replaces (sparse/layer.py:30-44): ``select(weight_values)``
+    returns a boolean tensor, true where a connection shall be rewired.  A selector may also offer
+    ``threshold_tensor(weight_values)`` (rewire everything strictly below a magnitude): the layer then selects,
+    redraws and clears optimizer state in one library call instead of torch index operations."""
+
+    def select(self, weight_values: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError()
+
+    def build(self, weight_values: torch.Tensor):
+        pass
+
+
+class FixedMagnitudeSelector(RewireSelector):
     """Rewire all weights below a fixed magnitude (sparse/layer.py:45-57)."""
 
     def __init__(self, threshold: float):
@@ -30,7 +43,7 @@ class FixedMagnitudeSelector:
         return torch.full((1,), self.threshold, dtype=torch.float32, device=weight_values.device)
 
 
-class FixedFractionSelector:
+class FixedFractionSelector(RewireSelector):
     """Rewire a fixed fraction of the connections, those of lowest magnitude (sparse/layer.py:60-84).
 
     As in the reference the threshold is the ``round(fraction * n)``-th smallest magnitude and the

@@ -345,3 +345,31 @@ def test_training_loop_wrapper_rewires_on_schedule(ffi):
     assert torch.equal(before, net.sparse.kernel_indices)
     cb.on_epoch_begin(1)
     assert not torch.equal(before, net.sparse.kernel_indices)
+
+
+def test_rewire_with_a_selector_that_only_offers_a_mask(ffi):
+    # a RewireSelector subclass with select() alone (sparse/layer.py:30-44): the layer redraws exactly the selected
+    # connections, keeps their weights, and returns optimizer state cleared at those places
+    class EveryThird(ffi.RewireSelector):
+        def select(self, weight_values):
+            return (torch.arange(weight_values.numel(), device=weight_values.device) % 3) == 0
+
+    gen = torch.Generator(device="cuda").manual_seed(9)
+    units, N, K = 40, 50, 6
+    layer = ffi.StratifiedRewireLayerV2(units, N, connections=units * K, rewire_selector=EveryThird(), arrange=False,
+                                        generator=gen)
+    before_idx, before_w = layer.kernel_indices.clone(), layer.kernel_weights.detach().clone()
+    m = torch.ones(units * K, device="cuda")
+    (new_m,) = layer.rewire([m])
+    picked = EveryThird().select(before_w)
+    assert torch.equal(layer.kernel_weights.detach(), before_w)
+    assert torch.equal(layer.kernel_indices[~picked], before_idx[~picked])
+    assert int((layer.kernel_indices[picked] != before_idx[picked]).sum()) > 0.8 * int(picked.sum())
+    assert bool(((layer.kernel_indices >= 0) & (layer.kernel_indices < N)).all())
+    assert torch.equal(new_m, torch.where(picked, torch.zeros_like(m), m))
+    # and the layer still computes what its (edited) variables say
+    x = torch.rand((8, N), device="cuda", generator=gen)
+    out = layer(x)
+    ref = oracle.forward(x.cpu().numpy(), layer.kernel_indices.view(units, K).cpu().numpy().astype(np.int32),
+                         layer.kernel_weights.detach().view(units, K).cpu().numpy()) + layer.bias.detach().cpu().numpy()[None, :]
+    assert rel_err(out.detach().cpu().numpy(), ref) <= FWD_RTOL
