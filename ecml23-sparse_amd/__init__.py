@@ -35,6 +35,7 @@ from .metrics import (  # noqa: E402
     SparseSquaredHingeLoss,
     SparseBinaryCrossEntropyLoss,
     PrecisionAtK,
+    topk_as_matrix,
     SparsePrecision,
     SparseRecall,
 )
@@ -63,6 +64,7 @@ __all__ = [
     "SparseSquaredHingeLoss",
     "SparseBinaryCrossEntropyLoss",
     "PrecisionAtK",
+    "topk_as_matrix",
     "SparsePrecision",
     "SparseRecall",
     "SparseAdam",

@@ -199,6 +199,18 @@ class SparseBinaryCrossEntropyLoss(SparseLossBase):
         super().__init__(name)
 
 
+def topk_as_matrix(data, k):
+    """The positions of the k best scores of every row as a sparse 0/1 matrix of ``data``'s shape
+    (sparse/metrics.py:9-28): ``(indices [B*k, 2] int64 in row-major order, values [B*k] of ones, dense_shape)``,
+    the triple a ``tf.sparse.SparseTensor`` holds.  Equal scores go to the lower label."""
+    _, top = topk_scores(data, int(k))
+    batch = data.shape[0]
+    cols, _ = torch.sort(top.to(torch.int64), dim=1)                           # tf.sparse.reorder: ascending columns
+    rows = torch.arange(batch, device=data.device).unsqueeze(1).expand_as(cols)
+    indices = torch.stack([rows.reshape(-1), cols.reshape(-1)], dim=1)
+    return indices, torch.ones(indices.shape[0], dtype=torch.float32, device=data.device), tuple(data.shape)
+
+
 class PrecisionAtK:
     """Fraction of the k best-scored labels of each sample that are true labels, accumulated over
     ``update_state`` calls (sparse/metrics.py:31-71: label values at the top-k positions are summed,

@@ -308,3 +308,15 @@ def test_forward_loss_with_topk_by_product(ffi, shape):
     truth = np.zeros((B, L), np.float32)
     truth[indices[:, 0], indices[:, 1]] = values
     assert abs(p5.result() - truth[np.arange(B)[:, None], ref_i].sum() / (B * 5)) < 1e-9
+
+
+def test_topk_as_matrix(ffi):
+    # sparse/metrics.py:9-28: a 0/1 matrix with k ones per row at the best scores, indices in row-major order
+    rng = np.random.default_rng(8)
+    scores = rng.standard_normal((9, 300)).astype(np.float32)
+    indices, values, shape = ffi.topk_as_matrix(torch.from_numpy(scores).cuda(), 3)
+    torch.cuda.synchronize()
+    assert shape == (9, 300) and values.tolist() == [1.0] * 27
+    _, oi = oracle.topk(scores, 3)
+    expect = np.stack([np.repeat(np.arange(9), 3), np.sort(oi, axis=1).reshape(-1)], axis=1)
+    assert np.array_equal(indices.cpu().numpy(), expect)
