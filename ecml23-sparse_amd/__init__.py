@@ -39,7 +39,7 @@ from .metrics import (  # noqa: E402
     SparsePrecision,
     SparseRecall,
 )
-from .custom_layer import StratifiedRewireLayerV2, RewireSelector, FixedFractionSelector, FixedMagnitudeSelector  # noqa: E402
+from .custom_layer import StratifiedRewireLayerV2, StratifiedRewireLayer, RewireSelector, FixedFractionSelector, FixedMagnitudeSelector  # noqa: E402
 
 __all__ = [
     "fan_in_sparse_matmul",
@@ -57,6 +57,7 @@ __all__ = [
     "backward_sparse",
     "fan_in_sparse_topk",
     "StratifiedRewireLayerV2",
+    "StratifiedRewireLayer",
     "RewireSelector",
     "FixedFractionSelector",
     "FixedMagnitudeSelector",

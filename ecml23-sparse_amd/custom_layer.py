@@ -211,3 +211,28 @@ class StratifiedRewireLayerV2(torch.nn.Module):
         if self.arrange:
             self.arrange_connections(outputs)
         return outputs
+
+
+class StratifiedRewireLayer(StratifiedRewireLayerV2):
+    """The reference's first fixed-fan-in layer (sparse/layer.py:339-390): the same variables and the same
+    arithmetic as ``StratifiedRewireLayerV2`` (there a ``tf.sparse`` product with a kernel whose rows all hold
+    ``connections // units`` entries), with one visible difference: every rewiring re-sorts the connections
+    (``tf.sparse.reorder``), so inside a unit the sources are in ascending order, and weights and optimizer state
+    move with them.  Here the call runs through the same fixed-fan-in kernels; sorted rows are also the layout the
+    inference configuration gathers fastest."""
+
+    def __init__(self, units: int, input_dim: int, **kwargs):
+        kwargs["arrange"] = False          # the order inside a unit is this layer's own
+        super().__init__(units, input_dim, **kwargs)
+
+    @torch.no_grad()
+    def _sort_rows(self, other_vars):
+        idx = self.kernel_indices.view(-1, self.fan_in)
+        order = torch.argsort(idx.to(torch.int64), dim=1, stable=True)
+        self.kernel_indices.copy_(torch.gather(idx, 1, order).reshape(-1))
+        self.kernel_weights.data.copy_(torch.gather(self.kernel_weights.data.view(-1, self.fan_in), 1, order).reshape(-1))
+        return [torch.gather(o.reshape(-1, self.fan_in), 1, order).reshape(o.shape) for o in other_vars]
+
+    @torch.no_grad()
+    def rewire(self, other_vars=None):
+        return self._sort_rows(super().rewire(other_vars))

@@ -373,3 +373,31 @@ def test_rewire_with_a_selector_that_only_offers_a_mask(ffi):
     ref = oracle.forward(x.cpu().numpy(), layer.kernel_indices.view(units, K).cpu().numpy().astype(np.int32),
                          layer.kernel_weights.detach().view(units, K).cpu().numpy()) + layer.bias.detach().cpu().numpy()[None, :]
     assert rel_err(out.detach().cpu().numpy(), ref) <= FWD_RTOL
+
+
+def test_first_generation_layer_keeps_rows_sorted(ffi):
+    # StratifiedRewireLayer (sparse/layer.py:339-390): same arithmetic, but a rewiring re-sorts every unit's sources
+    # (tf.sparse.reorder) and moves weights and optimizer state with them
+    gen = torch.Generator(device="cuda").manual_seed(13)
+    units, N, K = 60, 90, 8
+    layer = ffi.StratifiedRewireLayer(units, N, connections=units * K, rewire_selector=ffi.FixedFractionSelector(0.2),
+                                      generator=gen)
+    w_before = layer.kernel_weights.detach().clone()
+    idx_before = layer.kernel_indices.clone()
+    tag = torch.arange(units * K, device="cuda", dtype=torch.float32) + 1.0          # follows every connection around
+    (tag_after,) = layer.rewire([tag])
+    idx = layer.kernel_indices.view(units, K)
+    assert bool((idx[:, 1:] >= idx[:, :-1]).all())
+    # a connection that was not redrawn (tag not cleared) still has its weight and its source, at its new place
+    kept = tag_after > 0
+    origin = (tag_after[kept] - 1).long()
+    assert torch.equal(layer.kernel_weights.detach()[kept], w_before[origin])
+    assert torch.equal(layer.kernel_indices[kept], idx_before[origin])
+    assert int((~kept).sum()) == int(round(0.2 * units * K)) - 1 or int((~kept).sum()) == int(round(0.2 * units * K))
+    # redrawn connections keep their weights too (rows are permutations of the old rows)
+    assert torch.equal(torch.sort(layer.kernel_weights.detach().view(units, K), dim=1).values,
+                       torch.sort(w_before.view(units, K), dim=1).values)
+    x = torch.rand((16, N), device="cuda", generator=gen)
+    ref = oracle.forward(x.cpu().numpy(), idx.cpu().numpy().astype(np.int32),
+                         layer.kernel_weights.detach().view(units, K).cpu().numpy()) + layer.bias.detach().cpu().numpy()[None, :]
+    assert rel_err(layer(x).detach().cpu().numpy(), ref) <= FWD_RTOL
