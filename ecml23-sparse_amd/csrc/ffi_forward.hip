@@ -12,6 +12,8 @@
 #include "ffi_loss.h"
 
 #include <algorithm>
+#include <climits>
+#include <mutex>
 
 namespace ffi {
 namespace {
@@ -363,12 +365,14 @@ int launch_lane32_any(bool vec4, bool topk, const float* xT, const int32_t* idx,
 
 // Narrow-input forward pass with the given epilogue; `la` is needed for the loss epilogues only, `tk` (may be
 // null) asks for the per-sample top-k without the score matrix.
+// `xt_scratch` (may be null): room for N * B floats that takes the place of the library workspace for the
+// batch-major copy of [B,N] features.
 int forward_tiles(const float* x, const int32_t* idx, const float* w, const float* bias, float* out, float* gout, int epi,
-                  const LossArgs* la, const TopkArgs* tk, const Dims& d, hipStream_t s) {
+                  const LossArgs* la, const TopkArgs* tk, const Dims& d, hipStream_t s, float* xt_scratch = nullptr) {
     const float* xT = x;
     if (!d.tp) {
-        float* ws = nullptr;
-        FFI_TRY(workspace_get(s, kWsFeaturesT, (size_t)d.N * d.B * sizeof(float), (void**)&ws));
+        float* ws = xt_scratch;
+        if (ws == nullptr) FFI_TRY(workspace_get(s, kWsFeaturesT, (size_t)d.N * d.B * sizeof(float), (void**)&ws));
         FFI_TRY(launch_transpose(x, ws, d.B, d.N, s));   // [B,N] -> [N,B]
         xT = ws;
     }
@@ -468,4 +472,52 @@ int launch_forward_topk(const float* x, const int32_t* idx, const float* w, cons
     return launch_topk_f32(sc, d.B, d.L, tk.k, tk.values, tk.indices, s);
 }
 
+// ---- forward pass for callers that cannot allocate ------------------------------------------------
+// The only device memory the narrow forward pass needs beyond its inputs and outputs is the [N][B]
+// copy of [B,N] features.  Here it lives in a fixed array inside the library's code object (one copy
+// per GPU, held until the process ends) instead of a workspace from hipMalloc.
+namespace {
+
+constexpr size_t kNoAllocFloats = (size_t)1 << 20;             // 4 MiB: batch * num_features may not exceed this
+static __device__ __align__(256) float scratch[kNoAllocFloats];
+
+constexpr int kNoAllocMaxDevices = 64;
+std::mutex g_scratch_mutex;
+float* g_scratch_ptr[kNoAllocMaxDevices] = {nullptr};           // device address of `scratch` on each GPU
+
+// The address of this GPU's copy of `scratch` (looked up once per device, with that device current).
+int scratch_address(float** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return FFI_ERR_NO_DEVICE; }
+    if (dev < 0 || dev >= kNoAllocMaxDevices) return FFI_ERR_NO_DEVICE;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        float* ptr = nullptr;
+        FFI_HIP_TRY(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)));
+        if (ptr == nullptr) return FFI_ERR_HIP;
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return FFI_OK;
+}
+
+}  // namespace
 }  // namespace ffi
+
+extern "C" int ffi_forward_noalloc_f32(const float* features, const int32_t* lookup, const float* weights, float* result,
+                                       int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in, int transposed,
+                                       ffi_stream_t stream) {
+    using namespace ffi;
+    StreamCall call_lock((hipStream_t)stream);
+    if (!features || !lookup || !weights || !result) return FFI_ERR_NULL_POINTER;
+    if (batch <= 0 || num_features <= 0 || num_units <= 0 || fan_in <= 0) return FFI_ERR_BAD_SHAPE;
+    if (batch >= INT32_MAX || num_features >= INT32_MAX || num_units >= INT32_MAX || fan_in >= INT32_MAX) return FFI_ERR_TOO_LARGE;
+    if (num_units * fan_in >= INT32_MAX) return FFI_ERR_TOO_LARGE;
+    // only the shapes of the narrow kernel, which needs nothing but the fixed array
+    if (!tile_path_fits((int)num_features) || num_units >= (1 << 25)) return FFI_ERR_TOO_LARGE;
+    if ((uint64_t)batch * (uint64_t)num_features > kNoAllocFloats) return FFI_ERR_TOO_LARGE;
+    const Dims d{(int)batch, (int)num_features, (int)num_units, (int)fan_in, transposed != 0};
+    float* xt = nullptr;
+    if (!d.tp) FFI_TRY(scratch_address(&xt));
+    return forward_tiles(features, lookup, weights, nullptr, result, nullptr, kEpiScores, nullptr, nullptr, d, (hipStream_t)stream, xt);
+}

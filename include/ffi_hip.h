@@ -69,6 +69,21 @@ int ffi_forward_f32(const float* features, const int32_t* lookup, const float* w
                     int transposed, ffi_stream_t stream);
 
 /*
+ * ffi_forward_f32 for callers that cannot allocate device memory while they run: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.
+ * Same arguments and results (bit for bit) as ffi_forward_f32, but the call allocates nothing: the one buffer
+ * the kernels need beyond inputs and outputs -- the [num_features, batch] copy of [batch, num_features]
+ * features -- lives in a fixed 4 MiB array inside the library's code object (one per GPU, held until the
+ * process ends).  Limits: num_features <= 1216 (the kernel that keeps a tile of the features in LDS) and
+ * batch * num_features <= 1,048,576; anything larger returns FFI_ERR_TOO_LARGE.  Every call on a GPU uses
+ * that GPU's one array (it is overwritten, never read before it is written, so nothing needs clearing):
+ * calls that overlap on one GPU -- two streams, or two threads -- race, and the caller must serialise them.
+ */
+int ffi_forward_noalloc_f32(const float* features, const int32_t* lookup, const float* weights, float* result,
+                            int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in,
+                            int transposed, ffi_stream_t stream);
+
+/*
  * Backward, both gradients from one call, as the reference's grad op does:
  *   feature_grad[b,n] = sum over (j,k) with lookup[j,k]==n of weights[j,k] * out_grad[b,j]
  *   weight_grad[j,k]  = sum_b features[b, lookup[j,k]] * out_grad[b,j]
