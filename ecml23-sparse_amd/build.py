@@ -30,6 +30,7 @@ SOURCES = [
     "ffi_sparse_grad.hip",
     "ffi_optimizer.hip",
     "ffi_rewire.hip",
+    "ffi_fallback.hip",
 ]
 
 # gfx950 only.  Packed-fp32 VALU forms are switched off for all device code.

@@ -84,38 +84,59 @@ int create_cached_plan(const int32_t* lookup, const Dims& d, int dev, hipStream_
     return FFI_OK;
 }
 
+// What `between` computes through the plan, for the kernels that redo it when the plan turns out to be outdated
+// (all null: nothing).
+struct PlannedWeightGrad {
+    const float* features = nullptr;
+    float* weight_grad = nullptr;
+    float* bias_grad = nullptr;
+};
+
+void drop_cached_plan(ffi_plan* p) {
+    for (size_t i = 0; i < g_cache.size(); ++i)
+        if (g_cache[i] == p) { g_cache.erase(g_cache.begin() + i); break; }
+    (void)hipDeviceSynchronize();
+    plan_free(p);
+    delete p;
+}
+
 // Input gradient through the plan cache, with `between(plan)` (the weight-gradient launch, or
-// nothing) enqueued ahead of it.  The lookup's content fingerprint is re-checked on every call: its
-// kernel goes first, then `between` is enqueued with the cached plan, and the host waits for the
-// fingerprint kernel alone, so that it learns the result, and enqueues the input-gradient kernels,
-// while the weight gradient is still running.  If the lookup did change (a rewire), the plan is
-// rebuilt and `between` is enqueued again: it overwrites, in stream order, what the first launch
-// computed from the plan's outdated copy of the column ids (plan-driven kernels read the plan,
-// never the lookup, so that first launch is safe whatever the lookup holds now).
+// nothing) enqueued ahead of it.  The host never waits in the steady state (the reference's op only
+// enqueues, tfsparse/cc/kernels/backward.cu:59-64): the lookup's content is checked against the cached
+// plan by a kernel that leaves its verdict on the device; the plan-driven kernels follow -- they read the
+// plan, never the lookup, so they are safe whatever the lookup holds now -- and behind them kernels that
+// recompute both gradients straight from the lookup if the verdict says the plan is outdated (a rewire),
+// and return at once otherwise.  The host looks at the verdict of an earlier call when that has arrived
+// (a poll, not a wait) and only then rebuilds the plan, which does synchronise.
 template <class Between>
 int input_grad_cached(const int32_t* lookup, const float* weights, const float* out_grad, float* feature_grad,
-                      const Dims& d, hipStream_t s, Between between) {
+                      const Dims& d, hipStream_t s, Between between, const PlannedWeightGrad& wg = PlannedWeightGrad()) {
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess) return FFI_ERR_NO_DEVICE;
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     ffi_plan* p = find_cached_plan(lookup, d, dev);
-    if (p) {
-        FFI_TRY(plan_fingerprint_begin(p, lookup, s));
-        const int st_between = between(p);
-        unsigned long long fp = 0, bad = 0;
-        const int st_fp = plan_fingerprint_end(p, &fp, &bad);
-        if (st_between != FFI_OK) return st_between;
-        if (st_fp != FFI_OK) return st_fp;
-        if (bad) return FFI_ERR_BAD_LOOKUP;
-        if (fp != p->fingerprint) {
-            FFI_TRY(plan_build(p, lookup, s));
-            FFI_TRY(between(p));
-        }
-    } else {
+    if (!p) {
         FFI_TRY(create_cached_plan(lookup, d, dev, s, &p));
         FFI_TRY(between(p));
+        return launch_input_grad(p, weights, out_grad, feature_grad, d.B, d.tp, s);
     }
-    return launch_input_grad(p, weights, out_grad, feature_grad, d.B, d.tp, s);
+    bool seen = false, current = true;
+    unsigned long long bad = 0;
+    FFI_TRY(plan_guard_poll(p, &seen, &current, &bad));
+    if (seen && !current) {
+        // the lookup changed under the plan (the calls since then were served by the recomputing kernels);
+        // the build fingerprints the present content, so this call needs no check
+        const int st = plan_build(p, lookup, s);
+        if (st != FFI_OK) { drop_cached_plan(p); return st; }
+        FFI_TRY(between(p));
+        return launch_input_grad(p, weights, out_grad, feature_grad, d.B, d.tp, s);
+    }
+    FFI_TRY(plan_guard_enqueue(p, lookup, s));
+    FFI_TRY(between(p));
+    bool zeroed = false;
+    FFI_TRY(launch_input_grad(p, weights, out_grad, feature_grad, d.B, d.tp, s, p->d_guard + kGuardVerdict, &zeroed));
+    return launch_backward_if_outdated(p->d_guard + kGuardVerdict, wg.features, lookup, weights, out_grad, feature_grad,
+                                       wg.weight_grad, wg.bias_grad, d, s, zeroed);
 }
 
 }  // namespace
@@ -199,7 +220,9 @@ int ffi_backward_f32(const float* features, const int32_t* lookup, const float* 
         return weight_grad ? launch_weight_grad(features, lookup, out_grad, weight_grad, nullptr, d, s, plan) : (int)FFI_OK;
     };
     if (!feature_grad) return wgrad(nullptr);
-    return input_grad_cached(lookup, weights, out_grad, feature_grad, d, s, wgrad);
+    PlannedWeightGrad wg;
+    if (weight_grad) { wg.features = features; wg.weight_grad = weight_grad; }
+    return input_grad_cached(lookup, weights, out_grad, feature_grad, d, s, wgrad, wg);
 }
 
 int ffi_backward_bias_f32(const float* features, const int32_t* lookup, const float* weights,
@@ -214,7 +237,9 @@ int ffi_backward_bias_f32(const float* features, const int32_t* lookup, const fl
     // the bias gradient (column sums of out_grad) is a by-product of the weight-gradient kernel
     auto wgrad = [&](const ffi_plan* plan) { return launch_weight_grad(features, lookup, out_grad, weight_grad, bias_grad, d, s, plan); };
     if (!feature_grad) return wgrad(nullptr);
-    return input_grad_cached(lookup, weights, out_grad, feature_grad, d, s, wgrad);
+    PlannedWeightGrad wg;
+    wg.features = features; wg.weight_grad = weight_grad; wg.bias_grad = bias_grad;
+    return input_grad_cached(lookup, weights, out_grad, feature_grad, d, s, wgrad, wg);
 }
 
 int ffi_forward_bf16_f32(const uint16_t* features, const int32_t* lookup, const uint16_t* weights, float* result,
@@ -357,7 +382,9 @@ int ffi_backward_sparse_f32(const float* features, const int32_t* lookup, const 
         FFI_TRY(wgrad(nullptr));
         return launch_input_grad_sparse(lookup, weights, out_grad, words, feature_grad, d, s);
     }
-    return input_grad_cached(lookup, weights, out_grad, feature_grad, d, s, wgrad);
+    PlannedWeightGrad wg;                                  // (the sparse weight gradient reads the lookup itself)
+    if (weight_grad && !sparse) { wg.features = features; wg.weight_grad = weight_grad; wg.bias_grad = bias_grad; }
+    return input_grad_cached(lookup, weights, out_grad, feature_grad, d, s, wgrad, wg);
 }
 
 int ffi_adam_step_f32(float* variable, float* m, float* v, const float* gradient, int64_t count, float learning_rate,
@@ -419,7 +446,9 @@ int ffi_backward_sparse_adam_f32(const float* features, const int32_t* lookup, f
     // dense kernels: gradients into a workspace, then the Adam pass
     if (grad_is_partial) FFI_TRY(launch_zero_unmasked(out_grad, words, d.B, d.L, s));
     auto wgrad = [&](const ffi_plan* plan) { return launch_weight_grad(features, lookup, out_grad, gw, gb, d, s, plan); };
-    if (feature_grad) FFI_TRY(input_grad_cached(lookup, weights, out_grad, feature_grad, d, s, wgrad));
+    PlannedWeightGrad wg;
+    wg.features = features; wg.weight_grad = gw; wg.bias_grad = gb;
+    if (feature_grad) FFI_TRY(input_grad_cached(lookup, weights, out_grad, feature_grad, d, s, wgrad, wg));
     else FFI_TRY(wgrad(nullptr));
     FFI_TRY(launch_adam_step(weights, weight_m, weight_v, gw, wcount, learning_rate, beta_1, beta_2, epsilon, (long long)step, s));
     if (bias) FFI_TRY(launch_adam_step(bias, bias_m, bias_v, gb, (size_t)d.L, learning_rate, beta_1, beta_2, epsilon, (long long)step, s));

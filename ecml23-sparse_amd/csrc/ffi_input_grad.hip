@@ -233,10 +233,16 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
 // gx = sum over streams, ascending: a fixed order, so results are reproducible.
 template <bool TP>
 __global__ __launch_bounds__(256) void igrad_reduce_kernel(const float* __restrict__ partial, float* __restrict__ gx,
-                                                           int B, int N, int streams, int nthreads, int bpad) {
+                                                           int B, int N, int streams, int nthreads, int bpad,
+                                                           const unsigned long long* __restrict__ verdict) {
     const int b = blockIdx.x * 256 + threadIdx.x;
     const int n = blockIdx.y;
     if (b >= B) return;
+    // the plan is known to be outdated: zeros, for the kernel that recomputes the gradient from the lookup to add to
+    if (verdict != nullptr && *verdict == 0) {
+        if (TP) gx[(size_t)n * B + b] = 0.f; else gx[(size_t)b * N + n] = 0.f;
+        return;
+    }
     float v = 0.f;
     const size_t step = (size_t)nthreads * bpad;
     const float* p = partial + (size_t)n * bpad + b;
@@ -252,7 +258,8 @@ __global__ __launch_bounds__(256) void igrad_reduce_kernel(const float* __restri
     if (TP) gx[(size_t)n * B + b] = v; else gx[(size_t)b * N + n] = v;
 }
 
-int launch_tiled(const ffi_plan* p, const float* w, const float* g, float* gx, int B, bool tp, hipStream_t s) {
+int launch_tiled(const ffi_plan* p, const float* w, const float* g, float* gx, int B, bool tp, hipStream_t s,
+                 const unsigned long long* verdict) {
     const int nbt = (B + kTileBatch - 1) / kTileBatch;
     const int cus = device_cu_count();
     int streams = std::max(1, std::min(p->tiles, cus / std::max(1, nbt)));
@@ -288,9 +295,9 @@ int launch_tiled(const ffi_plan* p, const float* w, const float* g, float* gx, i
 #undef FFI_LAUNCH_TILE
     dim3 rgrid((B + 255) / 256, p->N);
     if (tp)
-        hipLaunchKernelGGL(igrad_reduce_kernel<true>, rgrid, dim3(256), 0, s, partial, gx, B, p->N, streams, p->threads, bpad);
+        hipLaunchKernelGGL(igrad_reduce_kernel<true>, rgrid, dim3(256), 0, s, partial, gx, B, p->N, streams, p->threads, bpad, verdict);
     else
-        hipLaunchKernelGGL(igrad_reduce_kernel<false>, rgrid, dim3(256), 0, s, partial, gx, B, p->N, streams, p->threads, bpad);
+        hipLaunchKernelGGL(igrad_reduce_kernel<false>, rgrid, dim3(256), 0, s, partial, gx, B, p->N, streams, p->threads, bpad, verdict);
     FFI_HIP_TRY(hipGetLastError());
     return FFI_OK;
 }
@@ -298,8 +305,16 @@ int launch_tiled(const ffi_plan* p, const float* w, const float* g, float* gx, i
 }  // namespace
 
 int launch_input_grad(const ffi_plan* p, const float* w, const float* g, float* gx, int B, bool tp,
-                      hipStream_t s) {
-    if (p->tiled) return launch_tiled(p, w, g, gx, B, tp, s);
+                      hipStream_t s, const unsigned long long* verdict, bool* zeroed_if_outdated) {
+    if (zeroed_if_outdated) *zeroed_if_outdated = false;
+    // (a plan whose last build failed holds no arrays)
+    if (p->lookup == nullptr) return FFI_ERR_BAD_ARGUMENT;
+    if (p->tiled) {
+        if (!p->lab16 || !p->pos16 || !p->slice_off || !p->rowpos) return FFI_ERR_BAD_ARGUMENT;
+        if (zeroed_if_outdated) *zeroed_if_outdated = verdict != nullptr;
+        return launch_tiled(p, w, g, gx, B, tp, s, verdict);
+    }
+    if (!p->perm || !p->col_ptr) return FFI_ERR_BAD_ARGUMENT;
     return launch_input_grad_wide(p, w, g, gx, B, tp, s);
 }
 

@@ -217,6 +217,14 @@ struct ffi_plan {
     unsigned long long* h_scratch = nullptr;  // pinned mirror
     hipEvent_t fp_done = nullptr;             // recorded behind the fingerprint kernel and its copy to h_scratch
     int fp_blocks = 0;                        // workgroups of the fingerprint kernel in flight: that many pairs of partial sums
+    // Check of the lookup's content on the device, without a host wait (plan_guard_*): device words
+    // {running sum, running count of bad ids, workgroups finished, expected fingerprint, verdict (1 = the plan is
+    // current), fingerprint found, bad ids found}; the last three are copied to the pinned mirror behind every check
+    unsigned long long* d_guard = nullptr;
+    unsigned long long* h_guard = nullptr;
+    hipEvent_t guard_done = nullptr;          // recorded behind that copy
+    bool guard_pending = false;               // a check has been enqueued whose result the host has not looked at
+    hipStream_t guard_stream = nullptr;       // the stream of that check
     size_t bytes = 0;
 };
 
@@ -234,9 +242,24 @@ int plan_fingerprint_end(ffi_plan* p, unsigned long long* out, unsigned long lon
 int plan_fingerprint(ffi_plan* p, const int32_t* lookup, hipStream_t s, unsigned long long* out,
                      unsigned long long* bad_ids);
 int plan_scratch_alloc(ffi_plan* p);
+// Enqueues a check of `lookup` against the plan's fingerprint on `s`: the verdict lands in p->d_guard[kGuardVerdict]
+// (device) for the kernels enqueued behind it, and in the pinned mirror for a later call of the host.
+constexpr int kGuardVerdict = 4;
+int plan_guard_enqueue(ffi_plan* p, const int32_t* lookup, hipStream_t s);
+// What the last finished check found, if the host has not seen it yet: *seen = false when no check has finished
+// since the last poll.  Never waits.
+int plan_guard_poll(ffi_plan* p, bool* seen, bool* current, unsigned long long* bad_ids);
+// Both gradients recomputed straight from `lookup` by plain kernels that run only if *verdict == 0 (and return at
+// once otherwise): enqueued behind plan-driven kernels, they overwrite what an outdated plan produced.  features /
+// weight_grad / bias_grad may be null (no weight gradient wanted), feature_grad may be null.
+int launch_backward_if_outdated(const unsigned long long* verdict, const float* features, const int32_t* lookup,
+                                const float* weights, const float* out_grad, float* feature_grad, float* weight_grad,
+                                float* bias_grad, const Dims& d, hipStream_t s, bool feature_grad_is_zeroed);
 void plan_free(ffi_plan* p);
+// `verdict` (may be null): device word of a lookup check enqueued ahead; where the kernels can, they leave zeros in gx
+// when it says the plan is outdated (*zeroed_if_outdated tells whether they could)
 int launch_input_grad(const ffi_plan* p, const float* w, const float* g, float* gx, int B, bool tp,
-                      hipStream_t s);
+                      hipStream_t s, const unsigned long long* verdict = nullptr, bool* zeroed_if_outdated = nullptr);
 int launch_input_grad_wide(const ffi_plan* p, const float* w, const float* g, float* gx, int B, bool tp, hipStream_t s);
 }  // namespace ffi
 

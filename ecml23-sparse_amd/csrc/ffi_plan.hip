@@ -73,6 +73,61 @@ __global__ __launch_bounds__(kBlock) void fingerprint_kernel(const int32_t* __re
     }
 }
 
+// The same fingerprint, checked on the device: workgroups add their sums to guard[0] / guard[1] (integer adds:
+// the total does not depend on their order), the last one to finish compares the total with guard[3], leaves the
+// verdict in guard[4] (1 = content unchanged and every id in range), the sums in guard[5] / guard[6], and clears
+// the accumulators for the next check.
+__global__ __launch_bounds__(kBlock) void fingerprint_guard_kernel(const int32_t* __restrict__ idx, size_t total, unsigned N,
+                                                                    unsigned long long* __restrict__ guard) {
+    unsigned long long h = 0;
+    unsigned bad = 0;
+    const size_t stride = (size_t)gridDim.x * kBlock;
+    const size_t tid = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    const bool vec = ((uintptr_t)idx & 15) == 0;
+    const size_t nvec = vec ? total / 4 : 0;
+    const int4* idx4 = reinterpret_cast<const int4*>(idx);
+#pragma unroll 4
+    for (size_t q = tid; q < nvec; q += stride) {
+        const int4 v = idx4[q];
+        const unsigned p = (unsigned)(q * 4);
+        h += mix32((unsigned)v.x + p * 0x9e3779b1u);
+        h += mix32((unsigned)v.y + (p + 1) * 0x9e3779b1u);
+        h += mix32((unsigned)v.z + (p + 2) * 0x9e3779b1u);
+        h += mix32((unsigned)v.w + (p + 3) * 0x9e3779b1u);
+        bad += ((unsigned)v.x >= N) + ((unsigned)v.y >= N) + ((unsigned)v.z >= N) + ((unsigned)v.w >= N);
+    }
+    for (size_t p = nvec * 4 + tid; p < total; p += stride) {
+        const unsigned id = (unsigned)idx[p];
+        h += mix32(id + (unsigned)p * 0x9e3779b1u);
+        bad += id >= N;
+    }
+    unsigned long long b64 = bad;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        h += __shfl_down(h, off);
+        b64 += __shfl_down(b64, off);
+    }
+    __shared__ unsigned long long part[2][kBlock / 64];
+    if ((threadIdx.x & 63) == 0) { part[0][threadIdx.x >> 6] = h; part[1][threadIdx.x >> 6] = b64; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned long long hs = 0, bs = 0;
+#pragma unroll
+        for (int i = 0; i < kBlock / 64; ++i) { hs += part[0][i]; bs += part[1][i]; }
+        atomicAdd(&guard[0], hs);
+        atomicAdd(&guard[1], bs);
+        __threadfence();
+        if (atomicAdd(&guard[2], 1ull) == (unsigned long long)gridDim.x - 1) {
+            __threadfence();
+            const unsigned long long sum = atomicAdd(&guard[0], 0ull), nbad = atomicAdd(&guard[1], 0ull);
+            guard[5] = sum;
+            guard[6] = nbad;
+            guard[4] = (sum == guard[3] && nbad == 0) ? 1ull : 0ull;
+            guard[0] = 0; guard[1] = 0; guard[2] = 0;
+        }
+    }
+}
+
 // ---- tiled form ---------------------------------------------------------------------------------
 
 // Order of a column's slots inside a tile.  The kernel that walks the plan reads, per slot, the
@@ -490,7 +545,11 @@ int plan_scratch_alloc(ffi_plan* p) {
     const bool ok = hipMalloc(&p->d_scratch, kScratchWords * sizeof(unsigned long long)) == hipSuccess &&
                     hipHostMalloc(&p->h_scratch, kScratchWords * sizeof(unsigned long long)) == hipSuccess &&
                     hipEventCreateWithFlags(&p->fp_done, hipEventDisableTiming) == hipSuccess &&
-                    hipMemset(p->d_scratch, 0, kScratchWords * sizeof(unsigned long long)) == hipSuccess;
+                    hipMemset(p->d_scratch, 0, kScratchWords * sizeof(unsigned long long)) == hipSuccess &&
+                    hipMalloc(&p->d_guard, 8 * sizeof(unsigned long long)) == hipSuccess &&
+                    hipHostMalloc(&p->h_guard, 8 * sizeof(unsigned long long)) == hipSuccess &&
+                    hipEventCreateWithFlags(&p->guard_done, hipEventDisableTiming) == hipSuccess &&
+                    hipMemset(p->d_guard, 0, 8 * sizeof(unsigned long long)) == hipSuccess;
     if (!ok) {
         (void)hipGetLastError();
         return FFI_ERR_OUT_OF_MEMORY;
@@ -529,7 +588,32 @@ int plan_fingerprint(ffi_plan* p, const int32_t* lookup, hipStream_t s, unsigned
     return plan_fingerprint_end(p, out, bad_ids);
 }
 
+namespace {
+int plan_build_arrays(ffi_plan* p, const int32_t* lookup, hipStream_t s, unsigned long long* fp_out);
+}
+
+// On failure the plan is left without arrays and without a lookup: it matches no cache key and
+// launch_input_grad refuses it.
 int plan_build(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
+    unsigned long long fp = 0;
+    const int st = plan_build_arrays(p, lookup, s, &fp);
+    if (st != FFI_OK) {
+        free_arrays(p);
+        p->lookup = nullptr;
+        p->fingerprint = ~0ull;
+        return st;
+    }
+    p->lookup = lookup;
+    p->fingerprint = fp;
+    // what the device-side check compares with; the build has synchronised, no check of this plan is in flight
+    const unsigned long long guard_init[8] = {0, 0, 0, fp, 1, fp, 0, 0};
+    FFI_HIP_TRY(hipMemcpy(p->d_guard, guard_init, sizeof(guard_init), hipMemcpyHostToDevice));
+    p->guard_pending = false;
+    return FFI_OK;
+}
+
+namespace {
+int plan_build_arrays(ffi_plan* p, const int32_t* lookup, hipStream_t s, unsigned long long* fp_out) {
     unsigned long long fp = 0, bad = 0;
     FFI_TRY(plan_fingerprint(p, lookup, s, &fp, &bad));
     if (bad != 0) return FFI_ERR_BAD_LOOKUP;   // also keeps the build kernels' LDS counters in range
@@ -552,8 +636,35 @@ int plan_build(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
         int st = build_arranged(p, lookup, s);
         if (st != FFI_OK) { free_arrays(p); return st; }
     }
-    p->lookup = lookup;
-    p->fingerprint = fp;
+    *fp_out = fp;
+    return FFI_OK;
+}
+}  // namespace
+
+int plan_guard_enqueue(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
+    // a check of this plan still running on another stream shares the accumulators: order the two
+    if (p->guard_pending && p->guard_stream != s) FFI_HIP_TRY(hipStreamWaitEvent(s, p->guard_done, 0));
+    const size_t total = (size_t)p->L * p->K;
+    const unsigned blocks = (unsigned)std::min<size_t>((total / 4 + kBlock - 1) / kBlock + 1, kFingerprintBlocks);
+    hipLaunchKernelGGL(fingerprint_guard_kernel, dim3(blocks), dim3(kBlock), 0, s, lookup, total, (unsigned)p->N, p->d_guard);
+    FFI_HIP_TRY(hipGetLastError());
+    FFI_HIP_TRY(hipMemcpyAsync(p->h_guard, p->d_guard + kGuardVerdict, 3 * sizeof(unsigned long long), hipMemcpyDeviceToHost, s));
+    FFI_HIP_TRY(hipEventRecord(p->guard_done, s));
+    p->guard_pending = true;
+    p->guard_stream = s;
+    return FFI_OK;
+}
+
+int plan_guard_poll(ffi_plan* p, bool* seen, bool* current, unsigned long long* bad_ids) {
+    *seen = false;
+    if (!p->guard_pending) return FFI_OK;
+    const hipError_t e = hipEventQuery(p->guard_done);
+    if (e == hipErrorNotReady) { (void)hipGetLastError(); return FFI_OK; }
+    if (e != hipSuccess) return hip_fail(e);
+    p->guard_pending = false;
+    *seen = true;
+    *current = p->h_guard[0] != 0;
+    *bad_ids = p->h_guard[2];
     return FFI_OK;
 }
 
@@ -563,7 +674,11 @@ void plan_free(ffi_plan* p) {
     if (p->d_scratch) (void)hipFree(p->d_scratch);
     if (p->h_scratch) (void)hipHostFree(p->h_scratch);
     if (p->fp_done) (void)hipEventDestroy(p->fp_done);
+    if (p->d_guard) (void)hipFree(p->d_guard);
+    if (p->h_guard) (void)hipHostFree(p->h_guard);
+    if (p->guard_done) (void)hipEventDestroy(p->guard_done);
     p->d_scratch = nullptr; p->h_scratch = nullptr; p->fp_done = nullptr;
+    p->d_guard = nullptr; p->h_guard = nullptr; p->guard_done = nullptr; p->guard_pending = false;
 }
 
 }  // namespace ffi

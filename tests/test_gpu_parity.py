@@ -302,9 +302,103 @@ def test_in_place_rewiring_is_picked_up(ffi):
     lookup2 = lookup.copy()
     lookup2[rows, cols] = rng.integers(0, N, 500)
     dl.copy_(dev(lookup2))                              # in place: data_ptr unchanged
-    after = run()
+    after = run()                                       # served by the kernels that recompute from the lookup
     assert rel_err(after, oracle.input_grad(x, lookup2, w, g)) <= GRAD_RTOL
     assert not np.array_equal(before, after)
+    rebuilt = run()                                     # the host has seen the verdict: the plan is rebuilt
+    assert rel_err(rebuilt, oracle.input_grad(x, lookup2, w, g)) <= GRAD_RTOL
+    assert np.array_equal(rebuilt, run())               # plan-driven again: bit-identical from call to call
+
+
+@pytest.mark.parametrize("transposed", [False, True])
+def test_backward_after_in_place_rewiring_without_host_wait(ffi, transposed):
+    # both gradients of ffi_backward_f32 / ffi_backward_bias_f32 right after the lookup changed under the cached plan,
+    # with no synchronisation between the calls (the verdict of the device-side check is all the kernels have)
+    B, N, L, K = 40, 200, 5000, 32
+    x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=77)
+    xin = np.ascontiguousarray(x.T) if transposed else x
+    dx, dl, dw, dg = dev(xin), dev(lookup), dev(w), dev(g)
+    lib = ffi._lib.lib()
+    gx, gw, gb = torch.empty_like(dx), torch.empty_like(dw), torch.empty(L, device="cuda")
+
+    def call():
+        ffi._lib.check(lib.ffi_backward_bias_f32(dx.data_ptr(), dl.data_ptr(), dw.data_ptr(), dg.data_ptr(), gx.data_ptr(),
+                                                  gw.data_ptr(), gb.data_ptr(), B, N, L, K, int(transposed), stream()))
+
+    call()
+    rng = np.random.default_rng(5)
+    lookup2 = lookup.copy()
+    lookup2[rng.integers(0, L, 800), rng.integers(0, K, 800)] = rng.integers(0, N, 800)
+    dl.copy_(dev(lookup2), non_blocking=True)
+    for _ in range(3):                                  # fallback kernels, then (whenever the host notices) a rebuilt plan
+        gx.fill_(float("nan")); gw.fill_(float("nan")); gb.fill_(float("nan"))
+        call()
+        ref_gx, ref_gw = oracle.backward(xin, lookup2, w, g, transposed=transposed)
+        torch.cuda.synchronize()
+        assert rel_err(gx.cpu().numpy(), ref_gx) <= GRAD_RTOL
+        assert rel_err(gw.cpu().numpy(), ref_gw) <= GRAD_RTOL
+        assert rel_err(gb.cpu().numpy(), g.sum(axis=0)) <= GRAD_RTOL
+
+
+def test_stateless_backward_does_not_wait_for_the_device(ffi):
+    # steady state: a call only enqueues (tfsparse/cc/kernels/backward.cu:59-64 never waits either); calls on two
+    # streams with two layers are enqueued back to back while the device is still busy with the first
+    B, N, L, K = 128, 768, 200_000, 32
+    lib = ffi._lib.lib()
+    rng = np.random.default_rng(0)
+    layers = []
+    for i in range(2):
+        x = dev(rng.standard_normal((N, B)).astype(np.float32))
+        lk = dev(rng.integers(0, N, (L, K)).astype(np.int32))
+        w = dev(rng.standard_normal((L, K)).astype(np.float32))
+        g = dev(rng.standard_normal((B, L)).astype(np.float32))
+        layers.append((x, lk, w, g, torch.empty_like(x), torch.empty_like(w), torch.cuda.Stream()))
+    torch.cuda.synchronize()
+
+    def enqueue(rounds):
+        for _ in range(rounds):
+            for x, lk, w, g, gx, gw, st in layers:
+                ffi._lib.check(lib.ffi_backward_f32(x.data_ptr(), lk.data_ptr(), w.data_ptr(), g.data_ptr(), gx.data_ptr(),
+                                                     gw.data_ptr(), B, N, L, K, 1, st.cuda_stream))
+
+    enqueue(2)                                          # plans built (that does synchronise), verdicts seen
+    torch.cuda.synchronize()
+    import time
+    t0 = time.perf_counter()
+    enqueue(20)
+    t_host = time.perf_counter() - t0
+    torch.cuda.synchronize()
+    t_all = time.perf_counter() - t0
+    assert t_host < 0.5 * t_all, f"enqueueing took {t_host * 1e3:.2f} ms of {t_all * 1e3:.2f} ms: the calls waited for the device"
+    for x, lk, w, g, gx, gw, st in layers:
+        a = [t.cpu().numpy() for t in (x, lk, w, g)]
+        ref_gx, ref_gw = oracle.backward(*a, transposed=True)
+        assert rel_err(gx.cpu().numpy(), ref_gx) <= GRAD_RTOL
+        assert rel_err(gw.cpu().numpy(), ref_gw) <= GRAD_RTOL
+
+
+def test_plan_is_unusable_after_a_failed_refresh(ffi):
+    # a rebuild that fails (here: an id out of range) leaves a plan without arrays; calls through it are refused
+    # with a status instead of walking freed memory
+    B, N, L, K = 16, 64, 1000, 8
+    x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=3)
+    dl, dw, dg = dev(lookup), dev(w), dev(g)
+    lib = ffi._lib.lib()
+    plan = ctypes.c_void_p()
+    ffi._lib.check(lib.ffi_plan_create(dl.data_ptr(), L, K, N, B, stream(), ctypes.byref(plan)))
+    try:
+        bad = lookup.copy()
+        bad[7, 3] = N + 5
+        dbad = dev(bad)
+        assert lib.ffi_plan_refresh(plan, dbad.data_ptr(), stream()) == -6
+        gx = torch.zeros((B, N), device="cuda")
+        assert lib.ffi_input_grad_planned_f32(plan, dw.data_ptr(), dg.data_ptr(), gx.data_ptr(), B, 0, stream()) == -8
+        ffi._lib.check(lib.ffi_plan_refresh(plan, dl.data_ptr(), stream()))          # a good lookup revives it
+        ffi._lib.check(lib.ffi_input_grad_planned_f32(plan, dw.data_ptr(), dg.data_ptr(), gx.data_ptr(), B, 0, stream()))
+        torch.cuda.synchronize()
+        assert rel_err(gx.cpu().numpy(), oracle.input_grad(x, lookup, w, g)) <= GRAD_RTOL
+    finally:
+        lib.ffi_plan_destroy(plan)
 
 
 def test_explicit_plan_matches_cached_path(ffi):
