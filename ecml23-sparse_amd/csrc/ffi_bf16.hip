@@ -373,12 +373,54 @@ __global__ __launch_bounds__(256) void topk_init_kernel(int* __restrict__ count,
     for (size_t e = i; e < n; e += (size_t)gridDim.x * 256) cand_idx[e] = -1;
 }
 
-// a sample whose candidates did not fit its list gets no answer: labels -2, scores NaN
-__global__ __launch_bounds__(256) void topk_overflow_kernel(const int* __restrict__ count, int cap, int B, int k,
-                                                            float* __restrict__ values, int* __restrict__ indices) {
-    const int b = blockIdx.x * 256 + threadIdx.x;
-    if (b >= B || count[b] <= cap) return;
-    for (int s = 0; s < k; ++s) { values[(size_t)b * k + s] = __builtin_nanf(""); indices[(size_t)b * k + s] = -2; }
+// A sample whose candidates did not fit its list (thousands of labels tied at the top: an all-zero feature row under a
+// constant bias, say) is answered the slow way, still on the device and without a host wait: one workgroup scans the
+// sample's whole row -- the stored scores, or, where the forward pass stored none, scores recomputed with that pass's own
+// order of additions (k ascending, bias last) -- every thread keeping the best eight of its share, then the lists are
+// merged under the same (score, lower label) order.  Workgroups of samples whose list was complete return at once.
+__global__ __launch_bounds__(256) void topk_overflow_rows_kernel(const int* __restrict__ count, int cap, int k, const float* __restrict__ scores,
+                                                                 const float* __restrict__ xT, const int32_t* __restrict__ idx,
+                                                                 const float* __restrict__ w, const float* __restrict__ bias, int B, int N,
+                                                                 int L, int K, float* __restrict__ values, int* __restrict__ indices) {
+    const int b = blockIdx.x;
+    if (count[b] <= cap) return;
+    float vals[kTopMax];
+    int ids[kTopMax];
+#pragma unroll
+    for (int s = 0; s < kTopMax; ++s) { vals[s] = -__builtin_inff(); ids[s] = 0x7fffffff; }
+    for (int j = threadIdx.x; j < L; j += 256) {          // ascending labels per thread: ties keep the lower label
+        float v;
+        if (scores != nullptr) {
+            v = scores[(size_t)b * L + j];
+        } else {
+            v = 0.f;
+            for (int c = 0; c < K; ++c) {
+                const unsigned id = (unsigned)idx[(size_t)j * K + c];
+                v = fmaf(w[(size_t)j * K + c], xT[(size_t)(id < (unsigned)N ? id : 0u) * B + b], v);
+            }
+            if (bias != nullptr) v += bias[j];
+        }
+        if (better(v, j, vals[kTopMax - 1], ids[kTopMax - 1])) topk_insert_ordered(vals, ids, v, j);
+    }
+    float ov;
+    int oi;
+    wave_topk(vals, ids, ov, oi);
+    __shared__ float lv[4][kTopMax];
+    __shared__ int li[4][kTopMax];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane < kTopMax) { lv[wave][lane] = ov; li[wave][lane] = oi; }
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int s = 0; s < kTopMax; ++s) {
+        vals[s] = lane < 4 ? lv[lane][s] : -__builtin_inff();
+        ids[s] = lane < 4 ? li[lane][s] : 0x7fffffff;
+    }
+    wave_topk(vals, ids, ov, oi);
+    if (lane < k) {
+        values[(size_t)b * k + lane] = ov;
+        indices[(size_t)b * k + lane] = oi != 0x7fffffff ? oi : -1;
+    }
 }
 
 // sample[b][i] = scores[b][(i * L) / S]: evenly spaced labels whose k-th best score is a threshold that at least k
@@ -474,9 +516,10 @@ int launch_topk_candidates_init(int* count, int* cand_idx, int B, int cap, hipSt
 }
 
 int launch_topk_candidates_select(const float* cand_val, const int* cand_idx, const int* count, int B, int cap, int k,
-                                  float* values, int32_t* indices, hipStream_t s) {
+                                  float* values, int32_t* indices, hipStream_t s, const TopkRowSource& src) {
     FFI_TRY(launch_topk_merge(cand_val, cand_idx, B, cap / 8, k, values, indices, s));
-    hipLaunchKernelGGL(topk_overflow_kernel, dim3((B + 255) / 256), dim3(256), 0, s, count, cap, B, k, values, indices);
+    hipLaunchKernelGGL(topk_overflow_rows_kernel, dim3(B), dim3(256), 0, s, count, cap, k, src.scores, src.xT, src.idx, src.w, src.bias,
+                       B, src.N, src.L, src.K, values, indices);
     FFI_HIP_TRY(hipGetLastError());
     return FFI_OK;
 }
@@ -487,7 +530,7 @@ int launch_topk_f32(const float* scores, int B, int L, int k, float* values, int
     if (L <= 16 * kTopkRowSample) return topk_by_lists(scores, B, L, k, values, indices, s);
     // Long rows: a sample of every row fixes a threshold that k of its labels reach (the k-th best of the sample), one
     // streaming pass collects the few scores at or above it, and the k best of those are the answer.  Exact; a row
-    // with more than kTopkCap scores at or above its threshold (thousands of ties) gets labels -2 instead.
+    // with more than kTopkCap scores at or above its threshold (thousands of ties) is scanned whole by one workgroup.
     const int S = kTopkRowSample;
     const size_t cand = (size_t)B * kTopkCap;
     unsigned char* ws = nullptr;
@@ -508,7 +551,9 @@ int launch_topk_f32(const float* scores, int B, int L, int k, float* values, int
     hipLaunchKernelGGL(topk_filter_kernel, dim3(splits, B), dim3(256), 0, s, scores, L, per, tau_val + (k - 1), k, count, cand_val,
                        cand_idx, kTopkCap);
     FFI_HIP_TRY(hipGetLastError());
-    return launch_topk_candidates_select(cand_val, cand_idx, count, B, kTopkCap, k, values, indices, s);
+    TopkRowSource src;
+    src.scores = scores; src.L = L;
+    return launch_topk_candidates_select(cand_val, cand_idx, count, B, kTopkCap, k, values, indices, s, src);
 }
 
 }  // namespace ffi

@@ -427,7 +427,11 @@ int forward_tiles(const float* x, const int32_t* idx, const float* w, const floa
     else if (epi == kEpiLossGradAndScores) FFI_TRY(launch_lane32_any<kEpiLossGradAndScores>(vec4, topk, xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds_topk, fl, ft, s));
     else FFI_TRY(launch_lane32_any<kEpiNone>(vec4, topk, xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds_topk, fl, ft, s));
     if (topk) {
-        FFI_TRY(launch_topk_candidates_select(ft.cand_val, ft.cand_idx, count, d.B, kTopkCap, tk->k, tk->values, tk->indices, s));
+        // (a sample with more candidates than its list holds: its row once more, from the score matrix if there is one)
+        TopkRowSource src;
+        if (epi == kEpiScores || epi == kEpiLossGradAndScores) src.scores = out;
+        src.xT = xT; src.idx = idx; src.w = w; src.bias = bias; src.N = d.N; src.L = d.L; src.K = d.K;
+        FFI_TRY(launch_topk_candidates_select(ft.cand_val, ft.cand_idx, count, d.B, kTopkCap, tk->k, tk->values, tk->indices, s, src));
     }
     if (epi != kEpiLossGrad && epi != kEpiLossGradAndScores) return FFI_OK;
     // the listed label positions: from the score matrix when it was written, else recomputed from x ([N,B] here)

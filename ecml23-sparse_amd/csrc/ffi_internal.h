@@ -121,9 +121,19 @@ int launch_forward_topk(const float* x, const int32_t* idx, const float* w, cons
 // Candidate lists for a threshold-based top-k: count[B] appended entries, cand_val / cand_idx [B][kTopkCap].
 constexpr int kTopkCap = 8192;          // candidate slots per sample (a multiple of 8)
 int launch_topk_candidates_init(int* count, int* cand_idx, int B, int cap, hipStream_t s);
-// the k best candidates of every sample; a sample whose count exceeds cap gets labels -2 and NaN scores
+// Where the scores of a whole row come from when a sample's candidate list has overflowed: the score matrix [B,L],
+// or (scores == null) the layer itself, features as xT [N][B].
+struct TopkRowSource {
+    const float* scores = nullptr;
+    const float* xT = nullptr;
+    const int32_t* idx = nullptr;
+    const float* w = nullptr;
+    const float* bias = nullptr;
+    int N = 0, L = 0, K = 0;
+};
+// the k best candidates of every sample; a sample whose count exceeds cap is answered from its whole row (src)
 int launch_topk_candidates_select(const float* cand_val, const int* cand_idx, const int* count, int B, int cap, int k,
-                                  float* values, int32_t* indices, hipStream_t s);
+                                  float* values, int32_t* indices, hipStream_t s, const TopkRowSource& src);
 // the k best of nlists * 8 (score, label) candidates per sample (label -1 = empty slot)
 int launch_topk_merge(const float* part_val, const int* part_idx, int B, int nlists, int k, float* values, int32_t* indices,
                       hipStream_t s);

@@ -224,6 +224,9 @@ class StratifiedRewireLayer(StratifiedRewireLayerV2):
     def __init__(self, units: int, input_dim: int, **kwargs):
         kwargs["arrange"] = False          # the order inside a unit is this layer's own
         super().__init__(units, input_dim, **kwargs)
+        # sorted from construction on, as build() leaves the reference's kernel (sparse/layer.py:197: _update_sparse_kernel
+        # runs tf.sparse.reorder)
+        self._sort_rows([])
 
     @torch.no_grad()
     def _sort_rows(self, other_vars):

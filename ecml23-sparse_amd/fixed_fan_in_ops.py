@@ -285,7 +285,7 @@ def backward_sparse(features, lookup, weights, out_grad, nz_words=None, max_dens
     ``nz_words`` has a bit set (``metrics.forward_loss(..., skip_zero_stores=True)``); the call may then
     write zeros into the rest of it.  ``decide_from_previous``: choose between sparse and dense kernels
     from the count of non-zeros the previous call of this shape on the stream found, so that the host
-    does not wait (same results; the first call of a shape still waits).  Returns ``(feature_grad or None, weight_grad,
+    does not wait (same results up to summation order; the first call of a shape still waits).  Returns ``(feature_grad or None, weight_grad,
     bias_grad or None, sparse_kernels_ran)``."""
     import ctypes
 
@@ -374,7 +374,7 @@ def fan_in_sparse_topk(features, lookup, weights, bias=None, k=5, transposed=Fal
     """``(values [B,k], labels [B,k] int32)`` of the k best fp32 scores per sample (best first, equal scores
     by ascending label), and the score matrix as a third result if ``want_scores``.  Without
     ``want_scores`` the ``[B,L]`` matrix is never written.  A sample whose candidate list overflows (see
-    the C header) gets labels -2."""
+    the C header) is answered from a scan of its whole row."""
     batch, num_features, num_units, fan_in = _check_inputs(features, lookup, weights, transposed)
     if bias is not None:
         _check_bias(bias, weights, num_units)

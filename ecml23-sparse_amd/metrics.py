@@ -107,8 +107,11 @@ def forward_loss(features, lookup, weights, bias, y_true, kind, grad_scale=None,
 
 
 def _scaled(out_grad, upstream):
-    # the usual upstream gradient of a scalar loss is exactly 1: the stored gradient is then used as it is
-    if upstream.numel() == 1 and float(upstream) == 1.0:
+    # multiplied on the device, whatever the factor: reading it on the host would make every training step wait
+    # for the GPU (a host-side scalar equal to 1 is the one case that can be skipped without looking at the device)
+    if not isinstance(upstream, torch.Tensor):
+        return out_grad if float(upstream) == 1.0 else out_grad * upstream
+    if upstream.device.type == "cpu" and upstream.numel() == 1 and float(upstream) == 1.0:
         return out_grad
     return out_grad * upstream
 

@@ -148,7 +148,8 @@ int ffi_weight_grad_planned_f32(const ffi_plan* plan, const float* features, con
 int ffi_arrange_connections_f32(int32_t* lookup, float* const* arrays, int n_arrays,
                                 int64_t num_units, int64_t fan_in, ffi_stream_t stream);
 
-/* Drops every cached plan and workspace of the calling thread's current device. */
+/* Drops every cached plan and workspace of the calling thread's current device.  Waits for the device first; no other
+   call of this library may be in flight on that device (from another thread) while it runs. */
 int ffi_cache_clear(void);
 /* Device bytes currently held by the library (plans + workspaces) on the current device. */
 size_t ffi_cache_bytes(void);
@@ -264,7 +265,9 @@ int ffi_forward_loss_f32(const float* features, const int32_t* lookup, const flo
  * first and fixes, per sample, a threshold that k labels are known to reach; the forward kernel then appends
  * every score at or above its sample's threshold to a candidate list (a tiny share of all labels), and the k
  * best candidates are selected.  The result is exact.  A sample whose candidates overflow its list (8192 slots;
- * e.g. thousands of labels tied with the k-th score) gets labels -2 and NaN scores instead.
+ * e.g. thousands of labels tied with the k-th score, as an all-zero feature row gives) is answered from a scan of its
+ * whole row instead (on the device, without a host wait; slower for that sample only), so ties still resolve to the
+ * lower labels as tf.nn.top_k resolves them.
  * ffi_forward_loss_topk_f32 is ffi_forward_loss_f32 with the same top-k of the scores as a by-product: what a
  * training step needs for the loss, the backward pass and the P@k metrics (sparse/metrics.py:31-71) without
  * the score matrix ever being stored.  No counterpart in the reference.
@@ -301,7 +304,10 @@ int ffi_forward_loss_topk_f32(const float* features, const int32_t* lookup, cons
  *   sparse_path_taken  HOST int, may be NULL: 1 if the sparse kernels ran, 0 if the dense ones did.
  * Synchronises `stream` once (the host reads the number of set bits), except as described under flags.  The sparse input gradient
  * covers num_features <= 4096; wider inputs take the dense input-gradient kernels.  It accumulates
- * with LDS float adds issued in a fixed order, no global atomics.
+ * with LDS float adds, no global atomics: where two lanes of one instruction add to the same column the
+ * hardware picks the order, so its results are reproducible up to summation order only (the dense kernels
+ * are bit-reproducible), and FFI_SPARSE_DECIDE_FROM_PREVIOUS, which picks sparse or dense kernels from an
+ * earlier call's count, can change the summation order of identical inputs with the call history.
  */
 enum ffi_sparse_flags {
     FFI_SPARSE_GRAD_IS_PARTIAL = 1,

@@ -229,15 +229,44 @@ def test_fp32_topk_argument_errors(ffi):
         ffi.fan_in_sparse_topk(x.cpu(), lookup.cpu(), w.cpu(), None, k=1)
 
 
-def test_fp32_topk_overflow_is_reported(ffi):
-    # every label ties with the best score: no list of 8192 candidates can hold them, the sample gets -2
+def test_fp32_topk_when_a_candidate_list_overflows(ffi):
+    # every label ties with the best score: no list of 8192 candidates can hold them; the sample is then answered from a
+    # scan of its whole row, and ties go to the lower labels as tf.nn.top_k (sparse/metrics.py:19) resolves them
     B, N, L, K = 3, 16, 20000, 2
     x = torch.ones((B, N), device="cuda")
     lookup = torch.zeros((L, K), dtype=torch.int32, device="cuda")
     w = torch.ones((L, K), device="cuda")
-    v, i = ffi.fan_in_sparse_topk(x, lookup, w, None, k=3)
+    for want_scores in (False, True):
+        out = ffi.fan_in_sparse_topk(x, lookup, w, None, k=3, want_scores=want_scores)
+        torch.cuda.synchronize()
+        v, i = out[0], out[1]
+        assert i.cpu().numpy().tolist() == [[0, 1, 2]] * B
+        assert bool((v == 2.0).all())
+
+
+def test_fp32_topk_of_an_all_zero_feature_row(ffi):
+    # what validation data does hold: a sample without features.  Its scores are the bias (zero-initialised: all labels
+    # tie), while the other samples of the batch take the fast path.  ffi_topk_f32 on the stored scores (L > 65536:
+    # the threshold filter) and the forward pass without a score matrix must both answer labels 0..k-1 for it
+    B, N, L, K, k = 5, 96, 70000, 8, 5
+    rng = np.random.default_rng(8)
+    x = np.abs(rng.standard_normal((B, N))).astype(np.float32)
+    x[2] = 0.0
+    lookup = rng.integers(0, N, size=(L, K)).astype(np.int32)
+    w = rng.standard_normal((L, K)).astype(np.float32)
+    bias = np.zeros(L, dtype=np.float32)
+    dev = lambda a: torch.from_numpy(a).cuda()  # noqa: E731
+    v1, i1, scores = ffi.fan_in_sparse_topk(dev(x), dev(lookup), dev(w), dev(bias), k=k, want_scores=True)
+    v2, i2 = ffi.fan_in_sparse_topk(dev(x), dev(lookup), dev(w), dev(bias), k=k)
+    v3 = torch.empty((B, k), device="cuda")
+    i3 = torch.empty((B, k), dtype=torch.int32, device="cuda")
+    ffi._lib.check(ffi._lib.lib().ffi_topk_f32(scores.data_ptr(), B, L, k, v3.data_ptr(), i3.data_ptr(),
+                                              torch.cuda.current_stream().cuda_stream))
     torch.cuda.synchronize()
-    assert bool((i == -2).all()) and bool(torch.isnan(v).all())
+    ref_v, ref_i = oracle.topk(scores.cpu().numpy(), k)
+    assert ref_i[2].tolist() == list(range(k))
+    for v, i in ((v1, i1), (v2, i2), (v3, i3)):
+        assert np.array_equal(i.cpu().numpy(), ref_i) and np.array_equal(v.cpu().numpy(), ref_v)
 
 
 def test_inference_config_full_size(ffi):

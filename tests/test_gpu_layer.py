@@ -382,6 +382,8 @@ def test_first_generation_layer_keeps_rows_sorted(ffi):
     units, N, K = 60, 90, 8
     layer = ffi.StratifiedRewireLayer(units, N, connections=units * K, rewire_selector=ffi.FixedFractionSelector(0.2),
                                       generator=gen)
+    idx0 = layer.kernel_indices.view(units, K)
+    assert bool((idx0[:, 1:] >= idx0[:, :-1]).all())                                  # sorted right after construction
     w_before = layer.kernel_weights.detach().clone()
     idx_before = layer.kernel_indices.clone()
     tag = torch.arange(units * K, device="cuda", dtype=torch.float32) + 1.0          # follows every connection around
