@@ -99,3 +99,42 @@ def test_layer_constructor_arithmetic():
         L(10, 8, sparsity=1.5, device="cpu")
     with pytest.raises(RuntimeError):          # the product path needs the GPU: no CPU fallback
         layer(torch.zeros(2, 64))
+
+
+def test_tensorflow_shim_declares_the_reference_ops():
+    # The op library a maintainer builds against ROCm TensorFlow (csrc/tf/ffi_tf_ops.cc) must declare the four ops
+    # exactly as tfsparse/cc/ops/fixed_fan_in_ops.cpp:55-93 does (names, attrs, inputs, outputs: the Python binding
+    # sparse/ops/fixed_fan_in_ops.py:9-40 is generated from them) and register the eight GPU kernels of
+    # tfsparse/cc/kernels/register.cpp:81-82,90-91,99-100,108-109.  TensorFlow is not in this image: the file is checked as text.
+    import os
+    import re
+
+    from conftest import ROOT
+    src = open(os.path.join(ROOT, "ecml23-sparse_amd", "csrc", "tf", "ffi_tf_ops.cc")).read()
+    code = re.sub(r"//[^\n]*", "", src)
+    fwd = re.search(r"#define FFI_DECLARE_FORWARD_OP\(NAME, TRANSPOSED\)(.*?)\n#define", code, re.S).group(1)
+    grad = re.search(r"#define FFI_DECLARE_GRAD_OP\(NAME, TRANSPOSED\)(.*?)\n\n", code, re.S).group(1)
+
+    def parts(text):
+        return (re.findall(r'\.Attr\("([^"]+)"\)', text), re.findall(r'\.Input\("([^"]+)"\)', text),
+                re.findall(r'\.Output\("([^"]+)"\)', text))
+
+    assert parts(fwd) == (["T: type", "I: type"], ["features: T", "lookup: I", "weights: T"], ["result: T"])
+    assert parts(grad) == (["T: type", "I: type"], ["features: T", "lookup: I", "weights: T", "output: T"],
+                           ["feature_grad: T", "weight_grad: T"])
+    declared = re.findall(r'FFI_DECLARE_(FORWARD|GRAD)_OP\("(\w+)", (true|false)\);', code)
+    assert declared == [("FORWARD", "FanInSparseMatmul", "false"), ("FORWARD", "FanInSparseMatmulTp", "true"),
+                        ("GRAD", "FanInSparseMatmulGrad", "false"), ("GRAD", "FanInSparseMatmulGradTp", "true")]
+    kernels = re.findall(r'FFI_REGISTER_GPU\("(\w+)", (\w+), (\w+), (true|false)\);', code)
+    assert len(kernels) == 8
+    for op, transposed in (("FanInSparseMatmul", "false"), ("FanInSparseMatmulTp", "true"),
+                           ("FanInSparseMatmulGrad", "false"), ("FanInSparseMatmulGradTp", "true")):
+        cls = "FanInSparseMatmulGradGpuOp" if "Grad" in op else "FanInSparseMatmulGpuOp"
+        for ids in ("int32", "uint32"):
+            assert (op, cls, ids, transposed) in kernels
+    assert "DEVICE_GPU" in code and 'TypeConstraint<float>("T")' in code
+    # no arithmetic in the shim: its Compute bodies end in exactly one C-ABI call each
+    assert code.count("ffi_forward_f32(") == 1 and code.count("ffi_backward_f32(") == 1
+    # and the default CMake build does not depend on TensorFlow
+    cm = open(os.path.join(ROOT, "ecml23-sparse_amd", "csrc", "CMakeLists.txt")).read()
+    assert "if(FFI_TF_INCLUDE_DIR AND FFI_TF_LIBRARY)" in cm and "tf/ffi_tf_ops.cc" in cm
