@@ -20,13 +20,13 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0        # MI355X published HBM3E peak
+# the other two resources every multiply-add of this path uses (published figures): the gathered operand comes out
+# of LDS (4 bytes per multiply-add; 256 bytes per clock per CU, 256 CUs, 2.4 GHz) and the multiply-add itself is a
+# plain FP32 FMA (packed FP32 forms are not used: half of the 157.3 TFLOP/s vector peak)
+LDS_PEAK_GBPS = 256 * 256 * 2.4
+FP32_FMA_PEAK_TFLOPS = 157.3 / 2
 
-# HBM bytes per launch of each pass, from rocprofv3 --pmc FETCH_SIZE (x2.00) and WRITE_SIZE (x1.00)
-# runs of this file (the factors are what the same counters read for a plain copy kernel of known
-# size); the summary with the commands is profiles/ffi_c2_counters.txt.  None where not measured.
-MEASURED_TRAFFIC_BYTES = {
-    "c2": {"forward": 556.5e6, "weight_grad": 647.1e6, "input_grad": 859.2e6},
-}
+PROFILE_DIR = os.path.join(ROOT, "profiles")
 
 # GPU kernels behind each pass (one C-ABI call)
 PASS_KERNELS = {
@@ -34,6 +34,27 @@ PASS_KERNELS = {
     "weight_grad": "wgrad_arranged_kernel",
     "input_grad": "igrad_permute_weights_kernel + igrad_tile_kernel + igrad_reduce_kernel",
 }
+WIDE_PASS_KERNELS = {
+    "forward": "fwd_wide_kernel",
+    "weight_grad": "wgrad_wide_kernel",
+    "input_grad": "transpose_kernel + igrad_wide_kernel",
+}
+
+
+def measured_traffic(config_name):
+    """HBM bytes per launch of each pass, read from the committed counter summary profiles/ffi_<config>_counters.txt
+    (lines `traffic_bytes <pass> <bytes>`; rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file, scaled by what the
+    same counters read for a plain copy kernel of known size).  Returns ({pass: bytes}, source) or ({}, None)."""
+    path = os.path.join(PROFILE_DIR, f"ffi_{config_name}_counters.txt")
+    out, stamp = {}, None
+    if os.path.exists(path):
+        for line in open(path):
+            f = line.split()
+            if len(f) >= 3 and f[0] == "traffic_bytes":
+                out[f[1]] = float(f[2])
+            elif len(f) >= 2 and f[0] == "measured_at":
+                stamp = " ".join(f[1:])
+    return out, (f"profiles/{os.path.basename(path)}" + (f" ({stamp})" if stamp else "")) if out else None
 
 
 def parse_args():
@@ -41,7 +62,8 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--config", default="c2", help="workload: c1..c4 (c2 is the headline)")
+    ap.add_argument("--config", default="c2", help="workload: c1..c4 forward + backward in fp32 (c2 is the headline); "
+                                                   "c5 = bf16 forward with top-5 per sample (inference)")
     ap.add_argument("--layout", default="nb", choices=["nb", "bn"],
                     help="features as [N,B] (the production 'Tp' op) or [B,N]")
     ap.add_argument("--seed", type=int, default=42)
@@ -74,31 +96,127 @@ def time_kernel(fn, stream, iters):
     return start.elapsed_time(stop) / iters
 
 
-def cpu_baseline(cfg, layout_tp, labels, seed):
-    """Times the CPU oracle (restatement of the reference's CPU kernels) on a bounded sample."""
+def cpu_baseline(cfg, layout_tp, arrays):
+    """Times the CPU oracle (restatement of the reference's CPU kernels) on a bounded sample: `arrays` are the first
+    labels of the very tensors the GPU leg runs on.  Returns the report and the oracle's three results."""
     import oracle
-    from ecml23_sparse_amd import synth
 
     threads = oracle.default_threads()
-    t = synth.make_inputs(cfg, seed=seed, device="cpu", transposed=layout_tp, num_units=labels)
-    x, lookup, w, g = (t[k].numpy() for k in ("features", "lookup", "weights", "out_grad"))
+    x, lookup, w, g = arrays
+    labels = lookup.shape[0]
     oracle.forward(x[:, :], lookup[:1024], w[:1024], transposed=layout_tp, threads=threads)   # warm-up
-    best = None
+    best, results = None, None
     for _ in range(2):
         t0 = time.perf_counter()
-        oracle.forward(x, lookup, w, transposed=layout_tp, threads=threads)
-        oracle.weight_grad(x, lookup, w, g, transposed=layout_tp, threads=threads)
-        oracle.input_grad(x, lookup, w, g, transposed=layout_tp, threads=threads)
+        out = oracle.forward(x, lookup, w, transposed=layout_tp, threads=threads)
+        gw = oracle.weight_grad(x, lookup, w, g, transposed=layout_tp, threads=threads)
+        gx = oracle.input_grad(x, lookup, w, g, transposed=layout_tp, threads=threads)
         dt = time.perf_counter() - t0
         best = dt if best is None else min(best, dt)
+        results = (out, gx, gw)
     full_time = best * cfg.num_units / labels        # every pass is linear in the label count
-    return {
+    report = {
         "value": cfg.batch / full_time,
         "unit": "samples/s",
         "cores": threads,
         "kind": "port",
-        "sample": f"{labels} of {cfg.num_units} labels (same B, N, K, laws); fwd+gW+gx in {best:.3f} s (best of 2)"
+        "sample": f"{labels} of {cfg.num_units} labels (same B, N, K, same tensors as the GPU leg); fwd+gW+gx in {best:.3f} s (best of 2)"
                   + ("" if labels == cfg.num_units else ", scaled linearly to the full label count"),
+    }
+    return report, results
+
+
+def rel_err(a, ref):
+    import numpy as np
+    denom = float(np.abs(ref).max())
+    return float(np.abs(a.astype(np.float64) - ref).max() / (denom if denom > 0 else 1.0))
+
+
+def parity_check(pkg, arrays, tp, stream, reference=None):
+    """The three passes on a label sample of the workload's own tensors, HIP path against the CPU oracle, before any
+    timing: forward max|a-b|/max|ref| <= 1e-5, gradients <= 1e-4 (the gates of the parity tests)."""
+    import numpy as np
+    import oracle
+    import torch
+
+    x, lookup, w, g = arrays
+    if reference is None:
+        reference = (oracle.forward(x, lookup, w, transposed=tp), oracle.input_grad(x, lookup, w, g, transposed=tp),
+                     oracle.weight_grad(x, lookup, w, g, transposed=tp))
+    L, K = lookup.shape
+    B = g.shape[0]
+    N = x.shape[0] if tp else x.shape[1]
+    dx, dl, dw, dg = (torch.from_numpy(np.ascontiguousarray(a)).cuda() for a in (x, lookup, w, g))
+    out = torch.full((B, L), float("nan"), device="cuda")
+    gx, gw = torch.full_like(dx, float("nan")), torch.full_like(dw, float("nan"))
+    lib, check, sh = pkg._lib.lib(), pkg._lib.check, stream.cuda_stream
+    check(lib.ffi_forward_f32(dx.data_ptr(), dl.data_ptr(), dw.data_ptr(), out.data_ptr(), B, N, L, K, int(tp), sh))
+    check(lib.ffi_backward_f32(dx.data_ptr(), dl.data_ptr(), dw.data_ptr(), dg.data_ptr(), gx.data_ptr(), gw.data_ptr(), B, N, L, K, int(tp), sh))
+    stream.synchronize()
+    errs = {"forward": rel_err(out.cpu().numpy(), reference[0]), "input_grad": rel_err(gx.cpu().numpy(), reference[1]),
+            "weight_grad": rel_err(gw.cpu().numpy(), reference[2])}
+    gates = {"forward": 1e-5, "input_grad": 1e-4, "weight_grad": 1e-4}
+    ok = all(errs[k] <= gates[k] for k in gates)
+    return {"checked_before_timing": True, "labels": int(L), "against": "CPU oracle (oracle/ffi_oracle.c)",
+            "rel_err": {k: float(f"{v:.3e}") for k, v in errs.items()}, "gates": gates, "pass": bool(ok)}
+
+
+def bench_inference(args, pkg, synth, cfg):
+    """c5: bf16 features and weights, fp32 accumulation, top-5 per sample without the score matrix."""
+    import numpy as np
+    import oracle
+    import torch
+
+    t = synth.make_inputs(cfg, seed=args.seed, device="cuda", transposed=True)
+    x, lookup, w = t["features"].to(torch.bfloat16), t["lookup"], t["weights"].to(torch.bfloat16)
+    B, N, L, K = cfg.batch, cfg.num_features, cfg.num_units, cfg.fan_in
+    lib, check = pkg._lib.lib(), pkg._lib.check
+    stream = torch.cuda.current_stream()
+    sh = stream.cuda_stream
+    vals = torch.empty((B, 5), device="cuda")
+    labels = torch.empty((B, 5), dtype=torch.int32, device="cuda")
+
+    def step():
+        check(lib.ffi_forward_topk_bf16(x.data_ptr(), lookup.data_ptr(), w.data_ptr(), vals.data_ptr(), labels.data_ptr(),
+                                        B, N, L, K, 5, 1, sh))
+
+    # parity before timing: the top-5 of 8 samples against the oracle's top-5 of fp32 scores of the same bf16-rounded inputs
+    step()
+    stream.synchronize()
+    rows = 8
+    xs = x[:, :rows].float().cpu().numpy()
+    ref = oracle.forward(np.ascontiguousarray(xs), lookup.cpu().numpy(), w.float().cpu().numpy(), transposed=True)
+    ref_v, ref_i = oracle.topk(ref, 5)
+    got_v, got_i = vals[:rows].cpu().numpy(), labels[:rows].cpu().numpy()
+    same_labels = float((got_i == ref_i).mean())
+    parity = {"checked_before_timing": True, "samples": rows, "against": "CPU oracle on the same bf16-rounded inputs",
+              "rel_err": {"top5_scores": float(f"{rel_err(got_v, ref_v):.3e}")}, "gates": {"top5_scores": 1e-2},
+              "top5_labels_equal": same_labels, "pass": bool(rel_err(got_v, ref_v) <= 1e-2)}
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    kernel_ms = time_kernel(step, stream, max(3, min(args.steps, 20)))
+    alg = 2 * L * K + 4 * L * K + 2 * B * N                  # bf16 W, int32 idx, bf16 x; the scores are never written
+    achieved = alg / (kernel_ms * 1e-3) / 1e9
+    traffic, source = measured_traffic(cfg.name)
+    return {
+        "metric": "ffi_bf16_fwd_top5_samples_per_s", "value": round(B / (ms * 1e-3), 1), "unit": "samples/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"{cfg.name}: FFI layer forward + top-5 per sample, bf16 features and weights with fp32 accumulation, "
+                               f"batch {B}, {N} inputs, {L} labels, fan-in {K} (sorted rows), features [N,B]"},
+        "roofline": {"bound": "hbm", "kernel": "forward pass (fwd_bf16_topk_kernel + topk_merge_kernel)", "achieved": round(achieved, 2),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": traffic.get("forward"), "traffic_source": source, "algorithmic_bytes": alg,
+                     "kernel_ms": {"forward": round(kernel_ms, 4)},
+                     "note": f"the gathers (B*L*K*2 = {B * L * K * 2 / 1e9:.1f} GB per call) are served by L2 / Infinity Cache, which is what bounds this workload"},
+        "parity": parity,
+        "library_bytes": int(lib.ffi_cache_bytes()),
     }
 
 
@@ -214,12 +332,30 @@ def main():
         sys.exit(3)
     torch.cuda.set_device(0)
     cfg = synth.CONFIGS[args.config]
+    if cfg.name == "c5":
+        print(json.dumps(bench_inference(args, pkg, synth, cfg)))
+        return
     tp = args.layout == "nb"
     t = synth.make_inputs(cfg, seed=args.seed, device="cuda", transposed=tp)
     x, lookup, w, g = t["features"], t["lookup"], t["weights"], t["out_grad"]
     B, N, L, K = cfg.batch, cfg.num_features, cfg.num_units, cfg.fan_in
     if args.arranged:
         pkg.arrange_connections(lookup, w)
+    # Parity first, outside the timed region: the HIP path against the CPU oracle on the first labels of these very
+    # tensors (all of them when the CPU baseline's time budget allows: then the input gradient is the full one).
+    # The oracle's run is also the CPU baseline.
+    labels = min(L, args.cpu_labels or max(4096, int(8.0e9 / (B * K))))
+    if args.no_cpu_baseline:
+        labels = min(L, args.cpu_labels or 8192)
+    sample = (x.cpu().numpy(), lookup[:labels].cpu().numpy(), w[:labels].cpu().numpy(),
+              g[:, :labels].contiguous().cpu().numpy())
+    cpu_report, cpu_results = (None, None) if args.no_cpu_baseline else cpu_baseline(cfg, tp, sample)
+    parity = parity_check(pkg, sample, tp, torch.cuda.current_stream(), cpu_results)
+    del sample, cpu_results
+    if not parity["pass"]:
+        print(f"bench.py: parity check failed, nothing is timed: {json.dumps(parity)}", file=sys.stderr)
+        sys.exit(4)
+    pkg._lib.lib().ffi_cache_clear()
     out = torch.empty((B, L), device="cuda")
     gx = torch.empty_like(x)
     gw = torch.empty_like(w)
@@ -266,18 +402,27 @@ def main():
     alg = synth.algorithmic_bytes(cfg)
     dominant = max(kernel_ms, key=kernel_ms.get)
     achieved = alg[dominant] / (kernel_ms[dominant] * 1e-3) / 1e9
+    traffic, traffic_source = measured_traffic(cfg.name)
+    narrow = N <= 1216
+    flops = 2.0 * B * L * K
     roofline = {
         "bound": "hbm",
-        "kernel": f"{dominant} pass ({PASS_KERNELS[dominant]})",
+        "kernel": f"{dominant} pass ({(PASS_KERNELS if narrow else WIDE_PASS_KERNELS)[dominant]})",
         "achieved": round(achieved, 2),
         "peak": HBM_PEAK_GBPS,
         "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBPS, 4),
-        "traffic": MEASURED_TRAFFIC_BYTES.get(cfg.name, {}).get(dominant),
+        "traffic": traffic.get(dominant),
+        "traffic_source": traffic_source,
         "algorithmic_bytes": alg[dominant],
         "kernel_ms": {k: round(v, 4) for k, v in kernel_ms.items()},
         "all_kernels_gbps": {k: round(alg[k] / (v * 1e-3) / 1e9, 1) for k, v in kernel_ms.items()},
         "three_pass_gbps": round(alg["total"] / (sum(kernel_ms.values()) * 1e-3) / 1e9, 1),
+        # what one pass cannot go below on the two other resources it uses for every multiply-add (published peaks):
+        # 4 bytes of LDS reads (narrow inputs: the gathered operand is staged in LDS) and one plain FP32 FMA
+        "other_floors_ms_per_pass": {"lds_gather": round(4.0 * B * L * K / (LDS_PEAK_GBPS * 1e9) * 1e3, 4) if narrow else None,
+                                     "fp32_fma_unpacked": round(flops / (FP32_FMA_PEAK_TFLOPS * 1e12) * 1e3, 4),
+                                     "hbm": round(alg[dominant] / (HBM_PEAK_GBPS * 1e9) * 1e3, 4)},
     }
 
     result = {
@@ -298,12 +443,16 @@ def main():
                                + (", connections of each label reordered by ffi_arrange_connections_f32" if args.arranged else ""),
                    "label_samples_per_s": round(B * L / (ms_per_step * 1e-3), 1)},
         "roofline": roofline,
+        "parity": parity,
+        # device memory the library holds beside the caller's tensors after these steps (cached plan + workspaces),
+        # and what ffi_workspace_bytes() predicts for this shape
+        "library_bytes": int(lib.ffi_cache_bytes()),
+        "library_bytes_estimate": int(lib.ffi_workspace_bytes(B, N, L, K, int(tp), 3)),
     }
     if args.train_step > 0:
         result["train_step"] = train_step(pkg, cfg, x, lookup, w, tp, args.train_step, stream, max(3, min(args.steps, 20)))
-    if not args.no_cpu_baseline:
-        labels = args.cpu_labels or max(4096, min(L, int(8.0e9 / (B * K))))
-        result["cpu_baseline"] = cpu_baseline(cfg, tp, min(labels, L), args.seed)
+    if cpu_report is not None:
+        result["cpu_baseline"] = cpu_report
     print(json.dumps(result))
 
 

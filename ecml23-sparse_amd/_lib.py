@@ -29,6 +29,7 @@ SIGNATURES = {
     "ffi_input_grad_planned_f32": (_int, [_vp, _vp, _vp, _vp, _i64, _int, _vp]),
     "ffi_cache_clear": (_int, []),
     "ffi_cache_bytes": (ctypes.c_size_t, []),
+    "ffi_workspace_bytes": (ctypes.c_size_t, [_i64, _i64, _i64, _i64, _int, _int]),
     "ffi_check_lookup": (_int, [_vp, _i64, _i64, _i64, _vp]),
     "ffi_weight_grad_planned_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _vp]),
     "ffi_arrange_connections_f32": (_int, [_vp, _vp, _int, _i64, _i64, _vp]),

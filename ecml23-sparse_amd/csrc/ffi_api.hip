@@ -1,8 +1,11 @@
 // extern "C" entry points of libffi_hip.so: argument checks, plan cache, dispatch.
 // No arithmetic lives here.
 #include "ffi_internal.h"
+#include "ffi_lds_tile.h"
 
+#include <algorithm>
 #include <climits>
+#include <cmath>
 #include <mutex>
 #include <new>
 #include <vector>
@@ -571,6 +574,44 @@ size_t ffi_cache_bytes(void) {
     for (ffi_plan* p : g_cache)
         if (p->device == dev) total += p->bytes;
     return total + workspace_bytes(dev);
+}
+
+size_t ffi_workspace_bytes(int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in, int transposed, int passes) {
+    Dims d;
+    if (check_dims(batch, num_features, num_units, fan_in, transposed, &d) != FFI_OK) return 0;
+    const size_t B = (size_t)d.B, N = (size_t)d.N, L = (size_t)d.L, K = (size_t)d.K;
+    const bool narrow = tile_path_fits(d.N) && d.L < (1 << 25);
+    const size_t ldw = (B + 31) / 32 * 32;                         // row stride of the wide kernels' own copies
+    // the batch-major copy of the features (one slot, shared by the passes and by the permuted weights below)
+    size_t features_slot = 0;
+    if (narrow) features_slot = d.tp ? 0 : N * B * 4;
+    else features_slot = (d.tp && ldw == B) ? 0 : N * ldw * 4;
+    size_t total = 0, partial_slot = 0;
+    if (passes & FFI_PASS_BACKWARD) {
+        if (d.N <= 1024 && d.K <= 1024 && d.L < (1 << 25)) {
+            // tiled plan: the geometry of ffi_plan.hip, the slot rows of a slice estimated for column ids drawn uniformly
+            // (longest of 64 columns whose lengths scatter like Poisson counts around tile_labels * fan_in / num_features)
+            const size_t threads = (N + 63) / 64 * 64;
+            size_t TL = std::min<size_t>(std::min<size_t>(kPlanTileLabels, L), threads > 768 ? threads : 2 * threads);
+            TL = std::min<size_t>((TL + 1) & ~(size_t)1, ((size_t)(kPadPos - 1) / K) & ~(size_t)1);
+            const size_t tiles = (L + TL - 1) / TL, slices = threads / 64;
+            const double mu = (double)TL * (double)K / (double)N;
+            const size_t rows = (size_t)(mu + 2.6 * std::sqrt(mu) + 3.0);
+            const size_t slots = tiles * slices * rows * 64;
+            total += slots * 2 * 2 + (tiles * slices + 1) * 4 + L * 2;                  // lab16 + pos16, slice_off, rowpos
+            if (tile_path_fits(d.N) && d.N < (1 << kArrIdBits)) total += L * ((K + 31) / 32) * 32 * 2;   // idx16
+            features_slot = std::max(features_slot, slots * 4);                        // weights in slot order
+            const size_t nbt = (B + 31) / 32;
+            const size_t streams = std::max<size_t>(1, std::min<size_t>(tiles, (size_t)device_cu_count() / std::max<size_t>(1, nbt)));
+            partial_slot = streams * threads * nbt * 32 * 4;
+        } else {
+            const size_t nblocks = (L + 65535) / 65536;
+            total += L * K * 4 + (nblocks * N + 1) * 4;                                 // perm, col_ptr
+            partial_slot = L * ldw * 4;                                                 // out_grad, batch-major
+            if (!d.tp) features_slot = std::max(features_slot, N * B * 4);
+        }
+    }
+    return total + features_slot + partial_slot;
 }
 
 int ffi_check_lookup(const int32_t* lookup, int64_t num_units, int64_t fan_in, int64_t num_features,

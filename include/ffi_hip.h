@@ -153,6 +153,17 @@ int ffi_arrange_connections_f32(int32_t* lookup, float* const* arrays, int n_arr
 int ffi_cache_clear(void);
 /* Device bytes currently held by the library (plans + workspaces) on the current device. */
 size_t ffi_cache_bytes(void);
+/*
+ * What the library will hold on the device, beside the caller's tensors, once ffi_forward_f32 (FFI_PASS_FORWARD) and / or
+ * ffi_backward_f32 (FFI_PASS_BACKWARD) have run at this shape on one stream: the cached plan of the lookup matrix and
+ * the per-stream workspaces.  The reference's op owns no memory (TensorFlow allocates every buffer,
+ * tfsparse/cc/kernels/register.cpp:29,59-60); this lets a caller budget for what this library adds.  The plan's size
+ * depends on the lookup's content: the figure assumes column ids drawn uniformly (as the reference draws them,
+ * sparse/custom_layer.py:15,38) and is an estimate; ffi_cache_bytes() reports the actual amount afterwards.  Needs a
+ * current device only for the number of compute units; returns 0 for shapes the entry points reject.
+ */
+enum ffi_pass_flags { FFI_PASS_FORWARD = 1, FFI_PASS_BACKWARD = 2 };
+size_t ffi_workspace_bytes(int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in, int transposed, int passes);
 
 /*
  * Host-side audit of a lookup matrix (the reference checks index ranges only in audit builds,
