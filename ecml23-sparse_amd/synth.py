@@ -107,6 +107,38 @@ def make_inputs(cfg: FfiConfig, seed: int = 42, device="cpu", transposed: bool =
     return {"features": features, "lookup": lookup, "weights": weights, "out_grad": out_grad}
 
 
+def _splitmix64(seed: int, first: int, count: int):
+    """Draws first .. first+count-1 of the counter-based generator the C++ caller uses (tests/cpp/cabi_harness.cpp):
+    draw i of seed s is mix(s + (i + 1) * 0x9e3779b97f4a7c15) with splitmix64's finaliser."""
+    import numpy as np
+
+    with np.errstate(over="ignore"):
+        z = np.uint64(seed) + (np.arange(first + 1, first + count + 1, dtype=np.uint64) * np.uint64(0x9E3779B97F4A7C15))
+        z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+        z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+        return z ^ (z >> np.uint64(31))
+
+
+def counter_case(batch, num_features, num_units, fan_in, transposed=False, seed=42):
+    """One case of the reference's test law (testing/test_case_templates.h:52-69,113-114: uniform [-1,1) features and
+    weights, column ids uniform with replacement, out_grad clipped at zero), drawn from the seeded counter-based
+    generator that the C++ caller of the C ABI draws from too: both produce the same bits for the same seed, so a
+    case can be run on one side and checked on the other.  numpy arrays (features, lookup, weights, out_grad)."""
+    import numpy as np
+
+    def uniform(first, count):
+        return ((_splitmix64(seed, first, count) >> np.uint64(11)).astype(np.float64) * (2.0 / 9007199254740992.0) - 1.0).astype(np.float32)
+
+    B, N, L, K = batch, num_features, num_units, fan_in
+    at = 0
+    x = uniform(at, B * N).reshape(B, N); at += B * N
+    lookup = (_splitmix64(seed, at, L * K) % np.uint64(N)).astype(np.int32).reshape(L, K); at += L * K
+    w = uniform(at, L * K).reshape(L, K); at += L * K
+    g = np.maximum(uniform(at, B * L), 0).astype(np.float32).reshape(B, L)
+    features = np.ascontiguousarray(x.T) if transposed else x
+    return features, lookup, w, g
+
+
 def algorithmic_bytes(cfg: FfiConfig, num_units=None):
     """Compulsory HBM traffic per pass (every input read once, every output written once), bytes."""
     B, N, K = cfg.batch, cfg.num_features, cfg.fan_in

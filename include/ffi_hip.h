@@ -13,7 +13,13 @@
  *     (the reference's "Tp" ops); lookup, weights, weight_grad are [num_units, fan_in];
  *     result / out_grad are [batch, num_units]; feature_grad has the shape of features;
  *   - lookup holds column ids in [0, num_features); int32 and uint32 share the entry points
- *     (same bits for valid ids), duplicates inside a row are legal and accumulate;
+ *     (same bits for valid ids), duplicates inside a row are legal and accumulate.  The backward entry points
+ *     reject ids outside that range (FFI_ERR_BAD_LOOKUP); the forward entry points do not look (neither does the
+ *     reference in release builds, kernel_data.cu.h:211) and their results for such a lookup are undefined, not
+ *     just for the offending connection: the narrow-input kernels keep two 16-bit ids per register, so an id of
+ *     65,536 or more also changes its neighbour, and an id in [num_features, 65,536) reads whatever lies behind
+ *     the staged features in LDS (reads past the end of LDS return zero; no device memory outside the call's
+ *     buffers is touched).  ffi_check_lookup audits a matrix;
  *   - outputs are fully overwritten; work is enqueued on `stream` (a hipStream_t passed as void*,
  *     NULL = the default stream) and, with two documented exceptions, never synchronises the host;
  *   - every function returns FFI_OK (0) or a negative ffi_status instead of aborting, where the

@@ -10,6 +10,10 @@
 //                                     against the oracle with the reference's absolute gates (1e-5 forward,
 //                                     1.5e-5 gradients: test_case_templates.h:82,139-140; relative gates where the
 //                                     sums are too long for those).  Exit code = failures.
+//   cabi_harness sums B N L K T SEED  draws one case (T = 1: features [N,B]) from the seeded generator below -- the same
+//                                     stream of draws as ecml23_sparse_amd.synth.counter_case in Python -- runs forward and
+//                                     backward, prints double-precision sums of every tensor: a Python caller drawing the same
+//                                     case can tell that both sides computed on identical bits.
 //   cabi_harness bench [B N L K]      forward and backward timings in both layouts, 1 warm-up + 5 timed calls
 //                                     (testing/quick-bench.cpp:14-35; default shape {50, 32768, 670000, 32}).
 #include <hip/hip_runtime.h>
@@ -53,6 +57,9 @@ namespace {
         }                                                                                         \
     } while (0)
 
+// Counter-based: draw i of seed s is mix(s + (i + 1) * 0x9e3779b97f4a7c15), so any implementation can produce any
+// draw without the ones before it (ecml23_sparse_amd/synth.py has the numpy twin).  Order of draws in a case: features
+// [B,N] row-major, lookup, weights, out_grad.
 struct Rng {                       // splitmix64
     uint64_t s;
     uint64_t next() {
@@ -213,6 +220,25 @@ int error_codes(hipStream_t stream) {
     return failures;
 }
 
+double sum_of(const std::vector<float>& a) { double t = 0; for (float v : a) t += (double)v; return t; }
+
+int sums(hipStream_t stream, const Shape& s, bool transposed, uint64_t seed) {
+    const Case c = make_case(s, transposed, seed);
+    DeviceBuffer<float> dx(c.features.size()), dw(c.weights.size()), dg(c.out_grad.size());
+    DeviceBuffer<float> dout(c.out_grad.size()), dgx(c.features.size()), dgw(c.weights.size());
+    DeviceBuffer<int32_t> dl(c.lookup.size());
+    dx.upload(c.features); dw.upload(c.weights); dg.upload(c.out_grad); dl.upload(c.lookup);
+    FFI_OK_OR_DIE(ffi_forward_f32(dx.p, dl.p, dw.p, dout.p, s.B, s.N, s.L, s.K, transposed, stream));
+    FFI_OK_OR_DIE(ffi_backward_f32(dx.p, dl.p, dw.p, dg.p, dgx.p, dgw.p, s.B, s.N, s.L, s.K, transposed, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    long long ids = 0;
+    for (int32_t v : c.lookup) ids += v;
+    std::printf("sums features %.17g lookup %lld weights %.17g out_grad %.17g result %.17g feature_grad %.17g weight_grad %.17g\n",
+                sum_of(c.features), ids, sum_of(c.weights), sum_of(c.out_grad), sum_of(dout.download()), sum_of(dgx.download()),
+                sum_of(dgw.download()));
+    return 0;
+}
+
 template <typename F>
 double time_ms(hipStream_t stream, int iters, F&& call) {
     call();                                             // warm-up (builds the plan of the lookup on first use)
@@ -272,8 +298,11 @@ int main(int argc, char** argv) {
         Shape s{50, 32768, 670000, 32};
         if (argc == 6) s = Shape{std::atoll(argv[2]), std::atoll(argv[3]), std::atoll(argv[4]), std::atoll(argv[5])};
         rc = bench(stream, s);
+    } else if (std::strcmp(mode, "sums") == 0 && argc == 8) {
+        rc = sums(stream, Shape{std::atoll(argv[2]), std::atoll(argv[3]), std::atoll(argv[4]), std::atoll(argv[5])},
+                  std::atoi(argv[6]) != 0, (uint64_t)std::strtoull(argv[7], nullptr, 10));
     } else {
-        std::fprintf(stderr, "usage: %s test | bench [B N L K]\n", argv[0]);
+        std::fprintf(stderr, "usage: %s test | bench [B N L K] | sums B N L K T SEED\n", argv[0]);
         rc = 2;
     }
     ffi_cache_clear();
