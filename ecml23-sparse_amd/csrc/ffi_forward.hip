@@ -309,6 +309,178 @@ __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* _
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// The same kernel over batch tiles of 64 for inputs narrow enough that an [N][64] fp32 tile of x fits in LDS
+// (N <= kLane64MaxN): a row is 256 bytes and covers all 64 banks, so with the chunk order skewed by (lane & 15)
+// the 32 lanes the LDS serves together hit every bank exactly twice whatever rows they read (128-byte rows sit in
+// one half of the banks and the random parities of the rows cost about 1.7x), and W/idx are read once per 64
+// batch rows instead of once per 32.  Plain scores only.
+// ------------------------------------------------------------------------------------------------
+constexpr int kLane64Batch = 64;
+constexpr int kLane64MaxN = 608;        // 152 KB of LDS
+
+template <int THREADS>
+__device__ __forceinline__ void stage_rows64(float* __restrict__ xs, const float* __restrict__ src, int rows, int ld, int c0) {
+    const bool vec = (ld % 4 == 0) && (c0 + kLane64Batch <= ld) && (((uintptr_t)src & 15) == 0);
+    if (vec) {
+        // thread -> (row, 16-byte chunk): 16 threads per row, all of a thread's loads before its first LDS write
+        constexpr int kRowsPerIter = THREADS / 16;
+        constexpr int kInFlight = 4;
+        const int q = threadIdx.x & 15;
+        const float* p = src + c0 + 4 * q;
+        for (int r0 = threadIdx.x >> 4; r0 < rows; r0 += kRowsPerIter * kInFlight) {
+            float4 v[kInFlight];
+#pragma unroll
+            for (int i = 0; i < kInFlight; ++i) {
+                const int r = r0 + i * kRowsPerIter;
+                v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (r < rows) v[i] = *reinterpret_cast<const float4*>(p + (size_t)r * ld);
+            }
+#pragma unroll
+            for (int i = 0; i < kInFlight; ++i) {
+                const int r = r0 + i * kRowsPerIter;
+                if (r < rows) *reinterpret_cast<float4*>(xs + r * kLane64Batch + 4 * q) = v[i];
+            }
+        }
+    } else {
+        const int c = threadIdx.x & 63;
+        const bool in = c0 + c < ld;
+        const float* p = src + c0 + c;
+        for (int r = threadIdx.x >> 6; r < rows; r += THREADS / 64)
+            xs[r * kLane64Batch + c] = in ? p[(size_t)r * ld] : 0.f;
+    }
+}
+
+// base = address of the row + (lane & 15) * 16 (the tile is 256-byte aligned: the chunk bits are flipped with XOR)
+template <int C>
+__device__ __forceinline__ void fwd_lane64_step(unsigned base, float wv, float (&acc)[64]) {
+    const lds_v4f v = *(lds_v4f_ptr)(size_t)(C == 0 ? base : (base ^ (unsigned)(C * 16)));
+    acc[4 * C + 0] = fmaf(wv, v.x, acc[4 * C + 0]);
+    acc[4 * C + 1] = fmaf(wv, v.y, acc[4 * C + 1]);
+    acc[4 * C + 2] = fmaf(wv, v.z, acc[4 * C + 2]);
+    acc[4 * C + 3] = fmaf(wv, v.w, acc[4 * C + 3]);
+}
+
+// v[4c+i] <-> v[4(c ^ r)+i] for r in [0,16): its own inverse; four stages of conditional swaps.
+__device__ __forceinline__ void xor_permute_groups64(float (&v)[64], int r) {
+    const bool b8 = r & 8, b4 = r & 4, b2 = r & 2, b1 = r & 1;
+#pragma unroll
+    for (int e = 0; e < 64; ++e)
+        if (!(e & 32)) cond_swap(b8, v[e], v[e + 32]);
+#pragma unroll
+    for (int e = 0; e < 64; ++e)
+        if (!(e & 16)) cond_swap(b4, v[e], v[e + 16]);
+#pragma unroll
+    for (int e = 0; e < 64; ++e)
+        if (!(e & 8)) cond_swap(b2, v[e], v[e + 8]);
+#pragma unroll
+    for (int e = 0; e < 64; ++e)
+        if (!(e & 4)) cond_swap(b1, v[e], v[e + 4]);
+}
+
+template <bool VEC4>
+__global__ __launch_bounds__(kTileThreads) void fwd_lane64_kernel(const float* __restrict__ xT, const int32_t* __restrict__ idx,
+                                                                  const float* __restrict__ w, const float* __restrict__ bias,
+                                                                  float* __restrict__ out, int B, int N, int L, int K, int nbt,
+                                                                  int labels_per_stream) {
+    extern __shared__ __align__(256) float xs[];
+    const int u = xcd_contiguous_block(blockIdx.x, gridDim.x);
+    const int bt = u % nbt, stream = u / nbt;
+    const int b0 = bt * kLane64Batch;
+    stage_rows64<kTileThreads>(xs, xT, N, B, b0);
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
+    const unsigned skewbase = (unsigned)(size_t)(__attribute__((address_space(3))) float*)xs + (unsigned)(lane & 15) * 16u;
+    const int l_begin = stream * labels_per_stream;
+    const int l_end = min(l_begin + labels_per_stream, L);
+    // rows of out for this batch tile, reached through a scalar row offset plus the lane's label; rows past the batch
+    // lie beyond the resource's size and their stores are dropped
+    const int nrows = min(kLane64Batch, B - b0);
+    const buffer_rsrc orsrc = make_rsrc(out + (size_t)b0 * (size_t)L, (size_t)nrows * (size_t)L * sizeof(float));
+    for (int base = l_begin; base < l_end; base += kTileThreads) {
+        if (base + (int)(threadIdx.x & ~63u) >= l_end) break;     // nothing left for this wavefront
+        const int j = base + (int)threadIdx.x;
+        const bool valid = j < l_end;
+        const int jj = valid ? j : l_end - 1;
+        const int32_t* irow = idx + (size_t)jj * K;
+        const float* wrow = w + (size_t)jj * K;
+        float acc[64];
+#pragma unroll
+        for (int i = 0; i < 64; ++i) acc[i] = 0.f;
+        for (int k0 = 0; k0 < K; k0 += 16) {
+            const bool full = VEC4 && k0 + 16 <= K;
+            unsigned idp[8];
+            float wv[16];
+            if (full) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int4 v = *reinterpret_cast<const int4*>(irow + k0 + 4 * q);
+                    idp[2 * q + 0] = (unsigned)v.x | ((unsigned)v.y << 16);
+                    idp[2 * q + 1] = (unsigned)v.z | ((unsigned)v.w << 16);
+                    const float4 f = *reinterpret_cast<const float4*>(wrow + k0 + 4 * q);
+                    wv[4 * q] = f.x; wv[4 * q + 1] = f.y; wv[4 * q + 2] = f.z; wv[4 * q + 3] = f.w;
+                }
+            } else {
+#pragma unroll
+                for (int q = 0; q < 8; ++q) {
+                    const unsigned a = (k0 + 2 * q < K) ? (unsigned)irow[k0 + 2 * q] : 0u;
+                    const unsigned b = (k0 + 2 * q + 1 < K) ? (unsigned)irow[k0 + 2 * q + 1] : 0u;
+                    idp[q] = a | (b << 16);
+                }
+#pragma unroll
+                for (int k = 0; k < 16; ++k) wv[k] = (k0 + k < K) ? wrow[k0 + k] : 0.f;
+            }
+            const int kn = min(16, K - k0);
+#pragma unroll
+            for (int k = 0; k < 16; ++k) {
+                if (full || k < kn) {
+                    const unsigned id = (k & 1) ? (idp[k >> 1] >> 16) : (idp[k >> 1] & 0xffffu);
+                    const unsigned rb = (id << 8) + skewbase;
+                    fwd_lane64_step<0>(rb, wv[k], acc); fwd_lane64_step<1>(rb, wv[k], acc);
+                    fwd_lane64_step<2>(rb, wv[k], acc); fwd_lane64_step<3>(rb, wv[k], acc);
+                    fwd_lane64_step<4>(rb, wv[k], acc); fwd_lane64_step<5>(rb, wv[k], acc);
+                    fwd_lane64_step<6>(rb, wv[k], acc); fwd_lane64_step<7>(rb, wv[k], acc);
+                    fwd_lane64_step<8>(rb, wv[k], acc); fwd_lane64_step<9>(rb, wv[k], acc);
+                    fwd_lane64_step<10>(rb, wv[k], acc); fwd_lane64_step<11>(rb, wv[k], acc);
+                    fwd_lane64_step<12>(rb, wv[k], acc); fwd_lane64_step<13>(rb, wv[k], acc);
+                    fwd_lane64_step<14>(rb, wv[k], acc); fwd_lane64_step<15>(rb, wv[k], acc);
+                }
+            }
+        }
+        xor_permute_groups64(acc, lane & 15);              // back to natural batch order
+        if (bias != nullptr) {                             // added after the sum, as a separate bias_add would
+            const float bj = bias[jj];
+#pragma unroll
+            for (int i = 0; i < 64; ++i) acc[i] += bj;
+        }
+        if (valid) {
+            const unsigned lane_off = (unsigned)j * 4u;
+            const unsigned stride = (unsigned)L * 4u;
+#pragma unroll
+            for (int b = 0; b < 64; ++b)
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, acc[b]), orsrc, lane_off, (unsigned)b * stride, 0);
+        }
+    }
+}
+
+template <bool VEC4>
+int launch_lane64(const float* xT, const int32_t* idx, const float* w, const float* bias, float* out, const Dims& d, hipStream_t s) {
+    const int cus = device_cu_count();
+    const int nbt = (d.B + kLane64Batch - 1) / kLane64Batch;
+    int streams = std::max(1, cus / nbt);
+    const int per_stream = (d.L + streams - 1) / streams;
+    streams = (d.L + per_stream - 1) / per_stream;
+    const size_t lds = (size_t)d.N * kLane64Batch * sizeof(float);
+    FFI_HIP_TRY(hipFuncSetAttribute((const void*)fwd_lane64_kernel<VEC4>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL((fwd_lane64_kernel<VEC4>), dim3(streams * nbt), dim3(kTileThreads), lds, s, xT, idx, w, bias, out, d.B, d.N,
+                       d.L, d.K, nbt, per_stream);
+    FFI_HIP_TRY(hipGetLastError());
+    return FFI_OK;
+}
+
+// (64 rows of out of a batch tile are reached through 32-bit byte offsets)
+bool lane64_fits(const Dims& d) { return d.N <= kLane64MaxN && d.B > kTileBatch && d.L < (1 << 24); }
+
 }  // namespace
 
 namespace {
@@ -378,6 +550,8 @@ int forward_tiles(const float* x, const int32_t* idx, const float* w, const floa
     }
     const size_t lds = tile_lds_bytes(d.N);
     const bool vec4 = (d.K % 4 == 0) && (((uintptr_t)w | (uintptr_t)idx) % 16 == 0);
+    if (epi == kEpiScores && tk == nullptr && lane64_fits(d))
+        return vec4 ? launch_lane64<true>(xT, idx, w, bias, out, d, s) : launch_lane64<false>(xT, idx, w, bias, out, d, s);
     const int cus = device_cu_count();
     const int nbt = (d.B + kTileBatch - 1) / kTileBatch;
     int streams = std::max(1, cus / nbt);

@@ -73,16 +73,21 @@ __global__ __launch_bounds__(kBlock) void fingerprint_kernel(const int32_t* __re
     }
 }
 
-// The same fingerprint, checked on the device: workgroups add their sums to guard[0] / guard[1] (integer adds:
-// the total does not depend on their order), the last one to finish compares the total with guard[3], leaves the
-// verdict in guard[4] (1 = content unchanged and every id in range), the sums in guard[5] / guard[6], and clears
-// the accumulators for the next check.
-__global__ __launch_bounds__(kBlock) void fingerprint_guard_kernel(const int32_t* __restrict__ idx, size_t total, unsigned N,
-                                                                    unsigned long long* __restrict__ guard) {
+// The same fingerprint, checked on the device.  Workgroups leave their pairs of sums in guard[8 + 2 * block ..]
+// (plain stores) and take a ticket from guard[2], the only atomic: a few hundred adds to one address, not
+// thousands (those serialise and were measured to triple the kernel's time).  The workgroup that draws the last
+// ticket adds the pairs up (integer adds: the total does not depend on the order), compares with guard[3], leaves
+// the verdict in guard[4] (1 = content unchanged and every id in range), the sums in guard[5] / guard[6], and
+// clears the ticket counter for the next check.
+constexpr int kGuardBlock = 1024;
+constexpr int kGuardBlocks = 256;                         // workgroups of the guard kernel (at most)
+constexpr int kGuardWords = 8 + 2 * kGuardBlocks;
+__global__ __launch_bounds__(kGuardBlock) void fingerprint_guard_kernel(const int32_t* __restrict__ idx, size_t total, unsigned N,
+                                                                         unsigned long long* __restrict__ guard) {
     unsigned long long h = 0;
     unsigned bad = 0;
-    const size_t stride = (size_t)gridDim.x * kBlock;
-    const size_t tid = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * kGuardBlock;
+    const size_t tid = (size_t)blockIdx.x * kGuardBlock + threadIdx.x;
     const bool vec = ((uintptr_t)idx & 15) == 0;
     const size_t nvec = vec ? total / 4 : 0;
     const int4* idx4 = reinterpret_cast<const int4*>(idx);
@@ -107,23 +112,39 @@ __global__ __launch_bounds__(kBlock) void fingerprint_guard_kernel(const int32_t
         h += __shfl_down(h, off);
         b64 += __shfl_down(b64, off);
     }
-    __shared__ unsigned long long part[2][kBlock / 64];
+    __shared__ unsigned long long part[2][kGuardBlock / 64];
+    __shared__ bool last;
     if ((threadIdx.x & 63) == 0) { part[0][threadIdx.x >> 6] = h; part[1][threadIdx.x >> 6] = b64; }
     __syncthreads();
     if (threadIdx.x == 0) {
         unsigned long long hs = 0, bs = 0;
 #pragma unroll
-        for (int i = 0; i < kBlock / 64; ++i) { hs += part[0][i]; bs += part[1][i]; }
-        atomicAdd(&guard[0], hs);
-        atomicAdd(&guard[1], bs);
+        for (int i = 0; i < kGuardBlock / 64; ++i) { hs += part[0][i]; bs += part[1][i]; }
+        __hip_atomic_store(&guard[8 + 2 * blockIdx.x], hs, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&guard[9 + 2 * blockIdx.x], bs, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __threadfence();
-        if (atomicAdd(&guard[2], 1ull) == (unsigned long long)gridDim.x - 1) {
-            __threadfence();
-            const unsigned long long sum = atomicAdd(&guard[0], 0ull), nbad = atomicAdd(&guard[1], 0ull);
-            guard[5] = sum;
-            guard[6] = nbad;
-            guard[4] = (sum == guard[3] && nbad == 0) ? 1ull : 0ull;
-            guard[0] = 0; guard[1] = 0; guard[2] = 0;
+        last = atomicAdd(&guard[2], 1ull) == (unsigned long long)gridDim.x - 1;
+    }
+    __syncthreads();
+    if (!last) return;
+    __threadfence();
+    // the last workgroup: its first wavefront adds the pairs of all workgroups
+    if (threadIdx.x < 64) {
+        unsigned long long hs = 0, bs = 0;
+        for (unsigned i = threadIdx.x; i < gridDim.x; i += 64) {
+            hs += __hip_atomic_load(&guard[8 + 2 * i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            bs += __hip_atomic_load(&guard[9 + 2 * i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            hs += __shfl_down(hs, off);
+            bs += __shfl_down(bs, off);
+        }
+        if (threadIdx.x == 0) {
+            guard[5] = hs;
+            guard[6] = bs;
+            guard[4] = (hs == guard[3] && bs == 0) ? 1ull : 0ull;
+            guard[2] = 0;
         }
     }
 }
@@ -546,10 +567,10 @@ int plan_scratch_alloc(ffi_plan* p) {
                     hipHostMalloc(&p->h_scratch, kScratchWords * sizeof(unsigned long long)) == hipSuccess &&
                     hipEventCreateWithFlags(&p->fp_done, hipEventDisableTiming) == hipSuccess &&
                     hipMemset(p->d_scratch, 0, kScratchWords * sizeof(unsigned long long)) == hipSuccess &&
-                    hipMalloc(&p->d_guard, 8 * sizeof(unsigned long long)) == hipSuccess &&
+                    hipMalloc(&p->d_guard, kGuardWords * sizeof(unsigned long long)) == hipSuccess &&
                     hipHostMalloc(&p->h_guard, 8 * sizeof(unsigned long long)) == hipSuccess &&
                     hipEventCreateWithFlags(&p->guard_done, hipEventDisableTiming) == hipSuccess &&
-                    hipMemset(p->d_guard, 0, 8 * sizeof(unsigned long long)) == hipSuccess;
+                    hipMemset(p->d_guard, 0, kGuardWords * sizeof(unsigned long long)) == hipSuccess;
     if (!ok) {
         (void)hipGetLastError();
         return FFI_ERR_OUT_OF_MEMORY;
@@ -645,8 +666,8 @@ int plan_guard_enqueue(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     // a check of this plan still running on another stream shares the accumulators: order the two
     if (p->guard_pending && p->guard_stream != s) FFI_HIP_TRY(hipStreamWaitEvent(s, p->guard_done, 0));
     const size_t total = (size_t)p->L * p->K;
-    const unsigned blocks = (unsigned)std::min<size_t>((total / 4 + kBlock - 1) / kBlock + 1, kFingerprintBlocks);
-    hipLaunchKernelGGL(fingerprint_guard_kernel, dim3(blocks), dim3(kBlock), 0, s, lookup, total, (unsigned)p->N, p->d_guard);
+    const unsigned blocks = (unsigned)std::min<size_t>((total / 4 + kGuardBlock - 1) / kGuardBlock + 1, kGuardBlocks);
+    hipLaunchKernelGGL(fingerprint_guard_kernel, dim3(blocks), dim3(kGuardBlock), 0, s, lookup, total, (unsigned)p->N, p->d_guard);
     FFI_HIP_TRY(hipGetLastError());
     FFI_HIP_TRY(hipMemcpyAsync(p->h_guard, p->d_guard + kGuardVerdict, 3 * sizeof(unsigned long long), hipMemcpyDeviceToHost, s));
     FFI_HIP_TRY(hipEventRecord(p->guard_done, s));

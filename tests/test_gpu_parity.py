@@ -134,7 +134,8 @@ def test_layouts_agree(ffi, shape):
 # shapes that steer the library through each of its code paths:
 #   narrow inputs (LDS tile kernels), wide inputs (generic kernels), the tiled and the global plan,
 #   partly filled batch tiles, fan-ins below / across / beyond the 32-connection register chunk,
-#   fewer labels than one tile, more than 1024 columns (global plan with tile forward/weight-grad)
+#   fewer labels than one tile, more than 1024 columns (global plan with tile forward/weight-grad),
+#   the forward kernel over batch tiles of 64
 PATH_SHAPES = [
     (300, 700, 5000, 32),      # 10 batch tiles, the last one partly filled
     (33, 96, 9, 5),            # fewer labels than lanes, odd fan-in
@@ -146,6 +147,11 @@ PATH_SHAPES = [
     (200, 2000, 600, 33),      # wide, two batch passes
     (7, 64, 70000, 3),         # many tiles of a tiny column set
     (128, 512, 4100, 100),     # four register chunks per label, tail of 4
+    # forward over batch tiles of 64 (N <= 608 and more than 32 samples):
+    (256, 512, 5000, 64),      # whole tiles, vector loads
+    (100, 608, 3100, 21),      # the widest input of that path, second tile partly filled, odd fan-in (scalar loads)
+    (33, 40, 2100, 24),        # one sample beyond a 32-tile; fan-in with a tail of 8 behind a half chunk of 16
+    (65, 300, 1500, 8),        # one sample in the second 64-tile; fan-in below a half chunk
 ]
 
 
