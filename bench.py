@@ -404,10 +404,13 @@ def main():
     achieved = alg[dominant] / (kernel_ms[dominant] * 1e-3) / 1e9
     traffic, traffic_source = measured_traffic(cfg.name)
     narrow = N <= 1216
+    pass_kernels = dict(PASS_KERNELS if narrow else WIDE_PASS_KERNELS)
+    if N <= 608 and B > 32:
+        pass_kernels["forward"] = "fwd_lane64_kernel"       # batch tiles of 64 when the [N][64] tile fits in LDS
     flops = 2.0 * B * L * K
     roofline = {
         "bound": "hbm",
-        "kernel": f"{dominant} pass ({(PASS_KERNELS if narrow else WIDE_PASS_KERNELS)[dominant]})",
+        "kernel": f"{dominant} pass ({pass_kernels[dominant]})",
         "achieved": round(achieved, 2),
         "peak": HBM_PEAK_GBPS,
         "unit": "GB/s",
