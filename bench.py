@@ -407,6 +407,10 @@ def main():
     pass_kernels = dict(PASS_KERNELS if narrow else WIDE_PASS_KERNELS)
     if N <= 608 and B > 32:
         pass_kernels["forward"] = "fwd_lane64_kernel"       # batch tiles of 64 when the [N][64] tile fits in LDS
+    threads, nbt = (N + 63) // 64 * 64, (B + 31) // 32
+    if narrow and threads <= 768 and (nbt <= 2 or (nbt <= 4 and threads >= 704)) and K <= 32:
+        # the plan's tiles are small enough for the walking kernel to keep the tile's weights in LDS: no permutation kernel
+        pass_kernels["input_grad"] = "igrad_tile_kernel + igrad_reduce_kernel"
     flops = 2.0 * B * L * K
     roofline = {
         "bound": "hbm",

@@ -80,6 +80,7 @@ int create_cached_plan(const int32_t* lookup, const Dims& d, int dev, hipStream_
     }
     ffi_plan* p = nullptr;
     FFI_TRY(plan_alloc(d.L, d.K, d.N, &p));
+    p->batch_hint = d.B;
     int st = plan_build(p, lookup, s);
     if (st != FFI_OK) { plan_free(p); delete p; return st; }
     g_cache.push_back(p);
@@ -488,6 +489,7 @@ int ffi_plan_create(const int32_t* lookup, int64_t num_units, int64_t fan_in, in
     FFI_TRY(check_dims(batch_hint > 0 ? batch_hint : 1, num_features, num_units, fan_in, 0, &d));
     ffi_plan* p = nullptr;
     FFI_TRY(plan_alloc(d.L, d.K, d.N, &p));
+    p->batch_hint = d.B;
     int st = plan_build(p, lookup, (hipStream_t)stream);
     if (st != FFI_OK) { plan_free(p); delete p; return st; }
     *plan = p;
@@ -592,15 +594,15 @@ size_t ffi_workspace_bytes(int64_t batch, int64_t num_features, int64_t num_unit
             // tiled plan: the geometry of ffi_plan.hip, the slot rows of a slice estimated for column ids drawn uniformly
             // (longest of 64 columns whose lengths scatter like Poisson counts around tile_labels * fan_in / num_features)
             const size_t threads = (N + 63) / 64 * 64;
-            size_t TL = std::min<size_t>(std::min<size_t>(kPlanTileLabels, L), threads > 768 ? threads : 2 * threads);
-            TL = std::min<size_t>((TL + 1) & ~(size_t)1, ((size_t)(kPadPos - 1) / K) & ~(size_t)1);
+            bool w_in_lds = false;
+            const size_t TL = (size_t)plan_tile_labels(d.N, d.K, d.L, d.B, &w_in_lds);
             const size_t tiles = (L + TL - 1) / TL, slices = threads / 64;
             const double mu = (double)TL * (double)K / (double)N;
             const size_t rows = (size_t)(mu + 2.6 * std::sqrt(mu) + 3.0);
             const size_t slots = tiles * slices * rows * 64;
             total += slots * 2 * 2 + (tiles * slices + 1) * 4 + L * 2;                  // lab16 + pos16, slice_off, rowpos
             if (tile_path_fits(d.N) && d.N < (1 << kArrIdBits)) total += L * ((K + 31) / 32) * 32 * 2;   // idx16
-            features_slot = std::max(features_slot, slots * 4);                        // weights in slot order
+            if (!w_in_lds) features_slot = std::max(features_slot, slots * 4);         // weights in slot order
             const size_t nbt = (B + 31) / 32;
             const size_t streams = std::max<size_t>(1, std::min<size_t>(tiles, (size_t)device_cu_count() / std::max<size_t>(1, nbt)));
             partial_slot = streams * threads * nbt * 32 * 4;

@@ -117,12 +117,16 @@ __device__ __forceinline__ void igrad_fmas(const float4 (&v)[8], float wv, float
 // partial[stream][n][b] over the stream's tiles.  grid = streams * batch tiles.
 // MAXT: largest workgroup the instantiation is launched with (sets the register budget);
 // LPT: labels of a tile staged per thread (tile_labels <= LPT * blockDim.x).
-template <int MAXT, int LPT>
+// WLDS: `wp` is the weight matrix itself and `pos16` the slots' positions in their tile's [tile_labels][K] block of it:
+// the tile's weights are staged in LDS behind the rows of out_grad (with a zero word at tile_labels * K that
+// padding slots read) and every slot fetches its weight from there, so no slot-ordered copy of the weights exists.
+template <int MAXT, int LPT, bool WLDS>
 __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* __restrict__ lab16, const float* __restrict__ wp,
                                   const unsigned* __restrict__ slice_off,
                                   const float* __restrict__ g, float* __restrict__ partial, int B, int L,
                                   int tile_labels, int tiles, int tiles_per_stream, int nbt, unsigned total_rows,
-                                  const unsigned short* __restrict__ rowpos, int zero_row) {
+                                  const unsigned short* __restrict__ rowpos, int zero_row,
+                                  const unsigned short* __restrict__ pos16, int K) {
     extern __shared__ __align__(16) float gs[];
     char* gs_bytes = reinterpret_cast<char*>(gs);
     const int nthreads = blockDim.x;
@@ -136,8 +140,13 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
     const int t_begin = stream * tiles_per_stream, t_end = min(t_begin + tiles_per_stream, tiles);
     // plan slots and permuted weights, addressed as (scalar row offset) + (lane offset); 4-GB buffers at most
     const buffer_rsrc lab_rsrc = make_rsrc(lab16, (size_t)total_rows * 128u);
-    const buffer_rsrc wp_rsrc = make_rsrc(wp, (size_t)total_rows * 256u);
+    const buffer_rsrc wp_rsrc = WLDS ? make_rsrc(pos16, (size_t)total_rows * 128u) : make_rsrc(wp, (size_t)total_rows * 256u);
     const unsigned lane2 = (unsigned)lane * 2u, lane4 = (unsigned)lane * 4u;
+    // (WLDS) the tile's weights behind the rows of out_grad and the two zero rows
+    float* ws = gs + (size_t)(zero_row + 2) * kTileBatch;
+    const unsigned wsbase = (unsigned)(size_t)(__attribute__((address_space(3))) float*)ws;
+    const unsigned tile_w = (unsigned)tile_labels * (unsigned)K;       // floats of a full tile; index of the zero word
+    constexpr int kWRegs = 8;                                           // 16-byte pieces of the tile's weights a thread carries
 
     float acc[32];
 #pragma unroll
@@ -154,9 +163,36 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
             const int jl = (int)threadIdx.x + p * nthreads;
             if (jl < nl) load_rows32(g, L, b0, B, (unsigned)(j0 + jl), gbn[p]);
         }
+        // (WLDS) the tile's block of the weight matrix, contiguous: requested with the rows of out_grad
+        float4 wreg[kWRegs];
+        const unsigned nw = (unsigned)nl * (unsigned)K;
+        const float* wt = wp + (size_t)j0 * K;
+        const bool wvec = WLDS && (nw % 4 == 0) && ((((uintptr_t)wt) & 15) == 0);
+        const unsigned nw4 = wvec ? nw / 4 : 0u;                         // 16-byte pieces; the first kWRegs * nthreads of them travel in registers
+#pragma unroll
+        for (int r = 0; r < kWRegs; ++r) {
+            const unsigned q = threadIdx.x + r * nthreads;
+            wreg[r] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (WLDS && q < nw4) wreg[r] = reinterpret_cast<const float4*>(wt)[q];
+        }
         __syncthreads();                       // the previous tile is no longer being read
         // rows `zero_row` (even) and `zero_row + 1` (odd) are all zero: the targets of padding slots
         if (t == t_begin && threadIdx.x < 64) gs[zero_row * kTileBatch + threadIdx.x] = 0.f;
+        if (WLDS) {
+            if (t == t_begin && threadIdx.x == 0) ws[tile_w] = 0.f;
+            if (wvec) {
+#pragma unroll
+                for (int r = 0; r < kWRegs; ++r) {
+                    const unsigned q = threadIdx.x + r * nthreads;
+                    if (q < nw4) reinterpret_cast<float4*>(ws)[q] = wreg[r];
+                }
+                // (tiles whose weights exceed that: the rest directly, one more round trip)
+                for (unsigned q = threadIdx.x + kWRegs * nthreads; q < nw4; q += nthreads)
+                    reinterpret_cast<float4*>(ws)[q] = reinterpret_cast<const float4*>(wt)[q];
+            } else {
+                for (unsigned q = threadIdx.x; q < nw; q += nthreads) ws[q] = wt[q];
+            }
+        }
         // gs[jl][c] = g[b0+c][j0+jl]: the rows were loaded coalesced along labels; 16-byte LDS writes
         // whose chunk order is skewed by the label id (no bank conflicts)
 #pragma unroll
@@ -186,7 +222,15 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
         auto load_lab = [&](unsigned r) {
             return (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(lab_rsrc, lane2, (row0 + r) * 128u, 0);
         };
-        auto load_w = [&](unsigned r) { return buffer_load_f32(wp_rsrc, lane4, (row0 + r) * 256u); };
+        // the slot's weight, or (WLDS) the LDS address of it: positions of padding slots (0xffff) end at the zero word
+        auto load_w = [&](unsigned r) {
+            if (WLDS) {
+                const unsigned pos = (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(wp_rsrc, lane2, (row0 + r) * 128u, 0);
+                return __builtin_bit_cast(float, wsbase + min(pos, tile_w) * 4u);
+            }
+            return buffer_load_f32(wp_rsrc, lane4, (row0 + r) * 256u);
+        };
+        const float w_none = WLDS ? __builtin_bit_cast(float, wsbase + tile_w * 4u) : 0.f;
         unsigned e4[kAhead];
         float w4[kAhead];
 #pragma unroll
@@ -213,7 +257,8 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
             for (int q = 0; q < kAhead; ++q) {
                 const bool in = i + q < rows;                       // wave-uniform
                 const unsigned e = in ? e4[q] : (unsigned)zero_row;
-                const float wv = in ? w4[q] : 0.f;
+                float wv = in ? w4[q] : w_none;
+                if (WLDS) wv = *(const float __attribute__((address_space(3)))*)(size_t)__builtin_bit_cast(unsigned, wv);
                 float4 xv[8];
                 igrad_reads(e, skewbase, xv);
                 igrad_fmas(xv, wv, acc);
@@ -269,28 +314,38 @@ int launch_tiled(const ffi_plan* p, const float* w, const float* g, float* gx, i
     const size_t slots = (size_t)p->total_rows * 64;
     float* wp = nullptr;
     float* partial = nullptr;
-    FFI_TRY(workspace_get(s, kWsFeaturesT, std::max<size_t>(slots, 1) * sizeof(float), (void**)&wp));
+    if (!p->w_in_lds) FFI_TRY(workspace_get(s, kWsFeaturesT, std::max<size_t>(slots, 1) * sizeof(float), (void**)&wp));
     FFI_TRY(workspace_get(s, kWsPartials, (size_t)streams * p->threads * bpad * sizeof(float), (void**)&partial));
     // large pieces (a whole tile of 1024 labels x 32 connections in one) as soon as the small one does not hold the
     // tile: every piece costs a walk over the tile's slots
     const int chunk = ((long long)p->tile_labels * p->K <= kPermChunk) ? kPermChunk : kPermChunkBig;
-    FFI_HIP_TRY(hipFuncSetAttribute((const void*)igrad_permute_weights_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, chunk * 4));
-    hipLaunchKernelGGL(igrad_permute_weights_kernel, dim3(p->tiles), dim3(p->threads), chunk * sizeof(float), s, p->pos16,
-                       p->slice_off, w, wp, p->L, p->K, p->tile_labels, chunk);
-    const size_t lds = tile_lds_bytes(p->zero_row + 2);         // the tile's rows + the two all-zero rows
+    if (!p->w_in_lds) {
+        FFI_HIP_TRY(hipFuncSetAttribute((const void*)igrad_permute_weights_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, chunk * 4));
+        hipLaunchKernelGGL(igrad_permute_weights_kernel, dim3(p->tiles), dim3(p->threads), chunk * sizeof(float), s, p->pos16,
+                           p->slice_off, w, wp, p->L, p->K, p->tile_labels, chunk);
+    }
+    // the tile's rows + the two all-zero rows (+ the tile's weights)
+    const size_t lds = tiled_lds_bytes(p->tile_labels, p->K, p->w_in_lds);
     const dim3 grid(streams * nbt), block(p->threads);
-#define FFI_LAUNCH_TILE(MAXT, LPT)                                                                                      \
+#define FFI_LAUNCH_TILE(MAXT, LPT, WLDS)                                                                                \
     do {                                                                                                                \
-        FFI_HIP_TRY(hipFuncSetAttribute((const void*)igrad_tile_kernel<MAXT, LPT>,                                      \
+        FFI_HIP_TRY(hipFuncSetAttribute((const void*)igrad_tile_kernel<MAXT, LPT, WLDS>,                                \
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));                        \
-        hipLaunchKernelGGL((igrad_tile_kernel<MAXT, LPT>), grid, block, lds, s, p->lab16, wp, p->slice_off, g, \
-                           partial, B, p->L, p->tile_labels, p->tiles, tps, nbt, (unsigned)p->total_rows, p->rowpos, p->zero_row);                                       \
+        hipLaunchKernelGGL((igrad_tile_kernel<MAXT, LPT, WLDS>), grid, block, lds, s, p->lab16, WLDS ? w : wp, p->slice_off, g, \
+                           partial, B, p->L, p->tile_labels, p->tiles, tps, nbt, (unsigned)p->total_rows, p->rowpos, p->zero_row, \
+                           p->pos16, p->K);                                                                             \
     } while (0)
     // the plan sizes its tiles so that one of these fits: tile_labels <= LPT * threads
-    if (p->threads <= 768) {
-        if (p->tile_labels <= p->threads) FFI_LAUNCH_TILE(768, 1); else FFI_LAUNCH_TILE(768, 2);
+    if (p->w_in_lds) {
+        if (p->threads <= 768) {
+            if (p->tile_labels <= p->threads) FFI_LAUNCH_TILE(768, 1, true); else FFI_LAUNCH_TILE(768, 2, true);
+        } else {
+            FFI_LAUNCH_TILE(1024, 1, true);
+        }
+    } else if (p->threads <= 768) {
+        if (p->tile_labels <= p->threads) FFI_LAUNCH_TILE(768, 1, false); else FFI_LAUNCH_TILE(768, 2, false);
     } else {
-        FFI_LAUNCH_TILE(1024, 1);
+        FFI_LAUNCH_TILE(1024, 1, false);
     }
 #undef FFI_LAUNCH_TILE
     dim3 rgrid((B + 255) / 256, p->N);

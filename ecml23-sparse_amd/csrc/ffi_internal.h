@@ -236,13 +236,24 @@ struct ffi_plan {
     bool guard_pending = false;               // a check has been enqueued whose result the host has not looked at
     hipStream_t guard_stream = nullptr;       // the stream of that check
     size_t bytes = 0;
+    int batch_hint = 0;                       // batch size the plan is expected to be used with (0 = unknown); steers layout choices only
+    bool w_in_lds = false;                    // tiled form: tiles small enough for the walking kernel to keep the tile's weights in LDS too
 };
 
 namespace ffi {
 constexpr int kPlanTileLabels = 1024;     // a [1024+1][32] fp32 tile fits LDS
 constexpr unsigned kPadPos = 0xffffu;      // pos16 of a padding slot; real positions are below it (tile_labels * K <= 0xffff)
+// LDS of the kernel that walks the tiled form: the tile's rows of out_grad (per bank half: half the tile plus some room
+// for the balancing) and two all-zero rows, 128 bytes each; with the tile's weights behind them, tile_labels * K floats
+// and one zero word that padding slots read.
+constexpr size_t kPlanLdsBudget = 160000;
+inline int tiled_rows_per_half(int tile_labels) { return tile_labels / 2 + (tile_labels / 16 < 64 ? tile_labels / 16 : 64); }
+inline size_t tiled_lds_bytes(int tile_labels, int K, bool with_weights) {
+    return (size_t)(2 * tiled_rows_per_half(tile_labels) + 2) * 128 + (with_weights ? ((size_t)tile_labels * K + 4) * 4 : 0);
+}
 constexpr int kArrIdBits = 11;            // column-id field of an arranged entry (narrow inputs: ids < 1216)
 int plan_build(ffi_plan* p, const int32_t* lookup, hipStream_t s);
+int plan_tile_labels(int N, int K, int L, int batch_hint, bool* weights_in_lds);
 int launch_arrange_in_place(int32_t* lookup, float* const* arrays, int n_arrays, int L, int K, hipStream_t s);
 // Content fingerprint of `lookup` (and the count of ids outside [0,N)).  _begin enqueues the kernel
 // on `s` and returns; _end waits for that kernel only, not for what the caller enqueued on `s`

@@ -346,7 +346,7 @@ void free_arrays(ffi_plan* p) {
     if (p->rowpos) (void)hipFree(p->rowpos);
     p->rowpos = nullptr;
     p->perm = nullptr; p->col_ptr = nullptr; p->slice_off = nullptr; p->lab16 = nullptr; p->pos16 = nullptr; p->idx16 = nullptr;
-    p->tiled = false; p->total_rows = 0; p->bytes = 0;
+    p->tiled = false; p->w_in_lds = false; p->total_rows = 0; p->bytes = 0;
 }
 
 template <class T>
@@ -359,6 +359,37 @@ bool dev_alloc(T** ptr, size_t count) {
     return true;
 }
 
+}  // namespace
+
+// Labels per tile of the tiled form, and whether the walking kernel keeps the tile's weights in LDS (then the tiles
+// are smaller).
+int plan_tile_labels(int N, int K, int L, int batch_hint, bool* weights_in_lds) {
+    const int threads = ((N + 63) / 64) * 64;
+    int TL = std::min((std::min(std::min(kPlanTileLabels, L), threads > 768 ? threads : 2 * threads) + 1) & ~1,
+                      (int)((kPadPos - 1) / (unsigned)K) & ~1);
+    // Tiles whose weights fit in LDS beside the tile of out_grad: the walking kernel then reads each slot's weight
+    // through pos16, and the weights need not be brought into slot order first (no permutation kernel, no slot-ordered
+    // copy of the weights in memory).
+    // Measured (gx pass, 0.3-0.67 M labels): 12-30 % faster than permutation + walk with one or two batch tiles at any
+    // width; with three or four batch tiles the tile's weights are staged three or four times per tile and the form
+    // breaks even only where the workgroup has at least 11 wavefronts to hide that (N >= 704: -1 % at batch 128,
+    // N = 768, fan-in 32, and 119 MB less memory; N <= 640: +4...17 %); beyond four batch tiles it loses 12-15 %.
+    // Tiles larger than the workgroup (two labels staged per thread) and weights beyond what a thread carries in
+    // registers (8 x 16 bytes) spill or add a round trip: not taken.
+    bool w_in_lds = false;
+    const int nbt_hint = (std::max(batch_hint, 1) + 31) / 32;
+    const bool wanted = nbt_hint <= 2 || (nbt_hint <= 4 && threads >= 704);
+    if (wanted && threads <= 768) {
+        int tw = std::min(TL, threads & ~1);                 // one label per thread to stage
+        while (tw >= 64 && tiled_lds_bytes(tw, K, true) > kPlanLdsBudget) tw -= 2;
+        if (tw >= 64 && (long long)tw * K <= (long long)threads * 32 && 2 * tw >= TL) { TL = tw; w_in_lds = true; }
+    }
+    *weights_in_lds = w_in_lds;
+    return TL;
+}
+
+namespace {
+
 // Builds the tiled form.  Returns FFI_OK with p->tiled == false if the padded size would exceed
 // three times the connection count (heavily skewed column usage): the caller then builds the
 // global form instead.
@@ -368,8 +399,8 @@ int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     // the workgroup is larger than 768 threads and registers are scarcer)
     // (even, so that label parity inside a tile is the parity of the LDS row)
     // and small enough for the positions inside a tile to fit 16 bits
-    const int TL = std::min((std::min(std::min(kPlanTileLabels, p->L), threads > 768 ? threads : 2 * threads) + 1) & ~1,
-                            (int)((kPadPos - 1) / (unsigned)p->K) & ~1);
+    bool w_in_lds = false;
+    const int TL = plan_tile_labels(p->N, p->K, p->L, p->batch_hint, &w_in_lds);
     const int slices = threads / 64;
     const int tiles = (p->L + TL - 1) / TL;
     const size_t nslices = (size_t)tiles * slices;
@@ -379,7 +410,7 @@ int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
         return FFI_ERR_OUT_OF_MEMORY;
     }
     // rows per bank half: half the tile plus some room for the balancing, within the LDS the walking kernel can have
-    const int cap = TL / 2 + std::min(TL / 16, 64);
+    const int cap = tiled_rows_per_half(TL);
     if (!dev_alloc(&p->rowpos, (size_t)p->L)) { (void)hipFree(slice_len); return FFI_ERR_OUT_OF_MEMORY; }
     {
         const size_t lds = 2 * (size_t)threads * sizeof(int) + (size_t)TL * p->K * sizeof(unsigned short);
@@ -407,6 +438,7 @@ int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     if (e == hipSuccess) e = hipStreamSynchronize(s);
     if (e != hipSuccess) return hip_fail(e);
     p->tiled = true;
+    p->w_in_lds = w_in_lds;
     p->tile_labels = TL; p->threads = threads; p->slices = slices; p->tiles = tiles; p->zero_row = 2 * cap;
     p->total_rows = (long long)rows;
     p->bytes = (size_t)rows * 64 * 2 * sizeof(unsigned short) + (nslices + 1) * sizeof(unsigned) + (size_t)p->L * sizeof(unsigned short);
