@@ -163,6 +163,36 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
             const int jl = (int)threadIdx.x + p * nthreads;
             if (jl < nl) load_rows32(g, L, b0, B, (unsigned)(j0 + jl), gbn[p]);
         }
+        const size_t sl = (size_t)t * (nthreads >> 6) + wave;
+        const unsigned row0 = __builtin_amdgcn_readfirstlane(slice_off[sl]);
+        const unsigned rows = __builtin_amdgcn_readfirstlane(slice_off[sl + 1]) - row0;
+        // The slice's first slot rows are requested here, before the barriers and the staging of the tile: they do not
+        // depend on LDS, and their round trip then runs beside that of the tile's rows instead of after it.
+        // Slots are fetched from memory kAhead rows ahead of the multiply-adds that use them, through
+        // buffer loads whose row offset is a scalar (row indices clamped, not predicated, so the loads
+        // carry neither branches nor per-lane address arithmetic).
+        constexpr int kAhead = 4;
+        const unsigned last = rows ? rows - 1 : 0u;     // (an empty slice: the loads land on the next slice's first row, or beyond the buffer, and are not used)
+        auto load_lab = [&](unsigned r) {
+            return (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(lab_rsrc, lane2, (row0 + r) * 128u, 0);
+        };
+        // the slot's weight, or (WLDS) the LDS address of it: positions of padding slots (0xffff) end at the zero word
+        auto load_w = [&](unsigned r) {
+            if (WLDS) {
+                const unsigned pos = (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(wp_rsrc, lane2, (row0 + r) * 128u, 0);
+                return __builtin_bit_cast(float, wsbase + min(pos, tile_w) * 4u);
+            }
+            return buffer_load_f32(wp_rsrc, lane4, (row0 + r) * 256u);
+        };
+        const float w_none = WLDS ? __builtin_bit_cast(float, wsbase + tile_w * 4u) : 0.f;
+        unsigned e4[kAhead];
+        float w4[kAhead];
+#pragma unroll
+        for (int q = 0; q < kAhead; ++q) {
+            const unsigned r = min((unsigned)q, last);
+            e4[q] = load_lab(r);
+            w4[q] = load_w(r);
+        }
         // (WLDS) the tile's block of the weight matrix, contiguous: requested with the rows of out_grad
         float4 wreg[kWRegs];
         const unsigned nw = (unsigned)nl * (unsigned)K;
@@ -210,35 +240,7 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
             }
         }
         __syncthreads();
-        const size_t sl = (size_t)t * (nthreads >> 6) + wave;
-        const unsigned row0 = __builtin_amdgcn_readfirstlane(slice_off[sl]);
-        const unsigned rows = __builtin_amdgcn_readfirstlane(slice_off[sl + 1]) - row0;
         if (rows == 0) continue;               // wave-uniform: no column of this slice is used in the tile
-        // Slots are fetched from memory kAhead rows ahead of the multiply-adds that use them, through
-        // buffer loads whose row offset is a scalar (row indices clamped, not predicated, so the loads
-        // carry neither branches nor per-lane address arithmetic).
-        constexpr int kAhead = 4;
-        const unsigned last = rows - 1;
-        auto load_lab = [&](unsigned r) {
-            return (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(lab_rsrc, lane2, (row0 + r) * 128u, 0);
-        };
-        // the slot's weight, or (WLDS) the LDS address of it: positions of padding slots (0xffff) end at the zero word
-        auto load_w = [&](unsigned r) {
-            if (WLDS) {
-                const unsigned pos = (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(wp_rsrc, lane2, (row0 + r) * 128u, 0);
-                return __builtin_bit_cast(float, wsbase + min(pos, tile_w) * 4u);
-            }
-            return buffer_load_f32(wp_rsrc, lane4, (row0 + r) * 256u);
-        };
-        const float w_none = WLDS ? __builtin_bit_cast(float, wsbase + tile_w * 4u) : 0.f;
-        unsigned e4[kAhead];
-        float w4[kAhead];
-#pragma unroll
-        for (int q = 0; q < kAhead; ++q) {
-            const unsigned r = min((unsigned)q, last);
-            e4[q] = load_lab(r);
-            w4[q] = load_w(r);
-        }
         for (unsigned i = 0; i < rows; i += kAhead) {
             unsigned en[kAhead];
             float wn[kAhead];
@@ -337,11 +339,9 @@ int launch_tiled(const ffi_plan* p, const float* w, const float* g, float* gx, i
     } while (0)
     // the plan sizes its tiles so that one of these fits: tile_labels <= LPT * threads
     if (p->w_in_lds) {
-        if (p->threads <= 768) {
-            if (p->tile_labels <= p->threads) FFI_LAUNCH_TILE(768, 1, true); else FFI_LAUNCH_TILE(768, 2, true);
-        } else {
-            FFI_LAUNCH_TILE(1024, 1, true);
-        }
+        // (plans take that form only with workgroups of at most 768 threads that stage one label each)
+        if (p->threads > 768 || p->tile_labels > p->threads) return FFI_ERR_BAD_ARGUMENT;
+        FFI_LAUNCH_TILE(768, 1, true);
     } else if (p->threads <= 768) {
         if (p->tile_labels <= p->threads) FFI_LAUNCH_TILE(768, 1, false); else FFI_LAUNCH_TILE(768, 2, false);
     } else {
