@@ -489,7 +489,7 @@ int ffi_plan_create(const int32_t* lookup, int64_t num_units, int64_t fan_in, in
     FFI_TRY(check_dims(batch_hint > 0 ? batch_hint : 1, num_features, num_units, fan_in, 0, &d));
     ffi_plan* p = nullptr;
     FFI_TRY(plan_alloc(d.L, d.K, d.N, &p));
-    p->batch_hint = d.B;
+    p->batch_hint = batch_hint > 0 ? d.B : 0;
     int st = plan_build(p, lookup, (hipStream_t)stream);
     if (st != FFI_OK) { plan_free(p); delete p; return st; }
     *plan = p;

@@ -377,8 +377,8 @@ int plan_tile_labels(int N, int K, int L, int batch_hint, bool* weights_in_lds) 
     // Tiles larger than the workgroup (two labels staged per thread) and weights beyond what a thread carries in
     // registers (8 x 16 bytes) spill or add a round trip: not taken.
     bool w_in_lds = false;
-    const int nbt_hint = (std::max(batch_hint, 1) + 31) / 32;
-    const bool wanted = nbt_hint <= 2 || (nbt_hint <= 4 && threads >= 704);
+    const int nbt_hint = (batch_hint + 31) / 32;
+    const bool wanted = batch_hint > 0 && (nbt_hint <= 2 || (nbt_hint <= 4 && threads >= 704));   // (unknown batch size: the form for large batches)
     if (wanted && threads <= 768) {
         int tw = std::min(TL, threads & ~1);                 // one label per thread to stage
         while (tw >= 64 && tiled_lds_bytes(tw, K, true) > kPlanLdsBudget) tw -= 2;

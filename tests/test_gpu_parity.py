@@ -434,6 +434,36 @@ def test_explicit_plan_matches_cached_path(ffi):
         ffi._lib.check(lib.ffi_plan_destroy(plan))
 
 
+@pytest.mark.parametrize("shape", [(768, 3000, 32), (512, 2500, 16), (100, 1800, 21), (300, 1500, 40)])
+def test_plan_layouts_serve_any_batch_size(ffi, shape):
+    # the batch hint picks the plan's layout (small batches: label tiles whose weights the kernel keeps in LDS, no
+    # slot-ordered copy of the weights; large or unknown: 1024-label tiles behind the permutation kernel); either
+    # layout must give the oracle's input gradient at any batch size, bit-identically from call to call
+    N, L, K = shape
+    lib = ffi._lib.lib()
+    for hint in (32, 128, 512, 0):
+        plan = None
+        for B in (20, 150):
+            x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=N + hint)
+            dl, dw, dg = dev(lookup), dev(w), dev(g)
+            if plan is None:
+                plan = ctypes.c_void_p()
+                ffi._lib.check(lib.ffi_plan_create(dl.data_ptr(), L, K, N, hint, stream(), ctypes.byref(plan)))
+                lookup0 = lookup
+            else:
+                lookup, dl = lookup0, dev(lookup0)          # the plan describes the first lookup
+            print(f"case N={N} L={L} K={K} hint={hint} B={B}", flush=True)
+            results = []
+            for _ in range(2):
+                gx = torch.full((B, N), float("nan"), device="cuda")
+                ffi._lib.check(lib.ffi_input_grad_planned_f32(plan, dw.data_ptr(), dg.data_ptr(), gx.data_ptr(), B, 0, stream()))
+                torch.cuda.synchronize()
+                results.append(gx.cpu().numpy())
+            assert np.array_equal(results[0], results[1])
+            assert rel_err(results[0], oracle.input_grad(x, lookup, w, g, transposed=False)) <= GRAD_RTOL
+        ffi._lib.check(lib.ffi_plan_destroy(plan))
+
+
 def test_bad_lookup_is_reported_not_dereferenced(ffi):
     B, N, L, K = 4, 10, 50, 3
     x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=51)
