@@ -120,32 +120,42 @@ __global__ __launch_bounds__(kGuardBlock) void fingerprint_guard_kernel(const in
         unsigned long long hs = 0, bs = 0;
 #pragma unroll
         for (int i = 0; i < kGuardBlock / 64; ++i) { hs += part[0][i]; bs += part[1][i]; }
-        __hip_atomic_store(&guard[8 + 2 * blockIdx.x], hs, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(&guard[9 + 2 * blockIdx.x], bs, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __threadfence();
-        last = atomicAdd(&guard[2], 1ull) == (unsigned long long)gridDim.x - 1;
+        // Published with atomic exchanges whose results are waited for, then the ticket: a read-modify-write at
+        // device scope is carried out where all XCDs see it, and its returned value says that it has been.  (A
+        // fence here would first write back every dirty line of this XCD's L2 -- the scores the forward kernel has
+        // just stored among them -- which was measured to cost a third of the kernel's time.)
+        const unsigned long long o1 = __hip_atomic_exchange(&guard[8 + 2 * blockIdx.x], hs, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned long long o2 = __hip_atomic_exchange(&guard[9 + 2 * blockIdx.x], bs, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        unsigned long long one = 1ull;
+        asm volatile("" : "+v"(one) : "v"(o1), "v"(o2));       // the ticket is not drawn before both exchanges have returned
+        last = __hip_atomic_fetch_add(&guard[2], one, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (unsigned long long)gridDim.x - 1;
     }
     __syncthreads();
     if (!last) return;
-    __threadfence();
-    // the last workgroup: its first wavefront adds the pairs of all workgroups
-    if (threadIdx.x < 64) {
-        unsigned long long hs = 0, bs = 0;
-        for (unsigned i = threadIdx.x; i < gridDim.x; i += 64) {
-            hs += __hip_atomic_load(&guard[8 + 2 * i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            bs += __hip_atomic_load(&guard[9 + 2 * i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
+    // the last workgroup adds the pairs of all workgroups: one load per thread, all in flight together (a loop of
+    // dependent loads per lane costs a memory round trip per step)
+    static_assert(kGuardBlocks <= kGuardBlock, "one thread per pair");
+    unsigned long long hs = 0, bs = 0;
+    if (threadIdx.x < gridDim.x) {
+        hs = __hip_atomic_fetch_add(&guard[8 + 2 * threadIdx.x], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        bs = __hip_atomic_fetch_add(&guard[9 + 2 * threadIdx.x], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
 #pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-            hs += __shfl_down(hs, off);
-            bs += __shfl_down(bs, off);
-        }
-        if (threadIdx.x == 0) {
-            guard[5] = hs;
-            guard[6] = bs;
-            guard[4] = (hs == guard[3] && bs == 0) ? 1ull : 0ull;
-            guard[2] = 0;
-        }
+    for (int off = 32; off > 0; off >>= 1) {
+        hs += __shfl_down(hs, off);
+        bs += __shfl_down(bs, off);
+    }
+    __syncthreads();                                       // (thread 0 has read part[] above)
+    if ((threadIdx.x & 63) == 0) { part[0][threadIdx.x >> 6] = hs; part[1][threadIdx.x >> 6] = bs; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        hs = 0; bs = 0;
+#pragma unroll
+        for (int i = 0; i < kGuardBlock / 64; ++i) { hs += part[0][i]; bs += part[1][i]; }
+        guard[5] = hs;
+        guard[6] = bs;
+        guard[4] = (hs == guard[3] && bs == 0) ? 1ull : 0ull;
+        guard[2] = 0;
     }
 }
 
