@@ -464,6 +464,28 @@ def test_plan_layouts_serve_any_batch_size(ffi, shape):
         ffi._lib.check(lib.ffi_plan_destroy(plan))
 
 
+@pytest.mark.parametrize("shape", [(128, 768, 60_000, 32, True), (32, 768, 40_000, 32, True), (256, 512, 30_000, 64, True),
+                                   (64, 300, 20_000, 12, False), (96, 2000, 5_000, 20, False), (40, 1100, 9_000, 16, True)])
+def test_workspace_estimate_brackets_what_the_library_holds(ffi, shape):
+    # ffi_workspace_bytes() is asked before anything is allocated; ffi_cache_bytes() says what forward + backward then
+    # hold (plans + workspaces).  The estimate models the padding of the plan for uniformly drawn ids.
+    B, N, L, K, tp = shape
+    lib = ffi._lib.lib()
+    torch.cuda.synchronize()
+    ffi._lib.check(lib.ffi_cache_clear())
+    assert lib.ffi_cache_bytes() == 0
+    estimate = lib.ffi_workspace_bytes(B, N, L, K, int(tp), 3)
+    x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=L)
+    xin = np.ascontiguousarray(x.T) if tp else x
+    hip_forward(ffi, xin, lookup, w, tp)
+    hip_backward(ffi, xin, lookup, w, g, tp)
+    held = lib.ffi_cache_bytes()
+    print(f"case shape={shape} estimate={estimate} held={held}", flush=True)
+    assert held > 0 and 0.8 * held <= estimate <= 1.3 * held + (1 << 20)
+    ffi._lib.check(lib.ffi_cache_clear())
+    assert lib.ffi_cache_bytes() == 0
+
+
 def test_bad_lookup_is_reported_not_dereferenced(ffi):
     B, N, L, K = 4, 10, 50, 3
     x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=51)
