@@ -228,12 +228,14 @@ struct ffi_plan {
     hipEvent_t fp_done = nullptr;             // recorded behind the fingerprint kernel and its copy to h_scratch
     int fp_blocks = 0;                        // workgroups of the fingerprint kernel in flight: that many pairs of partial sums
     // Check of the lookup's content on the device, without a host wait (plan_guard_*): device words
-    // {running sum, running count of bad ids, workgroups finished, expected fingerprint, verdict (1 = the plan is
-    // current), fingerprint found, bad ids found}; the last three are copied to the pinned mirror behind every check
+    // {unused, unused, workgroups finished, expected fingerprint, verdict (1 = the plan is current), fingerprint found,
+    // bad ids found, unused, then a pair of partial sums per workgroup}; the pinned mirror holds one word that the
+    // check writes last: (number of the check << 2) | (verdict << 1) | (bad ids seen)
     unsigned long long* d_guard = nullptr;
     unsigned long long* h_guard = nullptr;
-    hipEvent_t guard_done = nullptr;          // recorded behind that copy
-    bool guard_pending = false;               // a check has been enqueued whose result the host has not looked at
+    hipEvent_t guard_done = nullptr;          // orders checks of one plan that come in on different streams
+    unsigned long long guard_seq = 0;         // checks enqueued so far
+    unsigned long long guard_seen = 0;        // number of the last check whose result the host has looked at
     hipStream_t guard_stream = nullptr;       // the stream of that check
     size_t bytes = 0;
     int batch_hint = 0;                       // batch size the plan is expected to be used with (0 = unknown); steers layout choices only
