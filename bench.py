@@ -86,8 +86,10 @@ def time_kernel(fn, stream, iters):
     import torch
     start = torch.cuda.Event(enable_timing=True)
     stop = torch.cuda.Event(enable_timing=True)
-    fn()
-    stream.synchronize()
+    # untimed calls first, with no host wait between them and the timed ones: the GPU's clocks take tens of
+    # milliseconds of continuous load to settle, and a pass timed from idle reads 3-8 % slow
+    for _ in range(max(1, iters // 4)):
+        fn()
     start.record(stream)
     for _ in range(iters):
         fn()
