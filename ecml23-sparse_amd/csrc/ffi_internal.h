@@ -233,9 +233,9 @@ struct ffi_plan {
     // check writes last: (number of the check << 2) | (verdict << 1) | (bad ids seen)
     unsigned long long* d_guard = nullptr;
     unsigned long long* h_guard = nullptr;
-    hipEvent_t guard_done = nullptr;          // orders checks of one plan that come in on different streams
     unsigned long long guard_seq = 0;         // checks enqueued so far
     unsigned long long guard_seen = 0;        // number of the last check whose result the host has looked at
+    bool guard_stale = false;                 // such a look found the plan outdated and nobody has acted on it yet
     hipStream_t guard_stream = nullptr;       // the stream of that check
     size_t bytes = 0;
     int batch_hint = 0;                       // batch size the plan is expected to be used with (0 = unknown); steers layout choices only

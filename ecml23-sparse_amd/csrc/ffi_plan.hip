@@ -618,7 +618,6 @@ int plan_scratch_alloc(ffi_plan* p) {
                     hipMemset(p->d_scratch, 0, kScratchWords * sizeof(unsigned long long)) == hipSuccess &&
                     hipMalloc(&p->d_guard, kGuardWords * sizeof(unsigned long long)) == hipSuccess &&
                     hipHostMalloc(&p->h_guard, 8 * sizeof(unsigned long long)) == hipSuccess &&
-                    hipEventCreateWithFlags(&p->guard_done, hipEventDisableTiming) == hipSuccess &&
                     hipMemset(p->d_guard, 0, kGuardWords * sizeof(unsigned long long)) == hipSuccess;
     if (!ok) {
         (void)hipGetLastError();
@@ -681,6 +680,7 @@ int plan_build(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     FFI_HIP_TRY(hipMemcpy(p->d_guard, guard_init, sizeof(guard_init), hipMemcpyHostToDevice));
     // checks enqueued before this build (all finished: the build synchronises) are of no interest any more
     p->guard_seen = p->guard_seq;
+    p->guard_stale = false;
     return FFI_OK;
 }
 
@@ -714,11 +714,15 @@ int plan_build_arrays(ffi_plan* p, const int32_t* lookup, hipStream_t s, unsigne
 }  // namespace
 
 int plan_guard_enqueue(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
-    // a check of this plan that may still be running on another stream shares the accumulators: order the two (an
-    // event recorded now on that stream fires behind everything it holds, the check included)
+    // A check of this plan that may still be running on another stream shares the accumulators: the two must not
+    // overlap.  The other stream's handle may be gone by now (its owner may have destroyed it), so it is not touched:
+    // the host waits for the device.  Only a lookup used from two streams in turn pays this, once per switch.
     if (p->guard_seq != p->guard_seen && p->guard_stream != s) {
-        FFI_HIP_TRY(hipEventRecord(p->guard_done, p->guard_stream));
-        FFI_HIP_TRY(hipStreamWaitEvent(s, p->guard_done, 0));
+        FFI_HIP_TRY(hipDeviceSynchronize());
+        bool seen = false, current = true;
+        unsigned long long bad = 0;
+        (void)plan_guard_poll(p, &seen, &current, &bad);          // (the result stays with the next check if it was bad)
+        if (seen && !current) p->guard_stale = true;
     }
     const size_t total = (size_t)p->L * p->K;
     const unsigned blocks = (unsigned)std::min<size_t>((total / 4 + kGuardBlock - 1) / kGuardBlock + 1, kGuardBlocks);
@@ -734,6 +738,11 @@ int plan_guard_enqueue(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
 
 int plan_guard_poll(ffi_plan* p, bool* seen, bool* current, unsigned long long* bad_ids) {
     *seen = false;
+    if (p->guard_stale) {                                  // an outdated verdict met while switching streams
+        p->guard_stale = false;
+        *seen = true; *current = false; *bad_ids = 0;
+        return FFI_OK;
+    }
     if (p->guard_seq == p->guard_seen) return FFI_OK;
     // the last check that has finished (checks of a plan finish in the order they were enqueued)
     const unsigned long long word = __atomic_load_n(p->h_guard, __ATOMIC_ACQUIRE);
@@ -754,9 +763,8 @@ void plan_free(ffi_plan* p) {
     if (p->fp_done) (void)hipEventDestroy(p->fp_done);
     if (p->d_guard) (void)hipFree(p->d_guard);
     if (p->h_guard) (void)hipHostFree(p->h_guard);
-    if (p->guard_done) (void)hipEventDestroy(p->guard_done);
     p->d_scratch = nullptr; p->h_scratch = nullptr; p->fp_done = nullptr;
-    p->d_guard = nullptr; p->h_guard = nullptr; p->guard_done = nullptr; p->guard_seq = 0; p->guard_seen = 0;
+    p->d_guard = nullptr; p->h_guard = nullptr; p->guard_seq = 0; p->guard_seen = 0; p->guard_stale = false;
 }
 
 }  // namespace ffi

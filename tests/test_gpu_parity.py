@@ -383,6 +383,38 @@ def test_stateless_backward_does_not_wait_for_the_device(ffi):
         assert rel_err(gw.cpu().numpy(), ref_gw) <= GRAD_RTOL
 
 
+def test_one_lookup_used_from_two_streams_in_turn(ffi):
+    # the checks of a cached plan share their accumulators; calls that come in on alternating streams must not let two
+    # of them overlap, and an in-place edit of the lookup between them is still picked up
+    B, N, L, K = 64, 256, 30_000, 16
+    x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=77)
+    dx, dl, dw, dg = dev(x), dev(lookup), dev(w), dev(g)
+    lib = ffi._lib.lib()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    torch.cuda.synchronize()
+    gx = [torch.empty((B, N), device="cuda") for _ in streams]
+    gw = [torch.empty((L, K), device="cuda") for _ in streams]
+    ref_gx, ref_gw = oracle.backward(x, lookup, w, g, transposed=False)
+    for rnd in range(6):
+        if rnd == 3:                                       # rewire in place: a fifth of the rows get new columns
+            torch.cuda.synchronize()
+            rng = np.random.default_rng(5)
+            rows = rng.choice(L, L // 5, replace=False)
+            lookup = lookup.copy()
+            lookup[rows] = rng.integers(0, N, (rows.size, K)).astype(np.int32)
+            dl.copy_(torch.from_numpy(lookup))
+            torch.cuda.synchronize()
+            ref_gx, ref_gw = oracle.backward(x, lookup, w, g, transposed=False)
+        for i, st in enumerate(streams):
+            print(f"case round={rnd} stream={i}", flush=True)
+            ffi._lib.check(lib.ffi_backward_f32(dx.data_ptr(), dl.data_ptr(), dw.data_ptr(), dg.data_ptr(), gx[i].data_ptr(),
+                                                 gw[i].data_ptr(), B, N, L, K, 0, st.cuda_stream))
+        torch.cuda.synchronize()
+        for i in range(2):
+            assert rel_err(gx[i].cpu().numpy(), ref_gx) <= GRAD_RTOL, (rnd, i)
+            assert rel_err(gw[i].cpu().numpy(), ref_gw) <= GRAD_RTOL, (rnd, i)
+
+
 def test_plan_is_unusable_after_a_failed_refresh(ffi):
     # a rebuild that fails (here: an id out of range) leaves a plan without arrays; calls through it are refused
     # with a status instead of walking freed memory
