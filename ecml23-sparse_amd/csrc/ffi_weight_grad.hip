@@ -167,6 +167,7 @@ __global__ __launch_bounds__(kResThreads) void wgrad_resident_kernel(const float
 // slot before they are stored.
 // ------------------------------------------------------------------------------------------------
 constexpr unsigned kArrIdMask = (1u << kArrIdBits) - 1;
+constexpr int kSlotPitch = kWgChunk + 4;     // floats between the reordering slots of neighbouring threads (16-byte aligned)
 
 __global__ __launch_bounds__(kResThreads) void wgrad_arranged_kernel(const float* __restrict__ xT,
                                                                      const unsigned short* __restrict__ idx16,
@@ -234,8 +235,10 @@ __global__ __launch_bounds__(kResThreads) void wgrad_arranged_kernel(const float
             }
         }
     }
-    __syncthreads();                                       // xs is free: its first 64 KB become per-thread slots
-    float* slot = xs + (size_t)threadIdx.x * kWgChunk;
+    __syncthreads();                                       // xs is free: its first 72 KB become per-thread slots
+    // (a pitch of 36 floats: when the connection numbers are the same in every lane -- a lookup that is already in the
+    // arranged order has them 0, 1, 2, ... -- a pitch of 32 would send all lanes of a write to two banks)
+    float* slot = xs + (size_t)threadIdx.x * kSlotPitch;
     const bool vec4 = (K % 4 == 0) && (((uintptr_t)gw & 15) == 0);
 #pragma unroll
     for (int q = 0; q < kResUnits; ++q) {
@@ -291,8 +294,8 @@ int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float
         const unsigned blocks = (unsigned)(n1 + n2);
         const int upb = (int)cap;
         if (plan != nullptr && plan->idx16 != nullptr) {
-            // the unit slots of the final reordering need 128 bytes per thread
-            const size_t lds = std::max(tile_lds_bytes(d.N), (size_t)kResThreads * kWgChunk * sizeof(float));
+            // the unit slots of the final reordering need 144 bytes per thread
+            const size_t lds = std::max(tile_lds_bytes(d.N), (size_t)kResThreads * kSlotPitch * sizeof(float));
             FFI_HIP_TRY(hipFuncSetAttribute((const void*)wgrad_arranged_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
             hipLaunchKernelGGL(wgrad_arranged_kernel, dim3(blocks), dim3(kResThreads), lds, s, xT, plan->idx16, g, gw, bias_grad, d.B, d.N, d.L, d.K, nchunks, n1, upb, upb2);
             FFI_HIP_TRY(hipGetLastError());
