@@ -171,7 +171,7 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
         // Slots are fetched from memory kAhead rows ahead of the multiply-adds that use them, through
         // buffer loads whose row offset is a scalar (row indices clamped, not predicated, so the loads
         // carry neither branches nor per-lane address arithmetic).
-        constexpr int kAhead = 4;
+        constexpr int kAhead = MAXT <= 768 ? 6 : 4;     // (six rows ahead: 0.9 % of the whole step at 670,091 labels; the 1024-thread form has the registers for four)
         const unsigned last = rows ? rows - 1 : 0u;     // (an empty slice: the loads land on the next slice's first row, or beyond the buffer, and are not used)
         auto load_lab = [&](unsigned r) {
             return (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(lab_rsrc, lane2, (row0 + r) * 128u, 0);
