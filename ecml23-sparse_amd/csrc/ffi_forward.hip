@@ -124,7 +124,7 @@ __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* _
     const int u = xcd_contiguous_block(blockIdx.x, gridDim.x);
     const int bt = u % nbt, stream = u / nbt;
     const int b0 = bt * kTileBatch;
-    stage_rows32<kTileThreads>(xs, xT, N, B, b0);
+    stage_rows32<kTileThreads, 8>(xs, xT, N, B, b0);       // (eight loads in flight per thread: the tile arrives in one round trip at 768 rows)
     if (TOPK && threadIdx.x < kTileBatch) local_count[threadIdx.x] = 0;
     if (TOPK && threadIdx.x < kTileBatch)          // rows past the batch never qualify
         tau_s[threadIdx.x] = b0 + (int)threadIdx.x < B ? ft.tau[(size_t)(b0 + threadIdx.x) * ft.tau_stride] : __builtin_inff();
