@@ -158,10 +158,15 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
         // out_grad rows of this tile: requested before the barrier, so the loads are in flight
         // while the slower wavefronts finish the previous tile
         float gbn[LPT][32];
+        unsigned rowp_of[LPT];                   // the LDS row of each staged label (the plan's choice), fetched with its out_grad values
 #pragma unroll
         for (int p = 0; p < LPT; ++p) {
             const int jl = (int)threadIdx.x + p * nthreads;
-            if (jl < nl) load_rows32(g, L, b0, B, (unsigned)(j0 + jl), gbn[p]);
+            rowp_of[p] = 0;
+            if (jl < nl) {
+                load_rows32(g, L, b0, B, (unsigned)(j0 + jl), gbn[p]);
+                rowp_of[p] = rowpos[j0 + jl];
+            }
         }
         const size_t sl = (size_t)t * (nthreads >> 6) + wave;
         const unsigned row0 = __builtin_amdgcn_readfirstlane(slice_off[sl]);
@@ -232,7 +237,7 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
                 const int r = jl & 7;
                 xor_permute_groups(gbn[p], r);
                 // the label's row in LDS is the plan's choice (it balances the bank halves of every column)
-                char* rowp = gs_bytes + ((unsigned)rowpos[j0 + jl] << 7);
+                char* rowp = gs_bytes + (rowp_of[p] << 7);
 #pragma unroll
                 for (int c = 0; c < 8; ++c)
                     *reinterpret_cast<float4*>(rowp + ((c ^ r) << 4)) =
