@@ -181,11 +181,11 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
         auto load_lab = [&](unsigned r) {
             return (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(lab_rsrc, lane2, (row0 + r) * 128u, 0);
         };
-        // the slot's weight, or (WLDS) the LDS address of it: positions of padding slots (0xffff) end at the zero word
+        // the slot's weight, or (WLDS) the LDS address of it
         auto load_w = [&](unsigned r) {
             if (WLDS) {
                 const unsigned pos = (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(wp_rsrc, lane2, (row0 + r) * 128u, 0);
-                return __builtin_bit_cast(float, wsbase + min(pos, tile_w) * 4u);
+                return __builtin_bit_cast(float, wsbase + pos * 4u);     // (padding slots hold tile_w, the zero word)
             }
             return buffer_load_f32(wp_rsrc, lane4, (row0 + r) * 256u);
         };

@@ -285,12 +285,13 @@ __global__ __launch_bounds__(1024) void slice_scan_kernel(const unsigned* __rest
 // in chunks; every thread scans them in flat-position order and places the ones equal to its
 // column (see column_slots for the order), so the result is deterministic without any sort.
 // Per slot: lab16 = LDS row of the label (rowpos), pos16 = position inside the tile's rows of lookup; the
-// slots a column leaves empty up to the slice's length become padding: pos16 = kPadPos, lab16 =
+// slots a column leaves empty up to the slice's length become padding: pos16 = pad_pos (kPadPos; in plans whose walking
+// kernel keeps the tile's weights in LDS, tile_labels * K: the position of a zero word behind them), lab16 =
 // zero_row + parity (all-zero rows).
 constexpr int kFillChunk = 8192;
 __global__ void tile_fill_kernel(const int32_t* __restrict__ idx, const unsigned short* __restrict__ rowpos, int L, int K,
                                  int tile_labels, int zero_row, const unsigned* __restrict__ slice_off,
-                                 unsigned short* __restrict__ lab16, unsigned short* __restrict__ pos16) {
+                                 unsigned short* __restrict__ lab16, unsigned short* __restrict__ pos16, unsigned pad_pos) {
     __shared__ __align__(16) int keys[kFillChunk];
     __shared__ unsigned short rows_of[kPlanTileLabels];     // LDS row of each label of the tile
     const int t = blockIdx.x, nthreads = blockDim.x;
@@ -309,7 +310,7 @@ __global__ void tile_fill_kernel(const int32_t* __restrict__ idx, const unsigned
     // padding everywhere first; the thread's own slots are then overwritten (same thread: ordered)
     for (unsigned r = 0; r < rows; ++r) {
         dlab[(size_t)r * 64] = (unsigned short)((unsigned)zero_row + ((r & 1u) ^ first));
-        dpos[(size_t)r * 64] = (unsigned short)kPadPos;
+        dpos[(size_t)r * 64] = (unsigned short)pad_pos;
     }
     unsigned seen[2] = {0u, 0u};  // labels of each parity placed so far
     int label = 0, kk = 0;        // label and connection slot of the entry under the cursor
@@ -450,7 +451,7 @@ int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     if (rows * 64ull > 3ull * connections + 64ull * nslices || rows >= (1ull << 24)) return FFI_OK;
     if (!dev_alloc(&p->lab16, (size_t)rows * 64) || !dev_alloc(&p->pos16, (size_t)rows * 64)) return FFI_ERR_OUT_OF_MEMORY;
     hipLaunchKernelGGL(tile_fill_kernel, dim3(tiles), dim3(threads), 0, s, lookup, p->rowpos, p->L, p->K, TL, 2 * cap, p->slice_off,
-                       p->lab16, p->pos16);
+                       p->lab16, p->pos16, w_in_lds ? (unsigned)TL * (unsigned)p->K : kPadPos);
     e = hipGetLastError();
     if (e == hipSuccess) e = hipStreamSynchronize(s);
     if (e != hipSuccess) return hip_fail(e);
