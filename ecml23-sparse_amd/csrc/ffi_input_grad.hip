@@ -184,12 +184,13 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
         // the slot's weight, or (WLDS) the LDS address of it
         auto load_w = [&](unsigned r) {
             if (WLDS) {
-                const unsigned pos = (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(wp_rsrc, lane2, (row0 + r) * 128u, 0);
-                return __builtin_bit_cast(float, wsbase + pos * 4u);     // (padding slots hold tile_w, the zero word)
+                // the position itself: turned into the weight's LDS address where it is used, a group of rows later, so that
+                // nothing waits for this load here (padding slots hold tile_w, the zero word)
+                return __builtin_bit_cast(float, (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(wp_rsrc, lane2, (row0 + r) * 128u, 0));
             }
             return buffer_load_f32(wp_rsrc, lane4, (row0 + r) * 256u);
         };
-        const float w_none = WLDS ? __builtin_bit_cast(float, wsbase + tile_w * 4u) : 0.f;
+        const float w_none = WLDS ? __builtin_bit_cast(float, tile_w) : 0.f;
         unsigned e4[kAhead];
         float w4[kAhead];
 #pragma unroll
@@ -265,7 +266,7 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
                 const bool in = i + q < rows;                       // wave-uniform
                 const unsigned e = in ? e4[q] : (unsigned)zero_row;
                 float wv = in ? w4[q] : w_none;
-                if (WLDS) wv = *(const float __attribute__((address_space(3)))*)(size_t)__builtin_bit_cast(unsigned, wv);
+                if (WLDS) wv = *(const float __attribute__((address_space(3)))*)(size_t)(wsbase + __builtin_bit_cast(unsigned, wv) * 4u);
                 float4 xv[8];
                 igrad_reads(e, skewbase, xv);
                 igrad_fmas(xv, wv, acc);
