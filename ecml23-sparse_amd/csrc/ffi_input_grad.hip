@@ -96,6 +96,12 @@ __device__ __forceinline__ float4 igrad_read_chunk(unsigned base) {
     const lds_v4f t = *(lds_v4f_ptr)(size_t)(skew_addr<C>(base));
     return make_float4(t.x, t.y, t.z, t.w);
 }
+__device__ __forceinline__ void igrad_reads_at(unsigned base, float4 (&v)[8]) {
+    v[0] = igrad_read_chunk<0>(base); v[1] = igrad_read_chunk<1>(base);
+    v[2] = igrad_read_chunk<2>(base); v[3] = igrad_read_chunk<3>(base);
+    v[4] = igrad_read_chunk<4>(base); v[5] = igrad_read_chunk<5>(base);
+    v[6] = igrad_read_chunk<6>(base); v[7] = igrad_read_chunk<7>(base);
+}
 __device__ __forceinline__ void igrad_reads(unsigned e, unsigned skewbase, float4 (&v)[8]) {
     const unsigned base = (e << 7) + skewbase;
     v[0] = igrad_read_chunk<0>(base); v[1] = igrad_read_chunk<1>(base);
@@ -117,7 +123,8 @@ __device__ __forceinline__ void igrad_fmas(const float4 (&v)[8], float wv, float
 // partial[stream][n][b] over the stream's tiles.  grid = streams * batch tiles.
 // MAXT: largest workgroup the instantiation is launched with (sets the register budget);
 // LPT: labels of a tile staged per thread (tile_labels <= LPT * blockDim.x).
-// WLDS: `wp` is the weight matrix itself and `pos16` the slots' positions in their tile's [tile_labels][K] block of it:
+// WLDS: `wp` is the weight matrix itself and `slot32` holds one word per slot, (position in the tile's [tile_labels][K]
+// block of the weights << 17) | (LDS row << 7), in place of lab16:
 // the tile's weights are staged in LDS behind the rows of out_grad (with a zero word at tile_labels * K that
 // padding slots read) and every slot fetches its weight from there, so no slot-ordered copy of the weights exists.
 template <int MAXT, int LPT, bool WLDS>
@@ -126,7 +133,7 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
                                   const float* __restrict__ g, float* __restrict__ partial, int B, int L,
                                   int tile_labels, int tiles, int tiles_per_stream, int nbt, unsigned total_rows,
                                   const unsigned short* __restrict__ rowpos, int zero_row,
-                                  const unsigned short* __restrict__ pos16, int K) {
+                                  const unsigned* __restrict__ slot32, int K) {
     extern __shared__ __align__(16) float gs[];
     char* gs_bytes = reinterpret_cast<char*>(gs);
     const int nthreads = blockDim.x;
@@ -139,8 +146,8 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
     const unsigned skewbase = (unsigned)(size_t)(__attribute__((address_space(3))) float*)gs + skew;
     const int t_begin = stream * tiles_per_stream, t_end = min(t_begin + tiles_per_stream, tiles);
     // plan slots and permuted weights, addressed as (scalar row offset) + (lane offset); 4-GB buffers at most
-    const buffer_rsrc lab_rsrc = make_rsrc(lab16, (size_t)total_rows * 128u);
-    const buffer_rsrc wp_rsrc = WLDS ? make_rsrc(pos16, (size_t)total_rows * 128u) : make_rsrc(wp, (size_t)total_rows * 256u);
+    const buffer_rsrc lab_rsrc = WLDS ? make_rsrc(slot32, (size_t)total_rows * 256u) : make_rsrc(lab16, (size_t)total_rows * 128u);
+    const buffer_rsrc wp_rsrc = make_rsrc(wp, WLDS ? 0 : (size_t)total_rows * 256u);
     const unsigned lane2 = (unsigned)lane * 2u, lane4 = (unsigned)lane * 4u;
     // (WLDS) the tile's weights behind the rows of out_grad and the two zero rows
     float* ws = gs + (size_t)(zero_row + 2) * kTileBatch;
@@ -178,19 +185,15 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
         // carry neither branches nor per-lane address arithmetic).
         constexpr int kAhead = MAXT <= 768 ? 6 : 4;     // (six rows ahead: 0.9 % of the whole step at 670,091 labels; the 1024-thread form has the registers for four)
         const unsigned last = rows ? rows - 1 : 0u;     // (an empty slice: the loads land on the next slice's first row, or beyond the buffer, and are not used)
+        // per slot: the label's LDS row and the weight (the forms whose weights are in slot order), or (WLDS) the packed
+        // word whose bits 7..16 are the row's byte offset and whose bits 17..31 are the weight's position
         auto load_lab = [&](unsigned r) {
+            if (WLDS) return (unsigned)__builtin_amdgcn_raw_buffer_load_b32(lab_rsrc, lane4, (row0 + r) * 256u, 0);
             return (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(lab_rsrc, lane2, (row0 + r) * 128u, 0);
         };
-        // the slot's weight, or (WLDS) the LDS address of it
-        auto load_w = [&](unsigned r) {
-            if (WLDS) {
-                // the position itself: turned into the weight's LDS address where it is used, a group of rows later, so that
-                // nothing waits for this load here (padding slots hold tile_w, the zero word)
-                return __builtin_bit_cast(float, (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(wp_rsrc, lane2, (row0 + r) * 128u, 0));
-            }
-            return buffer_load_f32(wp_rsrc, lane4, (row0 + r) * 256u);
-        };
-        const float w_none = WLDS ? __builtin_bit_cast(float, tile_w) : 0.f;
+        auto load_w = [&](unsigned r) { return WLDS ? 0.f : buffer_load_f32(wp_rsrc, lane4, (row0 + r) * 256u); };
+        // (WLDS) rows past the end of the slice: the zero row and the zero word behind the tile's weights
+        const unsigned e_none = WLDS ? (tile_w << 17) | ((unsigned)zero_row << 7) : (unsigned)zero_row;
         unsigned e4[kAhead];
         float w4[kAhead];
 #pragma unroll
@@ -264,11 +267,17 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
 #pragma unroll
             for (int q = 0; q < kAhead; ++q) {
                 const bool in = i + q < rows;                       // wave-uniform
-                const unsigned e = in ? e4[q] : (unsigned)zero_row;
-                float wv = in ? w4[q] : w_none;
-                if (WLDS) wv = *(const float __attribute__((address_space(3)))*)(size_t)(wsbase + __builtin_bit_cast(unsigned, wv) * 4u);
+                const unsigned e = in ? e4[q] : e_none;
+                float wv = in ? w4[q] : 0.f;
                 float4 xv[8];
-                igrad_reads(e, skewbase, xv);
+                if (WLDS) {
+                    // (the tile starts at LDS address 0 -- the kernel has no other LDS -- so the row's byte offset and the
+                    // lane's skew, which share no bit, combine with an OR: one instruction with the mask)
+                    wv = *(const float __attribute__((address_space(3)))*)(size_t)(wsbase + (e >> 17) * 4u);
+                    igrad_reads_at((e & 0x1ff80u) | skewbase, xv);
+                } else {
+                    igrad_reads(e, skewbase, xv);
+                }
                 igrad_fmas(xv, wv, acc);
             }
 #pragma unroll
@@ -341,7 +350,7 @@ int launch_tiled(const ffi_plan* p, const float* w, const float* g, float* gx, i
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));                        \
         hipLaunchKernelGGL((igrad_tile_kernel<MAXT, LPT, WLDS>), grid, block, lds, s, p->lab16, WLDS ? w : wp, p->slice_off, g, \
                            partial, B, p->L, p->tile_labels, p->tiles, tps, nbt, (unsigned)p->total_rows, p->rowpos, p->zero_row, \
-                           p->pos16, p->K);                                                                             \
+                           p->slot32, p->K);                                                                             \
     } while (0)
     // the plan sizes its tiles so that one of these fits: tile_labels <= LPT * threads
     if (p->w_in_lds) {
@@ -371,7 +380,7 @@ int launch_input_grad(const ffi_plan* p, const float* w, const float* g, float* 
     // (a plan whose last build failed holds no arrays)
     if (p->lookup == nullptr) return FFI_ERR_BAD_ARGUMENT;
     if (p->tiled) {
-        if (!p->lab16 || !p->pos16 || !p->slice_off || !p->rowpos) return FFI_ERR_BAD_ARGUMENT;
+        if (!p->slice_off || !p->rowpos || (p->w_in_lds ? !p->slot32 : (!p->lab16 || !p->pos16))) return FFI_ERR_BAD_ARGUMENT;
         if (zeroed_if_outdated) *zeroed_if_outdated = verdict != nullptr;
         return launch_tiled(p, w, g, gx, B, tp, s, verdict);
     }

@@ -212,6 +212,7 @@ struct ffi_plan {
                                          // padding slots hold zero_row + parity (two all-zero rows)
     unsigned short* rowpos = nullptr;    // [L] LDS row each label is staged into, inside its tile (see ffi_plan.hip)
     int zero_row = 0;                    // first of the two all-zero rows = rows of the tile in LDS before them
+    unsigned* slot32 = nullptr;          // plans with w_in_lds, instead of lab16 and pos16: [total_rows*64] (position << 17) | (LDS row << 7)
     unsigned short* pos16 = nullptr;     // [total_rows*64] position (inside the tile's rows of lookup) of each slot;
                                          // kPadPos in padding slots
     // arranged copy of the column ids for the weight gradient (narrow inputs only, else null):

@@ -289,9 +289,12 @@ __global__ __launch_bounds__(1024) void slice_scan_kernel(const unsigned* __rest
 // kernel keeps the tile's weights in LDS, tile_labels * K: the position of a zero word behind them), lab16 =
 // zero_row + parity (all-zero rows).
 constexpr int kFillChunk = 8192;
+// With `slot32` (plans whose walking kernel keeps the tile's weights in LDS) the two go into one word per slot,
+// (position << 17) | (LDS row << 7): one load per slot, the row's byte offset already in place.
 __global__ void tile_fill_kernel(const int32_t* __restrict__ idx, const unsigned short* __restrict__ rowpos, int L, int K,
                                  int tile_labels, int zero_row, const unsigned* __restrict__ slice_off,
-                                 unsigned short* __restrict__ lab16, unsigned short* __restrict__ pos16, unsigned pad_pos) {
+                                 unsigned short* __restrict__ lab16, unsigned short* __restrict__ pos16, unsigned pad_pos,
+                                 unsigned* __restrict__ slot32) {
     __shared__ __align__(16) int keys[kFillChunk];
     __shared__ unsigned short rows_of[kPlanTileLabels];     // LDS row of each label of the tile
     const int t = blockIdx.x, nthreads = blockDim.x;
@@ -303,14 +306,16 @@ __global__ void tile_fill_kernel(const int32_t* __restrict__ idx, const unsigned
     const size_t sl = (size_t)t * (nthreads >> 6) + (threadIdx.x >> 6);
     const size_t row0 = slice_off[sl];
     const unsigned rows = slice_off[sl + 1] - slice_off[sl];
-    unsigned short* dlab = lab16 + row0 * 64 + (threadIdx.x & 63);
-    unsigned short* dpos = pos16 + row0 * 64 + (threadIdx.x & 63);
+    const size_t at = row0 * 64 + (threadIdx.x & 63);
+    auto put = [&](size_t r, unsigned lab, unsigned pos) {
+        if (slot32 != nullptr) slot32[at + r * 64] = (pos << 17) | (lab << 7);
+        else { lab16[at + r * 64] = (unsigned short)lab; pos16[at + r * 64] = (unsigned short)pos; }
+    };
     const unsigned first = parity_first(threadIdx.x);
     for (int i = threadIdx.x; i < nl; i += nthreads) rows_of[i] = rowpos[j0 + i];
     // padding everywhere first; the thread's own slots are then overwritten (same thread: ordered)
     for (unsigned r = 0; r < rows; ++r) {
-        dlab[(size_t)r * 64] = (unsigned short)((unsigned)zero_row + ((r & 1u) ^ first));
-        dpos[(size_t)r * 64] = (unsigned short)pad_pos;
+        put(r, (unsigned)zero_row + ((r & 1u) ^ first), pad_pos);
     }
     unsigned seen[2] = {0u, 0u};  // labels of each parity placed so far
     int label = 0, kk = 0;        // label and connection slot of the entry under the cursor
@@ -325,8 +330,7 @@ __global__ void tile_fill_kernel(const int32_t* __restrict__ idx, const unsigned
                 const unsigned par = row & 1u;
                 const unsigned t2 = par ? seen[1]++ : seen[0]++;
                 const unsigned slot = 2u * t2 + (par ^ first);
-                dlab[(size_t)slot * 64] = (unsigned short)row;
-                dpos[(size_t)slot * 64] = (unsigned short)(c0 + e);
+                put(slot, row, (unsigned)(c0 + e));
             }
             if (++kk == K) { kk = 0; ++label; }
         }
@@ -360,10 +364,11 @@ void free_arrays(ffi_plan* p) {
     if (p->slice_off) (void)hipFree(p->slice_off);
     if (p->lab16) (void)hipFree(p->lab16);
     if (p->pos16) (void)hipFree(p->pos16);
+    if (p->slot32) (void)hipFree(p->slot32);
     if (p->idx16) (void)hipFree(p->idx16);
     if (p->rowpos) (void)hipFree(p->rowpos);
     p->rowpos = nullptr;
-    p->perm = nullptr; p->col_ptr = nullptr; p->slice_off = nullptr; p->lab16 = nullptr; p->pos16 = nullptr; p->idx16 = nullptr;
+    p->perm = nullptr; p->col_ptr = nullptr; p->slice_off = nullptr; p->lab16 = nullptr; p->pos16 = nullptr; p->slot32 = nullptr; p->idx16 = nullptr;
     p->tiled = false; p->w_in_lds = false; p->total_rows = 0; p->bytes = 0;
 }
 
@@ -449,9 +454,13 @@ int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     const unsigned long long connections = (unsigned long long)p->L * p->K;
     // too skewed, or beyond what the walking kernel's 32-bit buffer offsets reach (256 bytes per row)
     if (rows * 64ull > 3ull * connections + 64ull * nslices || rows >= (1ull << 24)) return FFI_OK;
-    if (!dev_alloc(&p->lab16, (size_t)rows * 64) || !dev_alloc(&p->pos16, (size_t)rows * 64)) return FFI_ERR_OUT_OF_MEMORY;
+    if (w_in_lds) {
+        if (!dev_alloc(&p->slot32, (size_t)rows * 64)) return FFI_ERR_OUT_OF_MEMORY;
+    } else if (!dev_alloc(&p->lab16, (size_t)rows * 64) || !dev_alloc(&p->pos16, (size_t)rows * 64)) {
+        return FFI_ERR_OUT_OF_MEMORY;
+    }
     hipLaunchKernelGGL(tile_fill_kernel, dim3(tiles), dim3(threads), 0, s, lookup, p->rowpos, p->L, p->K, TL, 2 * cap, p->slice_off,
-                       p->lab16, p->pos16, w_in_lds ? (unsigned)TL * (unsigned)p->K : kPadPos);
+                       p->lab16, p->pos16, w_in_lds ? (unsigned)TL * (unsigned)p->K : kPadPos, p->slot32);
     e = hipGetLastError();
     if (e == hipSuccess) e = hipStreamSynchronize(s);
     if (e != hipSuccess) return hip_fail(e);
@@ -691,7 +700,7 @@ int plan_build_arrays(ffi_plan* p, const int32_t* lookup, hipStream_t s, unsigne
     FFI_TRY(plan_fingerprint(p, lookup, s, &fp, &bad));
     if (bad != 0) return FFI_ERR_BAD_LOOKUP;   // also keeps the build kernels' LDS counters in range
     // a rebuild replaces the arrays: whatever still reads the old ones must have drained
-    if (p->perm || p->lab16 || p->idx16) FFI_HIP_TRY(hipDeviceSynchronize());
+    if (p->perm || p->lab16 || p->slot32 || p->idx16) FFI_HIP_TRY(hipDeviceSynchronize());
     free_arrays(p);
     // tiled form: one thread per column (N <= 1024), tiles of at least 62 labels with positions in 16 bits
     // (and 32 rows of out_grad within 32-bit byte offsets, as the kernels' buffer loads need)
