@@ -267,6 +267,16 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
 #pragma unroll
             for (int q = 0; q < kAhead; ++q) {
                 const bool in = i + q < rows;                       // wave-uniform
+#if 1
+                if (WLDS) {
+                    if (!in) break;
+                    float4 xv[8];
+                    const float wv = *(const float __attribute__((address_space(3)))*)(size_t)(wsbase + (e4[q] >> 17) * 4u);
+                    igrad_reads_at((e4[q] & 0x1ff80u) | skewbase, xv);
+                    igrad_fmas(xv, wv, acc);
+                    continue;
+                }
+#endif
                 const unsigned e = in ? e4[q] : e_none;
                 float wv = in ? w4[q] : 0.f;
                 float4 xv[8];

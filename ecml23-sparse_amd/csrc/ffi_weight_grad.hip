@@ -169,19 +169,24 @@ __global__ __launch_bounds__(kResThreads) void wgrad_resident_kernel(const float
 constexpr unsigned kArrIdMask = (1u << kArrIdBits) - 1;
 constexpr int kSlotPitch = kWgChunk + 4;     // floats between the reordering slots of neighbouring threads (16-byte aligned)
 
+template <int NCH>
 __global__ __launch_bounds__(kResThreads) void wgrad_arranged_kernel(const float* __restrict__ xT,
                                                                      const unsigned short* __restrict__ idx16,
                                                                      const float* __restrict__ g,
                                                                      float* __restrict__ gw,
                                                                      float* __restrict__ bias_grad, int B, int N,
-                                                                     int L, int K, int nchunks, int n1, int upb1,
-                                                                     int upb2) {
+                                                                     int L, int K, int nchunks, int n1, int ipb1,
+                                                                     int ipb2) {
     extern __shared__ __align__(16) float xs[];
     const int lane = threadIdx.x & 63;
     const int blk = blockIdx.x;
-    const long long total_units = (long long)L * nchunks;
-    const long long u_begin = blk < n1 ? (long long)blk * upb1 : (long long)n1 * upb1 + (long long)(blk - n1) * upb2;
-    const long long u_end = min(u_begin + (blk < n1 ? upb1 : upb2), total_units);
+    // NCH == 1: an item is a unit (label, chunk) and a thread owns kResUnits of them, of kResUnits labels;
+    // NCH > 1 (= the number of chunks of a label): an item is a label and a thread owns all NCH units of kResUnits / NCH
+    // labels, so that the label's 32 out_grad values of a batch tile are loaded once for all its chunks.
+    constexpr int kItems = kResUnits / NCH;
+    const long long total_items = NCH == 1 ? (long long)L * nchunks : (long long)L;
+    const long long i_begin = blk < n1 ? (long long)blk * ipb1 : (long long)n1 * ipb1 + (long long)(blk - n1) * ipb2;
+    const long long i_end = min(i_begin + (blk < n1 ? ipb1 : ipb2), total_items);
     const int nbt = (B + kTileBatch - 1) / kTileBatch;
 
     float res[kResUnits][kWgChunk];
@@ -189,9 +194,9 @@ __global__ __launch_bounds__(kResThreads) void wgrad_arranged_kernel(const float
     for (int q = 0; q < kResUnits; ++q)
 #pragma unroll
         for (int k = 0; k < kWgChunk; ++k) res[q][k] = 0.f;
-    float gsum[kResUnits];                                 // column sums of out_grad (the bias gradient)
+    float gsum[kItems];                                    // column sums of out_grad (the bias gradient)
 #pragma unroll
-    for (int q = 0; q < kResUnits; ++q) gsum[q] = 0.f;
+    for (int q = 0; q < kItems; ++q) gsum[q] = 0.f;
 
     for (int bt = 0; bt < nbt; ++bt) {
         const int b0 = bt * kTileBatch;
@@ -202,35 +207,39 @@ __global__ __launch_bounds__(kResThreads) void wgrad_arranged_kernel(const float
         unsigned skew = (unsigned)(size_t)(__attribute__((address_space(3))) float*)xs + (unsigned)(lane & 7) * 16u;
         asm volatile("" : "+v"(skew));                     // keep the LDS addresses out of loop-invariant hoisting
 #pragma unroll
-        for (int q = 0; q < kResUnits; ++q) {
-            const long long ubase = u_begin + (long long)q * kResThreads;
-            if (ubase + (long long)(threadIdx.x & ~63u) < u_end) {          // the wavefront has units in this round
-                const long long u = min(ubase + (long long)threadIdx.x, u_end - 1);   // clamped: loads stay in bounds
-                const int j = (int)(u % L);
+        for (int qq = 0; qq < kItems; ++qq) {
+            const long long ibase = i_begin + (long long)qq * kResThreads;
+            if (ibase + (long long)(threadIdx.x & ~63u) < i_end) {          // the wavefront has items in this round
+                const long long it = min(ibase + (long long)threadIdx.x, i_end - 1);   // clamped: loads stay in bounds
+                const int j = NCH == 1 ? (int)(it % L) : (int)it;
                 float gb[32];
                 load_rows32(g, L, b0, B, (unsigned)j, gb);
                 if (bias_grad != nullptr) {
-                    float t = gsum[q];
+                    float t = gsum[qq];
 #pragma unroll
                     for (int b = 0; b < 32; ++b) t += gb[b];
-                    gsum[q] = t;
-                }
-                unsigned idp[kWgChunk / 2];                // two 16-bit entries per register
-                const uint4* erow = reinterpret_cast<const uint4*>(idx16 + (size_t)u * kWgChunk);
-#pragma unroll
-                for (int t = 0; t < kWgChunk / 8; ++t) {
-                    const uint4 v = erow[t];
-                    idp[4 * t] = v.x; idp[4 * t + 1] = v.y; idp[4 * t + 2] = v.z; idp[4 * t + 3] = v.w;
+                    gsum[qq] = t;
                 }
                 xor_permute_groups(gb, lane & 7);          // match the skewed chunk order of the gathers
 #pragma unroll
-                for (int k = 0; k < kWgChunk; ++k) {
-                    const unsigned e = (k & 1) ? (idp[k >> 1] >> 16) : idp[k >> 1];
-                    float4 xv[8];
-                    wgrad_reads(((e & kArrIdMask) << 7) + skew, xv);
-                    __builtin_amdgcn_sched_barrier(0);
-                    res[q][k] = wgrad_dot(xv, gb, res[q][k]);
-                    __builtin_amdgcn_sched_barrier(0);
+                for (int c = 0; c < NCH; ++c) {
+                    const long long u = NCH == 1 ? it : (long long)c * L + it;
+                    unsigned idp[kWgChunk / 2];            // two 16-bit entries per register
+                    const uint4* erow = reinterpret_cast<const uint4*>(idx16 + (size_t)u * kWgChunk);
+#pragma unroll
+                    for (int t = 0; t < kWgChunk / 8; ++t) {
+                        const uint4 v = erow[t];
+                        idp[4 * t] = v.x; idp[4 * t + 1] = v.y; idp[4 * t + 2] = v.z; idp[4 * t + 3] = v.w;
+                    }
+#pragma unroll
+                    for (int k = 0; k < kWgChunk; ++k) {
+                        const unsigned e = (k & 1) ? (idp[k >> 1] >> 16) : idp[k >> 1];
+                        float4 xv[8];
+                        wgrad_reads(((e & kArrIdMask) << 7) + skew, xv);
+                        __builtin_amdgcn_sched_barrier(0);
+                        res[qq * NCH + c][k] = wgrad_dot(xv, gb, res[qq * NCH + c][k]);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
                 }
             }
         }
@@ -241,23 +250,28 @@ __global__ __launch_bounds__(kResThreads) void wgrad_arranged_kernel(const float
     float* slot = xs + (size_t)threadIdx.x * kSlotPitch;
     const bool vec4 = (K % 4 == 0) && (((uintptr_t)gw & 15) == 0);
 #pragma unroll
-    for (int q = 0; q < kResUnits; ++q) {
-        const long long u = u_begin + (long long)q * kResThreads + threadIdx.x;
-        if (u < u_end) {
-            const int c = (int)(u / L), j = (int)(u - (long long)c * L);
-            const int k0 = c * kWgChunk;
-            if (bias_grad != nullptr && c == 0) bias_grad[j] = gsum[q];
-            const unsigned short* erow = idx16 + (size_t)u * kWgChunk;
+    for (int qq = 0; qq < kItems; ++qq) {
+        const long long it = i_begin + (long long)qq * kResThreads + threadIdx.x;
+        if (it < i_end) {
 #pragma unroll
-            for (int i = 0; i < kWgChunk; ++i) slot[erow[i] >> kArrIdBits] = res[q][i];
-            float* grow = gw + (size_t)j * K + k0;
-            if (vec4 && k0 + kWgChunk <= K) {
+            for (int cc = 0; cc < NCH; ++cc) {
+                const int c = NCH == 1 ? (int)(it / L) : cc;
+                const int j = NCH == 1 ? (int)(it - (long long)c * L) : (int)it;
+                const long long u = (long long)c * L + j;
+                const int k0 = c * kWgChunk;
+                if (bias_grad != nullptr && c == 0) bias_grad[j] = gsum[qq];
+                const unsigned short* erow = idx16 + (size_t)u * kWgChunk;
 #pragma unroll
-                for (int t = 0; t < kWgChunk / 4; ++t)
-                    *reinterpret_cast<float4*>(grow + 4 * t) = *reinterpret_cast<const float4*>(slot + 4 * t);
-            } else {
-                for (int k = 0; k < kWgChunk; ++k)
-                    if (k0 + k < K) grow[k] = slot[k];
+                for (int i = 0; i < kWgChunk; ++i) slot[erow[i] >> kArrIdBits] = res[qq * NCH + cc][i];
+                float* grow = gw + (size_t)j * K + k0;
+                if (vec4 && k0 + kWgChunk <= K) {
+#pragma unroll
+                    for (int t = 0; t < kWgChunk / 4; ++t)
+                        *reinterpret_cast<float4*>(grow + 4 * t) = *reinterpret_cast<const float4*>(slot + 4 * t);
+                } else {
+                    for (int k = 0; k < kWgChunk; ++k)
+                        if (k0 + k < K) grow[k] = slot[k];
+                }
             }
         }
     }
@@ -280,27 +294,41 @@ int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float
         // A first round of full workgroups (kResUnits units per thread), one per CU, as long as whole rounds
         // fit; what is left is shared evenly by a second set of workgroups in the same launch.
         const int nchunks = (d.K + kWgChunk - 1) / kWgChunk;
-        const long long units = (long long)d.L * nchunks;
-        const long long cap = (long long)kResUnits * kResThreads;      // units a workgroup can hold
-        const int n1 = (int)(units / (cap * cus)) * cus;
-        const long long rest = units - (long long)n1 * cap;
-        int n2 = 0, upb2 = 0;
-        if (rest > 0) {
-            const long long rounds = (rest + cap * cus - 1) / (cap * cus);
-            n2 = (int)std::min<long long>(rounds * cus, (rest + 63) / 64);
-            upb2 = (int)((rest + n2 - 1) / n2);
-            n2 = (int)((rest + upb2 - 1) / upb2);
-        }
-        const unsigned blocks = (unsigned)(n1 + n2);
-        const int upb = (int)cap;
+        int n1 = 0, n2 = 0, ipb = 0, ipb2 = 0;
+        auto split = [&](long long items, long long cap) {             // cap: items a workgroup can hold
+            n1 = (int)(items / (cap * cus)) * cus;
+            const long long rest = items - (long long)n1 * cap;
+            n2 = 0; ipb2 = 0;
+            if (rest > 0) {
+                const long long rounds = (rest + cap * cus - 1) / (cap * cus);
+                n2 = (int)std::min<long long>(rounds * cus, (rest + 63) / 64);
+                ipb2 = (int)((rest + n2 - 1) / n2);
+                n2 = (int)((rest + ipb2 - 1) / ipb2);
+            }
+            ipb = (int)cap;
+        };
         if (plan != nullptr && plan->idx16 != nullptr) {
             // the unit slots of the final reordering need 144 bytes per thread
             const size_t lds = std::max(tile_lds_bytes(d.N), (size_t)kResThreads * kSlotPitch * sizeof(float));
-            FFI_HIP_TRY(hipFuncSetAttribute((const void*)wgrad_arranged_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-            hipLaunchKernelGGL(wgrad_arranged_kernel, dim3(blocks), dim3(kResThreads), lds, s, xT, plan->idx16, g, gw, bias_grad, d.B, d.N, d.L, d.K, nchunks, n1, upb, upb2);
+            // a label of two or four chunks: all its units in one thread (its out_grad values are loaded once per
+            // batch tile instead of once per chunk); the work is then split by labels, not by units
+#define FFI_LAUNCH_ARRANGED(NCH)                                                                                                       \
+            do {                                                                                                                       \
+                split(NCH == 1 ? (long long)d.L * nchunks : (long long)d.L, (long long)(kResUnits / NCH) * kResThreads);               \
+                FFI_HIP_TRY(hipFuncSetAttribute((const void*)wgrad_arranged_kernel<NCH>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
+                hipLaunchKernelGGL(wgrad_arranged_kernel<NCH>, dim3((unsigned)(n1 + n2)), dim3(kResThreads), lds, s, xT, plan->idx16, g, gw, \
+                                   bias_grad, d.B, d.N, d.L, d.K, nchunks, n1, ipb, ipb2);                                             \
+            } while (0)
+            if (nchunks == 2) FFI_LAUNCH_ARRANGED(2);
+            else if (nchunks == 4) FFI_LAUNCH_ARRANGED(4);
+            else FFI_LAUNCH_ARRANGED(1);
+#undef FFI_LAUNCH_ARRANGED
             FFI_HIP_TRY(hipGetLastError());
             return FFI_OK;
         }
+        split((long long)d.L * nchunks, (long long)kResUnits * kResThreads);
+        const unsigned blocks = (unsigned)(n1 + n2);
+        const int upb = ipb, upb2 = ipb2;
         const size_t lds = tile_lds_bytes(d.N);
         const bool vec4 = (d.K % 4 == 0) && (((uintptr_t)gw | (uintptr_t)idx) % 16 == 0);
         if (vec4) {
