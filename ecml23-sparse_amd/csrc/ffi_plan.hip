@@ -391,21 +391,23 @@ int plan_tile_labels(int N, int K, int L, int batch_hint, bool* weights_in_lds) 
     int TL = std::min((std::min(std::min(kPlanTileLabels, L), threads > 768 ? threads : 2 * threads) + 1) & ~1,
                       (int)((kPadPos - 1) / (unsigned)K) & ~1);
     // Tiles whose weights fit in LDS beside the tile of out_grad: the walking kernel then reads each slot's weight
-    // through pos16, and the weights need not be brought into slot order first (no permutation kernel, no slot-ordered
+    // through the slot's word, and the weights need not be brought into slot order first (no permutation kernel, no slot-ordered
     // copy of the weights in memory).
-    // Measured (gx pass, 0.3-0.67 M labels): 12-30 % faster than permutation + walk with one or two batch tiles at any
-    // width; with three or four batch tiles the tile's weights are staged three or four times per tile and the form
-    // breaks even only where the workgroup has at least 11 wavefronts to hide that (N >= 704: -1 % at batch 128,
-    // N = 768, fan-in 32, and 119 MB less memory; N <= 640: +4...17 %); beyond four batch tiles it loses 12-15 %.
-    // Tiles larger than the workgroup (two labels staged per thread) and weights beyond what a thread carries in
-    // registers (8 x 16 bytes) spill or add a round trip: not taken.
+    // Measured (gx pass, 0.2-0.67 M labels, fan-in 8...128, 64...1024 columns): with up to four batch tiles the form is
+    // never slower than permutation + walk (0...-60 %, most where the fan-in exceeds 32); with eight batch tiles the
+    // tile's weights are staged eight times per tile: -8 % at fan-in 32 and 512 or 768 columns, even at 256 columns,
+    // +9 % at 128 columns, +1 % at fan-in 64; with sixteen +2...4 %.
+    // The tile: as many labels as fit the LDS with their weights, one label per thread to stage; a thread carries
+    // 8 x 16 bytes of the tile's weights in registers across the barrier, what exceeds that is copied behind it.
+    // A slot's position inside the tile's weights has 15 bits (the zero word that padding slots read included).
     bool w_in_lds = false;
     const int nbt_hint = (batch_hint + 31) / 32;
-    const bool wanted = batch_hint > 0 && (nbt_hint <= 2 || (nbt_hint <= 4 && threads >= 704));   // (unknown batch size: the form for large batches)
+    const bool wanted = batch_hint > 0 && (nbt_hint <= 4 || (nbt_hint <= 8 && K <= 32 && threads >= 512));   // (unknown batch size: the form for large batches)
     if (wanted && threads <= 768) {
-        int tw = std::min(TL, threads & ~1);                 // one label per thread to stage
+        int tw = std::min(TL, threads & ~1);
         while (tw >= 64 && tiled_lds_bytes(tw, K, true) > kPlanLdsBudget) tw -= 2;
-        if (tw >= 64 && (long long)tw * K <= (long long)threads * 32 && 2 * tw >= TL) { TL = tw; w_in_lds = true; }
+        while (tw >= 64 && (long long)tw * K >= 32768) tw -= 2;
+        if (tw >= 64) { TL = tw; w_in_lds = true; }
     }
     *weights_in_lds = w_in_lds;
     return TL;
