@@ -61,7 +61,7 @@ def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=50)      # (the GPU clock takes tens of milliseconds of load to settle)
     ap.add_argument("--config", default="c2", help="workload: c1..c4 forward + backward in fp32 (c2 is the headline); "
                                                    "c5 = bf16 forward with top-5 per sample (inference)")
     ap.add_argument("--layout", default="nb", choices=["nb", "bn"],

@@ -600,7 +600,7 @@ size_t ffi_workspace_bytes(int64_t batch, int64_t num_features, int64_t num_unit
             const double mu = (double)TL * (double)K / (double)N;
             const size_t rows = (size_t)(mu + 2.6 * std::sqrt(mu) + 3.0);
             const size_t slots = tiles * slices * rows * 64;
-            total += slots * 2 * 2 + (tiles * slices + 1) * 4 + L * 2;                  // lab16 + pos16, slice_off, rowpos
+            total += slots * 2 * 2 + (tiles * slices + 1) * 4 + L * 2;                  // 4 bytes per slot (lab16 + pos16, or slot32), slice_off, rowpos
             if (tile_path_fits(d.N) && d.N < (1 << kArrIdBits)) total += L * ((K + 31) / 32) * 32 * 2;   // idx16
             if (!w_in_lds) features_slot = std::max(features_slot, slots * 4);         // weights in slot order
             const size_t nbt = (B + 31) / 32;
