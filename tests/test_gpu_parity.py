@@ -147,6 +147,8 @@ PATH_SHAPES = [
     (200, 2000, 600, 33),      # wide, two batch passes
     (7, 64, 70000, 3),         # many tiles of a tiny column set
     (128, 512, 4100, 100),     # four register chunks per label, tail of 4
+    (64, 768, 900, 300),       # a tile's weights far beyond what its threads carry in registers: most are copied behind the barrier
+    (96, 200, 3000, 7),        # weights of a tile not a multiple of 16 bytes: staged word by word
     # forward over batch tiles of 64 (N <= 608 and more than 32 samples):
     (256, 512, 5000, 64),      # whole tiles, vector loads
     (100, 608, 3100, 21),      # the widest input of that path, second tile partly filled, odd fan-in (scalar loads)
