@@ -192,8 +192,6 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
             return (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(lab_rsrc, lane2, (row0 + r) * 128u, 0);
         };
         auto load_w = [&](unsigned r) { return WLDS ? 0.f : buffer_load_f32(wp_rsrc, lane4, (row0 + r) * 256u); };
-        // (WLDS) rows past the end of the slice: the zero row and the zero word behind the tile's weights
-        const unsigned e_none = WLDS ? (tile_w << 17) | ((unsigned)zero_row << 7) : (unsigned)zero_row;
         unsigned e4[kAhead];
         float w4[kAhead];
 #pragma unroll
@@ -262,33 +260,26 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
             // keep these loads here, a whole group of rows ahead of their use (left alone, the
             // scheduler sinks them below the multiply-adds and every group waits a full round trip)
             __builtin_amdgcn_sched_barrier(0);
-            // branch-free: padding slots carry weight 0 and point at an all-zero LDS row, rows past
-            // the end of the slice are redirected there too
+            // Padding slots inside the slice carry weight 0 (or the position of a zero word) and point at an all-zero
+            // LDS row.  The rows past the slice's end: the weights-in-LDS form does not walk them (a wave-uniform branch
+            // per row; against redirecting them to the zero row it saves two selects per row and 2.5 rows per slice,
+            // 5 us of a 0.66-ms step at 670,091 labels); the forms with weights in slot order redirect them, branch-free
+            // (there the branch measured 0.4 % slower at fan-in 64 and 501,070 labels).
 #pragma unroll
             for (int q = 0; q < kAhead; ++q) {
                 const bool in = i + q < rows;                       // wave-uniform
-#if 1
+                float4 xv[8];
                 if (WLDS) {
                     if (!in) break;
-                    float4 xv[8];
+                    // (the tile starts at LDS address 0 -- the kernel has no other LDS -- so the row's byte offset and the
+                    // lane's skew, which share no bit, combine with an OR: one instruction with the mask)
                     const float wv = *(const float __attribute__((address_space(3)))*)(size_t)(wsbase + (e4[q] >> 17) * 4u);
                     igrad_reads_at((e4[q] & 0x1ff80u) | skewbase, xv);
                     igrad_fmas(xv, wv, acc);
-                    continue;
-                }
-#endif
-                const unsigned e = in ? e4[q] : e_none;
-                float wv = in ? w4[q] : 0.f;
-                float4 xv[8];
-                if (WLDS) {
-                    // (the tile starts at LDS address 0 -- the kernel has no other LDS -- so the row's byte offset and the
-                    // lane's skew, which share no bit, combine with an OR: one instruction with the mask)
-                    wv = *(const float __attribute__((address_space(3)))*)(size_t)(wsbase + (e >> 17) * 4u);
-                    igrad_reads_at((e & 0x1ff80u) | skewbase, xv);
                 } else {
-                    igrad_reads(e, skewbase, xv);
+                    igrad_reads(in ? e4[q] : (unsigned)zero_row, skewbase, xv);
+                    igrad_fmas(xv, in ? w4[q] : 0.f, acc);
                 }
-                igrad_fmas(xv, wv, acc);
             }
 #pragma unroll
             for (int q = 0; q < kAhead; ++q) { e4[q] = en[q]; w4[q] = wn[q]; }
