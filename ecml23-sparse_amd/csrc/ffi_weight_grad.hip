@@ -169,7 +169,7 @@ __global__ __launch_bounds__(kResThreads) void wgrad_resident_kernel(const float
 constexpr unsigned kArrIdMask = (1u << kArrIdBits) - 1;
 constexpr int kSlotPitch = kWgChunk + 4;     // floats between the reordering slots of neighbouring threads (16-byte aligned)
 
-template <int NCH>
+template <int NCH, int UNITS>
 __global__ __launch_bounds__(kResThreads) void wgrad_arranged_kernel(const float* __restrict__ xT,
                                                                      const unsigned short* __restrict__ idx16,
                                                                      const float* __restrict__ g,
@@ -180,18 +180,20 @@ __global__ __launch_bounds__(kResThreads) void wgrad_arranged_kernel(const float
     extern __shared__ __align__(16) float xs[];
     const int lane = threadIdx.x & 63;
     const int blk = blockIdx.x;
-    // NCH == 1: an item is a unit (label, chunk) and a thread owns kResUnits of them, of kResUnits labels;
-    // NCH > 1 (= the number of chunks of a label): an item is a label and a thread owns all NCH units of kResUnits / NCH
+    // UNITS: units a thread owns.
+    // NCH == 1: an item is a unit (label, chunk) and a thread owns UNITS of them, of UNITS labels;
+    // NCH > 1 (= the number of chunks of a label): an item is a label and a thread owns all NCH units of UNITS / NCH
     // labels, so that the label's 32 out_grad values of a batch tile are loaded once for all its chunks.
-    constexpr int kItems = kResUnits / NCH;
+    static_assert(UNITS % NCH == 0 && UNITS <= kResUnits, "whole labels per thread");
+    constexpr int kItems = UNITS / NCH;
     const long long total_items = NCH == 1 ? (long long)L * nchunks : (long long)L;
     const long long i_begin = blk < n1 ? (long long)blk * ipb1 : (long long)n1 * ipb1 + (long long)(blk - n1) * ipb2;
     const long long i_end = min(i_begin + (blk < n1 ? ipb1 : ipb2), total_items);
     const int nbt = (B + kTileBatch - 1) / kTileBatch;
 
-    float res[kResUnits][kWgChunk];
+    float res[UNITS][kWgChunk];
 #pragma unroll
-    for (int q = 0; q < kResUnits; ++q)
+    for (int q = 0; q < UNITS; ++q)
 #pragma unroll
         for (int k = 0; k < kWgChunk; ++k) res[q][k] = 0.f;
     float gsum[kItems];                                    // column sums of out_grad (the bias gradient)
@@ -279,6 +281,32 @@ __global__ __launch_bounds__(kResThreads) void wgrad_arranged_kernel(const float
 
 }  // namespace
 
+// Four units per thread or three?  A CU works through its share of the units in workgroups, one at a time (the tile of x
+// fills the LDS), each of which stages x once per batch tile and then runs one round per unit of its threads; the last
+// workgroup's last round may be partly filled.  Whether 3 x 512 or 4 x 512 units per workgroup leaves the cheaper
+// remainder depends on the unit count.  The model is in units of a full four-unit round, from timings at 768 columns,
+// batch 128 (524,288 / 393,216 / 131,072 / 145,803 labels, fan-in 32): staging 0.36 (scaled with the column count), a
+// round of the three-unit kernel 0.93 (it needs 227 registers instead of 256), a partly filled round 0.33 + 0.084 per
+// wavefront.  Three units are taken when the model sees more than 5 % in them (measured then: -2.5 % at 670,091 labels, -5.5 % at 393,216
+// labels and 512 columns; where it sees 3-5 %, measurements at other widths went both ways).
+bool three_units_cheaper(long long units, int N, int cus) {
+    const double stage = 0.36 * (double)N / 768.0;
+    auto cost = [&](int u, double round) {
+        const long long cap = (long long)u * kResThreads;
+        const long long full = units / (cap * cus);                       // whole workgroups per CU
+        const long long rest = units - full * cap * cus;
+        double c = (double)full * (stage + u * round);
+        if (rest > 0) {
+            const long long wgs = std::min<long long>(cus, (rest + 63) / 64);
+            const long long per = (rest + wgs - 1) / wgs;                  // units of a workgroup of the second set
+            const long long part = per % kResThreads;
+            c += stage + (double)(per / kResThreads) * round + (part ? 0.33 + 0.084 * (double)((part + 63) / 64) : 0.0);
+        }
+        return c;
+    };
+    return cost(3, 0.93) < 0.95 * cost(4, 1.0);
+}
+
 int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float* gw, float* bias_grad, const Dims& d,
                        hipStream_t s, const ffi_plan* plan) {
     // (32 rows of out_grad must be reachable through 32-bit byte offsets)
@@ -312,16 +340,17 @@ int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float
             const size_t lds = std::max(tile_lds_bytes(d.N), (size_t)kResThreads * kSlotPitch * sizeof(float));
             // a label of two or four chunks: all its units in one thread (its out_grad values are loaded once per
             // batch tile instead of once per chunk); the work is then split by labels, not by units
-#define FFI_LAUNCH_ARRANGED(NCH)                                                                                                       \
+#define FFI_LAUNCH_ARRANGED(NCH, UNITS)                                                                                                \
             do {                                                                                                                       \
-                split(NCH == 1 ? (long long)d.L * nchunks : (long long)d.L, (long long)(kResUnits / NCH) * kResThreads);               \
-                FFI_HIP_TRY(hipFuncSetAttribute((const void*)wgrad_arranged_kernel<NCH>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
-                hipLaunchKernelGGL(wgrad_arranged_kernel<NCH>, dim3((unsigned)(n1 + n2)), dim3(kResThreads), lds, s, xT, plan->idx16, g, gw, \
+                split(NCH == 1 ? (long long)d.L * nchunks : (long long)d.L, (long long)(UNITS / NCH) * kResThreads);                   \
+                FFI_HIP_TRY(hipFuncSetAttribute((const void*)wgrad_arranged_kernel<NCH, UNITS>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
+                hipLaunchKernelGGL((wgrad_arranged_kernel<NCH, UNITS>), dim3((unsigned)(n1 + n2)), dim3(kResThreads), lds, s, xT, plan->idx16, g, gw, \
                                    bias_grad, d.B, d.N, d.L, d.K, nchunks, n1, ipb, ipb2);                                             \
             } while (0)
-            if (nchunks == 2) FFI_LAUNCH_ARRANGED(2);
-            else if (nchunks == 4) FFI_LAUNCH_ARRANGED(4);
-            else FFI_LAUNCH_ARRANGED(1);
+            if (nchunks == 2) FFI_LAUNCH_ARRANGED(2, 4);
+            else if (nchunks == 4) FFI_LAUNCH_ARRANGED(4, 4);
+            else if (three_units_cheaper((long long)d.L * nchunks, d.N, cus)) FFI_LAUNCH_ARRANGED(1, 3);
+            else FFI_LAUNCH_ARRANGED(1, 4);
 #undef FFI_LAUNCH_ARRANGED
             FFI_HIP_TRY(hipGetLastError());
             return FFI_OK;

@@ -175,7 +175,8 @@ def test_code_paths(ffi, shape, transposed):
 @pytest.mark.parametrize("shape", [(300, 700, 5000, 32), (33, 96, 9, 5), (128, 512, 4100, 100), (40, 1216, 2500, 36), (64, 1100, 3000, 12),
                                    (48, 1300, 2000, 20),
                                    (96, 512, 20000, 64),     # two chunks per label, both held by one thread
-                                   (64, 300, 2600, 128)])     # four chunks per label
+                                   (64, 300, 2600, 128),      # four chunks per label
+                                   (32, 64, 360000, 32)])     # enough units per CU for the kernel that holds three units per thread
 def test_planned_weight_grad_code_paths(ffi, shape):
     B, N, L, K = shape
     x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=B + K)
