@@ -325,7 +325,8 @@ int launch_tiled(const ffi_plan* p, const float* w, const float* g, float* gx, i
                  const unsigned long long* verdict) {
     const int nbt = (B + kTileBatch - 1) / kTileBatch;
     const int cus = device_cu_count();
-    int streams = std::max(1, std::min(p->tiles, cus / std::max(1, nbt)));
+    const int per_cu = tiled_workgroups_per_cu(p->threads, p->tile_labels, p->K, p->w_in_lds);
+    int streams = std::max(1, std::min(p->tiles, per_cu * cus / std::max(1, nbt)));
     const int tps = (p->tiles + streams - 1) / streams;
     streams = (p->tiles + tps - 1) / tps;
     const int bpad = nbt * kTileBatch;
@@ -358,6 +359,8 @@ int launch_tiled(const ffi_plan* p, const float* w, const float* g, float* gx, i
         // (plans take that form only with workgroups of at most 768 threads that stage one label each)
         if (p->threads > 768 || p->tile_labels > p->threads) return FFI_ERR_BAD_ARGUMENT;
         FFI_LAUNCH_TILE(768, 1, true);
+    } else if (per_cu > 1) {
+        FFI_LAUNCH_TILE(1024, 1, false);                 // (the instantiation of at most 128 registers)
     } else if (p->threads <= 768) {
         if (p->tile_labels <= p->threads) FFI_LAUNCH_TILE(768, 1, false); else FFI_LAUNCH_TILE(768, 2, false);
     } else {

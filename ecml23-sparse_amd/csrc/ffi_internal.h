@@ -254,6 +254,20 @@ inline int tiled_rows_per_half(int tile_labels) { return tile_labels / 2 + (tile
 inline size_t tiled_lds_bytes(int tile_labels, int K, bool with_weights) {
     return (size_t)(2 * tiled_rows_per_half(tile_labels) + 2) * 128 + (with_weights ? ((size_t)tile_labels * K + 4) * 4 : 0);
 }
+// Workgroups of the walking kernel that one CU holds at a time.  The forms whose weights are in slot order have an
+// instantiation of at most 128 registers per thread, so a CU takes as many of its workgroups as fit its 16 wavefronts
+// of that size and its 160 KB of LDS; plans size their tiles for that (one label per thread for workgroups of at most
+// 512 threads: two workgroups of 512, four of 256, ...).  Measured at eight batch tiles against one workgroup of
+// two-label-per-thread tiles: input gradient -9 % at 512 columns / fan-in 64 / 501,070 labels, -22 % at 256 columns,
+// -13 % at 384 columns / fan-in 48, -5 % at 512 columns and sixteen batch tiles.
+inline int tiled_workgroups_per_cu(int threads, int tile_labels, int K, bool with_weights) {
+    if (with_weights || threads > 512 || tile_labels > threads) return 1;
+    const size_t lds = tiled_lds_bytes(tile_labels, K, false);
+    const int by_lds = (int)((size_t)160 * 1024 / (lds > 0 ? lds : 1));
+    const int by_waves = 1024 / (threads > 0 ? threads : 1);
+    const int n = by_lds < by_waves ? by_lds : by_waves;
+    return n < 1 ? 1 : n;
+}
 constexpr int kArrIdBits = 11;            // column-id field of an arranged entry (narrow inputs: ids < 1216)
 int plan_build(ffi_plan* p, const int32_t* lookup, hipStream_t s);
 int plan_tile_labels(int N, int K, int L, int batch_hint, bool* weights_in_lds);

@@ -436,6 +436,9 @@ int plan_tile_labels(int N, int K, int L, int batch_hint, bool* weights_in_lds) 
         while (tw >= 64 && (long long)tw * K >= 32768) tw -= 2;
         if (tw >= 64) { TL = tw; w_in_lds = true; }
     }
+    // the forms with weights in slot order, workgroups of at most 512 threads: one label per thread, so that two or more
+    // workgroups share a CU (see tiled_workgroups_per_cu)
+    if (!w_in_lds && threads <= 512) TL = std::min(TL, std::max(2, threads & ~1));
     *weights_in_lds = w_in_lds;
     return TL;
 }
