@@ -325,7 +325,7 @@ int launch_tiled(const ffi_plan* p, const float* w, const float* g, float* gx, i
                  const unsigned long long* verdict) {
     const int nbt = (B + kTileBatch - 1) / kTileBatch;
     const int cus = device_cu_count();
-    const int per_cu = tiled_workgroups_per_cu(p->threads, p->tile_labels, p->K, p->w_in_lds);
+    const int per_cu = tiled_workgroups_per_cu(p->threads, p->tile_labels, p->K, p->w_in_lds, nbt);
     int streams = std::max(1, std::min(p->tiles, per_cu * cus / std::max(1, nbt)));
     const int tps = (p->tiles + streams - 1) / streams;
     streams = (p->tiles + tps - 1) / tps;

@@ -254,17 +254,22 @@ inline int tiled_rows_per_half(int tile_labels) { return tile_labels / 2 + (tile
 inline size_t tiled_lds_bytes(int tile_labels, int K, bool with_weights) {
     return (size_t)(2 * tiled_rows_per_half(tile_labels) + 2) * 128 + (with_weights ? ((size_t)tile_labels * K + 4) * 4 : 0);
 }
-// Workgroups of the walking kernel that one CU holds at a time.  The forms whose weights are in slot order have an
-// instantiation of at most 128 registers per thread, so a CU takes as many of its workgroups as fit its 16 wavefronts
-// of that size and its 160 KB of LDS; plans size their tiles for that (one label per thread for workgroups of at most
-// 512 threads: two workgroups of 512, four of 256, ...).  Measured at eight batch tiles against one workgroup of
-// two-label-per-thread tiles: input gradient -9 % at 512 columns / fan-in 64 / 501,070 labels, -22 % at 256 columns,
-// -13 % at 384 columns / fan-in 48, -5 % at 512 columns and sixteen batch tiles.
-inline int tiled_workgroups_per_cu(int threads, int tile_labels, int K, bool with_weights) {
-    if (with_weights || threads > 512 || tile_labels > threads) return 1;
-    const size_t lds = tiled_lds_bytes(tile_labels, K, false);
+// Workgroups of the walking kernel that one CU holds at a time: as many as fit its LDS and its wavefront slots at the
+// kernel's register count (16 wavefronts per CU for the instantiation of at most 128 registers that the forms with
+// weights in slot order have, 12 for the weights-in-LDS instantiation).  Plans size their tiles for that: one label per
+// thread for workgroups of at most 512 threads (slot-ordered weights: two workgroups of 512, four of 256, ...), and for
+// weights-in-LDS plans of at most 256 threads a share of the LDS (three workgroups of 256, six of 128).
+// Measured, input gradient at 300,000-501,070 labels against one workgroup per CU: slot-ordered weights at eight batch
+// tiles -9 % at 512 columns / fan-in 64, -22 % at 256 columns, -51 % at 128, -74 % at 64; weights in LDS with two to
+// four batch tiles -28 % at 256 columns, -40...-60 % at 64-128 columns, but +16 % with two workgroups of 384 threads
+// (half-size tiles pad more than the sharing gains) and 0...+30 % with a single batch tile (nothing to overlap): those
+// two cases keep one workgroup per CU.
+inline int tiled_workgroups_per_cu(int threads, int tile_labels, int K, bool with_weights, int batch_tiles) {
+    if (threads > 512 || tile_labels > threads) return 1;
+    if (with_weights && (threads > 256 || batch_tiles < 2)) return 1;
+    const size_t lds = tiled_lds_bytes(tile_labels, K, with_weights);
     const int by_lds = (int)((size_t)160 * 1024 / (lds > 0 ? lds : 1));
-    const int by_waves = 1024 / (threads > 0 ? threads : 1);
+    const int by_waves = (with_weights ? 768 : 1024) / (threads > 0 ? threads : 1);
     const int n = by_lds < by_waves ? by_lds : by_waves;
     return n < 1 ? 1 : n;
 }

@@ -420,19 +420,25 @@ int plan_tile_labels(int N, int K, int L, int batch_hint, bool* weights_in_lds) 
     // Tiles whose weights fit in LDS beside the tile of out_grad: the walking kernel then reads each slot's weight
     // through the slot's word, and the weights need not be brought into slot order first (no permutation kernel, no slot-ordered
     // copy of the weights in memory).
-    // Measured (gx pass, 0.2-0.67 M labels, fan-in 8...128, 64...1024 columns): with up to four batch tiles the form is
-    // never slower than permutation + walk (0...-60 %, most where the fan-in exceeds 32); with eight batch tiles the
-    // tile's weights are staged eight times per tile: -8 % at fan-in 32 and 512 or 768 columns, even at 256 columns,
-    // +9 % at 128 columns, +1 % at fan-in 64; with sixteen +2...4 %.
+    // Measured (gx pass, 0.2-0.67 M labels, fan-in 8...128, 64...1024 columns), against permutation + walk with the
+    // tiles and workgroups per CU that suit each form (tiled_workgroups_per_cu): with up to four batch tiles the form is
+    // 5-60 % faster (most where the fan-in exceeds 32 or the layer has at most 256 columns); with five to eight batch
+    // tiles the tile's weights are staged that many times per tile: at fan-in 32 and below still -5...-30 % with at
+    // most 256 columns (several workgroups per CU overlap the staging) and -1...-8 % with 512 or 768, but +1 % at fan-in
+    // 64 / 512 columns against the two-workgroup slot-ordered form, which also wins at 320-448 columns; with sixteen
+    // batch tiles -7...+4 %: not taken.
     // The tile: as many labels as fit the LDS with their weights, one label per thread to stage; a thread carries
     // 8 x 16 bytes of the tile's weights in registers across the barrier, what exceeds that is copied behind it.
     // A slot's position inside the tile's weights has 15 bits (the zero word that padding slots read included).
     bool w_in_lds = false;
     const int nbt_hint = (batch_hint + 31) / 32;
-    const bool wanted = batch_hint > 0 && (nbt_hint <= 4 || (nbt_hint <= 8 && K <= 32 && threads >= 512));   // (unknown batch size: the form for large batches)
+    const bool wanted = batch_hint > 0 &&
+                        (nbt_hint <= 4 || (nbt_hint <= 8 && K <= 32 && (threads >= 512 || threads <= 256)));   // (unknown batch size: the form for large batches)
     if (wanted && threads <= 768) {
         int tw = std::min(TL, threads & ~1);
-        while (tw >= 64 && tiled_lds_bytes(tw, K, true) > kPlanLdsBudget) tw -= 2;
+        // (workgroups of at most 256 threads share a CU when there are batch tiles to overlap: tiled_workgroups_per_cu)
+        const size_t budget = (threads <= 256 && nbt_hint >= 2) ? kPlanLdsBudget / (size_t)(768 / threads) : kPlanLdsBudget;
+        while (tw >= 64 && tiled_lds_bytes(tw, K, true) > budget) tw -= 2;
         while (tw >= 64 && (long long)tw * K >= 32768) tw -= 2;
         if (tw >= 64) { TL = tw; w_in_lds = true; }
     }
