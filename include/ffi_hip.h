@@ -123,9 +123,9 @@ int ffi_input_grad_f32(const int32_t* lookup, const float* weights, const float*
  * reference, whose input gradient scatters with atomicAdd (backward.cu.h:119,139,161,182).
  * ffi_plan_create synchronises `stream` once.  A plan is tied to the device it was made on.
  * `batch_hint` is the batch size the plan will mostly be used with (0 = unknown).  It steers the plan's layout only:
- * for batches of at most 128 (at most 256 with fan_in <= 32 and 448 < num_features <= 768) and num_features <= 768
- * the plan uses smaller label tiles whose weights the input-gradient kernel keeps on chip, which needs no
- * slot-ordered copy of the weights per call;
+ * for batches of at most 128 (at most 256 with fan_in <= 32 and num_features <= 256 or 448 < num_features <= 768)
+ * and num_features <= 768 the plan uses smaller label tiles whose weights the input-gradient kernel keeps on chip,
+ * which needs no slot-ordered copy of the weights per call;
  * any batch size may be used with any plan, a mismatch costs time (up to 30 %), not correctness.  The plans the stateless
  * entry points cache take the batch size of the call that builds them.
  */
