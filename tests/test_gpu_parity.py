@@ -149,6 +149,11 @@ PATH_SHAPES = [
     (128, 512, 4100, 100),     # four register chunks per label, tail of 4
     (64, 768, 900, 300),       # a tile's weights far beyond what its threads carry in registers: most are copied behind the barrier
     (96, 200, 3000, 7),        # weights of a tile not a multiple of 16 bytes: staged word by word
+    # several workgroups of the input-gradient kernel per CU (narrow layers):
+    (300, 200, 9000, 16),      # ten batch tiles, weights in slot order: four workgroups of 256 threads
+    (96, 128, 12000, 16),      # three batch tiles, weights in LDS: six workgroups of 128 threads, a share of the LDS each
+    (160, 256, 9000, 32),      # five batch tiles, weights in LDS: three workgroups of 256 threads
+    (288, 64, 20000, 8),       # nine batch tiles, weights in slot order: sixteen workgroups of 64 threads
     # forward over batch tiles of 64 (N <= 608 and more than 32 samples):
     (256, 512, 5000, 64),      # whole tiles, vector loads
     (100, 608, 3100, 21),      # the widest input of that path, second tile partly filled, odd fan-in (scalar loads)
