@@ -605,7 +605,9 @@ size_t ffi_workspace_bytes(int64_t batch, int64_t num_features, int64_t num_unit
             if (!w_in_lds) features_slot = std::max(features_slot, slots * 4);         // weights in slot order
             const size_t nbt = (B + 31) / 32;
             const size_t per_cu = (size_t)tiled_workgroups_per_cu((int)threads, (int)TL, d.K, w_in_lds, (int)((B + 31) / 32));
-            const size_t streams = std::max<size_t>(1, std::min<size_t>(tiles, per_cu * (size_t)device_cu_count() / std::max<size_t>(1, nbt)));
+            size_t streams = std::max<size_t>(1, std::min<size_t>(tiles, per_cu * (size_t)device_cu_count() / std::max<size_t>(1, nbt)));
+            const size_t tiles_per_stream = (tiles + streams - 1) / streams;            // (as the launcher evens them out)
+            streams = (tiles + tiles_per_stream - 1) / tiles_per_stream;
             partial_slot = streams * threads * nbt * 32 * 4;
         } else {
             const size_t nblocks = (L + 65535) / 65536;
