@@ -215,9 +215,10 @@ struct ffi_plan {
     unsigned* slot32 = nullptr;          // plans with w_in_lds, instead of lab16 and pos16: [total_rows*64] (position << 17) | (LDS row << 7)
     unsigned short* pos16 = nullptr;     // [total_rows*64] position (inside the tile's rows of lookup) of each slot;
                                          // kPadPos in padding slots
-    // arranged copy of the column ids for the weight gradient (narrow inputs only, else null):
-    // [chunks of 32 connections][L][32] entries of (connection inside the chunk << 11) | column id, each
-    // label's connections reordered so that even and odd columns alternate (see ffi_plan.hip)
+    // arranged copy of the column ids for the weight gradient (narrow inputs only, else null): per unit u = chunk * L +
+    // label (a chunk = 32 connections) 32 entries of (connection inside the chunk << 11) | column id, each label's
+    // connections reordered so that even and odd columns alternate (see ffi_plan.hip); stored in blocks of 64 units,
+    // quarter by quarter (ffi::arranged_quarter_offset), so that the 64 lanes of a wavefront load 1 KB in one piece
     unsigned short* idx16 = nullptr;
     // blocked global form
     int block_labels = 0;     // labels per block (bounds the part of out_grad that is live at a time)
@@ -274,6 +275,12 @@ inline int tiled_workgroups_per_cu(int threads, int tile_labels, int K, bool wit
     return n < 1 ? 1 : n;
 }
 constexpr int kArrIdBits = 11;            // column-id field of an arranged entry (narrow inputs: ids < 1216)
+// 16-bit word at which quarter t (entries 8 t ... 8 t + 7) of unit u starts in ffi_plan::idx16: units in blocks of 64, a
+// block = [quarter][unit][8 entries]
+__host__ __device__ inline size_t arranged_quarter_offset(long long u, int t) {
+    return ((size_t)(u >> 6) * 4 + (size_t)t) * 512 + (size_t)(u & 63) * 8;
+}
+inline size_t arranged_words(long long units) { return (size_t)((units + 63) / 64) * 64 * 32; }
 int plan_build(ffi_plan* p, const int32_t* lookup, hipStream_t s);
 int plan_tile_labels(int N, int K, int L, int batch_hint, bool* weights_in_lds);
 int launch_arrange_in_place(int32_t* lookup, float* const* arrays, int n_arrays, int L, int K, hipStream_t s);

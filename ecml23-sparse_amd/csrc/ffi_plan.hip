@@ -573,7 +573,8 @@ int build_global(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
 // the others as odd, even, odd, ..., the two lanes always read opposite halves (as far as a label's
 // even and odd columns pair up; what is left over comes last).  One thread per (label, chunk of 32
 // connections); entry i of a unit = (connection inside the chunk << 11) | column id; units are
-// stored chunk-major ([chunk][label][32]) so that consecutive lanes work on consecutive labels.
+// numbered chunk-major (u = chunk * L + label) so that consecutive lanes work on consecutive labels, and stored in
+// blocks of 64 (arranged_quarter_offset).
 __global__ __launch_bounds__(kBlock) void arrange_units_kernel(const int32_t* __restrict__ idx, int L, int K, int nchunks,
                                                                 unsigned short* __restrict__ out) {
     const long long u = (long long)blockIdx.x * kBlock + threadIdx.x;
@@ -585,17 +586,17 @@ __global__ __launch_bounds__(kBlock) void arrange_units_kernel(const int32_t* __
     unsigned nfirst = 0;
     for (int k = 0; k < kn; ++k) nfirst += (((unsigned)row[k] & 1u) == role) ? 1u : 0u;
     const unsigned m = min(nfirst, (unsigned)kn - nfirst);
-    unsigned short* dst = out + (size_t)u * 32;
+    auto dst = [&](unsigned pos) -> unsigned short& { return out[arranged_quarter_offset(u, (int)(pos >> 3)) + (pos & 7u)]; };
     unsigned tf = 0, ts = 0;
     for (int k = 0; k < kn; ++k) {
         const unsigned id = (unsigned)row[k];
         const bool first = (id & 1u) == role;
         const unsigned t = first ? tf++ : ts++;
         const unsigned pos = t < m ? 2u * t + (first ? 0u : 1u) : 2u * m + (t - m);
-        dst[pos] = (unsigned short)(((unsigned)k << kArrIdBits) | id);
+        dst(pos) = (unsigned short)(((unsigned)k << kArrIdBits) | id);
     }
     // a chunk the fan-in does not fill: the rest points at connection 31, which such a chunk never stores
-    for (int k = kn; k < 32; ++k) dst[k] = (unsigned short)(31u << kArrIdBits);
+    for (int k = kn; k < 32; ++k) dst((unsigned)k) = (unsigned short)(31u << kArrIdBits);
 }
 
 // The same reordering applied in place to the lookup matrix itself and to up to four float
@@ -648,11 +649,11 @@ namespace {
 int build_arranged(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     const int nchunks = (p->K + 31) / 32;
     const long long units = (long long)p->L * nchunks;
-    if (!dev_alloc(&p->idx16, (size_t)units * 32)) return FFI_ERR_OUT_OF_MEMORY;
+    if (!dev_alloc(&p->idx16, arranged_words(units))) return FFI_ERR_OUT_OF_MEMORY;
     hipLaunchKernelGGL(arrange_units_kernel, dim3((unsigned)((units + kBlock - 1) / kBlock)), dim3(kBlock), 0, s, lookup,
                        p->L, p->K, nchunks, p->idx16);
     FFI_HIP_TRY(hipGetLastError());
-    p->bytes += (size_t)units * 32 * sizeof(unsigned short);
+    p->bytes += arranged_words(units) * sizeof(unsigned short);
     return FFI_OK;
 }
 

@@ -5,6 +5,8 @@
 #include "ffi_lds_tile.h"
 
 #include <algorithm>
+#include <type_traits>
+#include <utility>
 
 namespace ffi {
 namespace {
@@ -167,6 +169,7 @@ __global__ __launch_bounds__(kResThreads) void wgrad_resident_kernel(const float
 // slot before they are stored.
 // ------------------------------------------------------------------------------------------------
 constexpr unsigned kArrIdMask = (1u << kArrIdBits) - 1;
+constexpr size_t kLdsPerWorkgroup = 160 * 1024;   // gfx950: all of a CU's LDS can go to one workgroup
 constexpr int kSlotPitch = kWgChunk + 4;     // floats between the reordering slots of neighbouring threads (16-byte aligned)
 
 template <int NCH, int UNITS>
@@ -227,10 +230,9 @@ __global__ __launch_bounds__(kResThreads) void wgrad_arranged_kernel(const float
                 for (int c = 0; c < NCH; ++c) {
                     const long long u = NCH == 1 ? it : (long long)c * L + it;
                     unsigned idp[kWgChunk / 2];            // two 16-bit entries per register
-                    const uint4* erow = reinterpret_cast<const uint4*>(idx16 + (size_t)u * kWgChunk);
 #pragma unroll
                     for (int t = 0; t < kWgChunk / 8; ++t) {
-                        const uint4 v = erow[t];
+                        const uint4 v = *reinterpret_cast<const uint4*>(idx16 + arranged_quarter_offset(u, t));
                         idp[4 * t] = v.x; idp[4 * t + 1] = v.y; idp[4 * t + 2] = v.z; idp[4 * t + 3] = v.w;
                     }
 #pragma unroll
@@ -262,9 +264,9 @@ __global__ __launch_bounds__(kResThreads) void wgrad_arranged_kernel(const float
                 const long long u = (long long)c * L + j;
                 const int k0 = c * kWgChunk;
                 if (bias_grad != nullptr && c == 0) bias_grad[j] = gsum[qq];
-                const unsigned short* erow = idx16 + (size_t)u * kWgChunk;
 #pragma unroll
-                for (int i = 0; i < kWgChunk; ++i) slot[erow[i] >> kArrIdBits] = res[qq * NCH + cc][i];
+                for (int i = 0; i < kWgChunk; ++i)
+                    slot[idx16[arranged_quarter_offset(u, i >> 3) + (i & 7)] >> kArrIdBits] = res[qq * NCH + cc][i];
                 float* grow = gw + (size_t)j * K + k0;
                 if (vec4 && k0 + kWgChunk <= K) {
 #pragma unroll
@@ -273,6 +275,284 @@ __global__ __launch_bounds__(kResThreads) void wgrad_arranged_kernel(const float
                 } else {
                     for (int k = 0; k < kWgChunk; ++k)
                         if (k0 + k < K) grow[k] = slot[k];
+                }
+            }
+        }
+    }
+}
+
+
+// ------------------------------------------------------------------------------------------------
+// The arranged kernel with its memory traffic taken off the wavefronts' critical path.  Every wavefront owns a
+// [32 batch rows][64 labels] slice of LDS behind the tile of x; the out_grad values of its NEXT step (an item in a
+// batch tile) are fetched straight into that slice by LDS-direct buffer loads (no registers, no wait), issued one
+// by one between the connections of the current step's walk once the current values have been read out of the
+// slice, and the arranged ids of the next chunk travel in a second set of 16 registers.  A step therefore starts
+// with everything it needs already on the chip: with two wavefronts per SIMD nothing else hides the stream from
+// HBM (per-wavefront phase stamps of the arranged kernel at 670,091 labels x 768 columns x batch 128, fan-in 32:
+// of a workgroup's 110 us, 68 are walks, 12 the wait for out_grad, 15 the epilogue, 14 staging and barriers).
+// The slice is read in the lane's skewed chunk order, which also replaces the 96 conditional moves that used to
+// permute the values in registers; x is staged by LDS-direct 16-byte loads; at the end every wavefront puts its
+// sums back in connection order through its own slice (no workgroup barrier) and stores whole rows.
+// LDS: N * 128 bytes of x + 8 slices of 8 KB: fits for N <= 768.
+// ------------------------------------------------------------------------------------------------
+typedef __attribute__((address_space(3))) float* lds_f32_ptr;
+constexpr int kSliceFloats = kTileBatch * 64;               // one wavefront's slice of out_grad
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant expression
+template <class F, int... Is>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) { (f(std::integral_constant<int, Is>{}), ...); }
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) { static_for_impl(f, std::make_integer_sequence<int, N>{}); }
+
+// LDS-direct buffer loads put lane i's value at M0 + immediate + i * size, and an M0 that changes between two of them
+// costs about 30 ns (measured: 32 loads with one M0 each 0.53 us, with an M0 per 16 of them 0.22 us).  So the
+// destination's offset inside a 4-KB window goes into the instruction's immediate -- which the hardware also adds to
+// the memory address, hence it is taken back out of the scalar offset.
+template <int SIZE, int LDS_BYTES>
+__device__ __forceinline__ void load_to_lds(const buffer_rsrc& r, lds_f32_ptr window, unsigned lane_off, unsigned wave_off) {
+    static_assert(LDS_BYTES >= 0 && LDS_BYTES < 4096, "immediate offset field");
+    static_assert(SIZE == 4 || SIZE == 16, "bytes per lane");
+    if constexpr (SIZE == 4) __builtin_amdgcn_raw_ptr_buffer_load_lds(r, window, 4, lane_off, wave_off - (unsigned)LDS_BYTES, LDS_BYTES, 0);
+    else __builtin_amdgcn_raw_ptr_buffer_load_lds(r, window, 16, lane_off, wave_off - (unsigned)LDS_BYTES, LDS_BYTES, 0);
+}
+
+// xs[r][0..32) = src[r * ld + c0 ...] for r < rows by LDS-direct 16-byte loads: one instruction fills eight rows.
+// Needs ld % 4 == 0, c0 + 32 <= ld, rows % 8 == 0, src 16-byte aligned, rows * ld * 4 < 2^32.  The caller waits
+// (vmcnt) and synchronises.
+template <int THREADS>
+__device__ __forceinline__ void stage_rows32_direct(float* xs, const float* __restrict__ src, int rows, int ld, int c0, int wave,
+                                                    int lane) {
+    const buffer_rsrc r = make_rsrc(src, (size_t)rows * (size_t)ld * sizeof(float));
+    const unsigned lane_off = (unsigned)(lane >> 3) * (unsigned)ld * 4u + (unsigned)(lane & 7) * 16u;
+    const unsigned step = 8u * (unsigned)ld * 4u;          // eight rows further in memory: 1 KB further in LDS
+    const int ninstr = rows / 8;
+    for (int i0 = wave * 4; i0 < ninstr; i0 += (THREADS / 64) * 4) {
+        const lds_f32_ptr window = (lds_f32_ptr)xs + (size_t)i0 * 256;
+        const unsigned off = (unsigned)i0 * step + (unsigned)c0 * 4u;
+        load_to_lds<16, 0>(r, window, lane_off, off);
+        if (i0 + 1 < ninstr) load_to_lds<16, 1024>(r, window, lane_off, off + step);
+        if (i0 + 2 < ninstr) load_to_lds<16, 2048>(r, window, lane_off, off + 2 * step);
+        if (i0 + 3 < ninstr) load_to_lds<16, 3072>(r, window, lane_off, off + 3 * step);
+    }
+}
+
+template <int NCH, int UNITS, bool QUADS>
+__global__ __launch_bounds__(kResThreads) void wgrad_stream_kernel(const float* __restrict__ xT,
+                                                                   const unsigned short* __restrict__ idx16,
+                                                                   const float* __restrict__ g,
+                                                                   float* __restrict__ gw,
+                                                                   float* __restrict__ bias_grad, int B, int N,
+                                                                   int L, int K, int nchunks, int n1, int ipb1,
+                                                                   int ipb2) {
+    extern __shared__ __align__(16) float xs[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int blk = blockIdx.x;
+    static_assert(UNITS % NCH == 0 && UNITS <= kResUnits, "whole labels per thread");
+    constexpr int kItems = UNITS / NCH;
+    const long long total_items = NCH == 1 ? (long long)L * nchunks : (long long)L;
+    const long long i_begin = blk < n1 ? (long long)blk * ipb1 : (long long)n1 * ipb1 + (long long)(blk - n1) * ipb2;
+    const long long i_end = min(i_begin + (blk < n1 ? ipb1 : ipb2), total_items);
+    const int nbt = (B + kTileBatch - 1) / kTileBatch;
+
+    float res[UNITS][kWgChunk];
+#pragma unroll
+    for (int q = 0; q < UNITS; ++q)
+#pragma unroll
+        for (int k = 0; k < kWgChunk; ++k) res[q][k] = 0.f;
+    float gsum[kItems];
+#pragma unroll
+    for (int q = 0; q < kItems; ++q) gsum[q] = 0.f;
+
+    // the thread's items (clamped, so that every address stays in bounds), their labels, and which of them the
+    // wavefront really has (wave-uniform; once false it stays false)
+    long long item[kItems];
+    unsigned jq[kItems];
+    bool act[kItems];
+#pragma unroll
+    for (int qq = 0; qq < kItems; ++qq) {
+        const long long ibase = i_begin + (long long)qq * kResThreads;
+        act[qq] = __builtin_amdgcn_readfirstlane((int)(ibase + (long long)(threadIdx.x & ~63u) < i_end)) != 0;
+        item[qq] = max(min(ibase + (long long)threadIdx.x, i_end - 1), 0ll);
+        jq[qq] = NCH == 1 ? (unsigned)(item[qq] % L) : (unsigned)item[qq];
+    }
+    const lds_f32_ptr gslice = (lds_f32_ptr)xs + (size_t)N * kTileBatch + wave * kSliceFloats;
+    // byte address of the lane's column of the slice; register group c of the lane holds batch entries 4 (c ^ t) ...
+    const unsigned gcol = (unsigned)(size_t)gslice + (unsigned)lane * 4u;
+    const unsigned tsk = (unsigned)(lane & 7) << 10;       // 4 rows of 256 bytes per group
+
+    // out_grad rows [32 bt, 32 bt + 32) as a buffer (rows beyond the batch read as zero); bt == nbt: an empty buffer,
+    // whose loads write zeros
+    auto g_rows = [&](int bt) {
+        const int b0 = bt * kTileBatch;
+        const int nrows = bt < nbt ? min(kTileBatch, B - b0) : 0;
+        return make_rsrc(g + (size_t)(bt < nbt ? b0 : 0) * (size_t)L, (size_t)nrows * (size_t)L * sizeof(float));
+    };
+    const unsigned gstride = (unsigned)L * 4u;
+    // row b of that buffer for the 64 labels `label` of the wavefront -> row b of the slice, without passing through registers
+    auto fetch_g_row = [&](const buffer_rsrc& r, unsigned label, auto bc) {
+        constexpr int b = decltype(bc)::value;
+        load_to_lds<4, (b & 15) * 256>(r, gslice + (b & 16) * 64, label * 4u, (unsigned)b * gstride);
+    };
+    // The same, four rows per instruction (16 bytes per lane: lanes 16 r ... 16 r + 15 fetch row 4 m + r for the labels
+    // first ... first + 63, which land in the slice exactly as the row-by-row loads put them).  For wavefronts whose
+    // lanes have consecutive labels; lanes behind the wavefront's last item then receive the out_grad of labels that are
+    // not theirs, and never store anything.
+    const unsigned quad_off = (unsigned)(lane >> 4) * gstride + (unsigned)(lane & 15) * 16u;
+    auto fetch_g_rows4 = [&](const buffer_rsrc& r, unsigned first, auto mc) {
+        constexpr int m = decltype(mc)::value;
+        load_to_lds<16, (m & 3) * 1024>(r, gslice + (m & 4) * 256, quad_off + first * 4u, (unsigned)(4 * m) * gstride);
+    };
+    // (QUADS: chosen by the launcher for NCH > 1 or a single chunk; otherwise chunk-major unit numbers wrap from the last
+    // label of one chunk to the first of the next inside a wavefront)
+    // quarter t of the 32 arranged entries of chunk c of item `it`
+    auto fetch_ids_quarter = [&](long long it, int c, int t, unsigned (&dst)[kWgChunk / 2]) {
+        const long long u = NCH == 1 ? it : (long long)c * L + it;
+        const uint4 v = *reinterpret_cast<const uint4*>(idx16 + arranged_quarter_offset(u, t));
+        dst[4 * t] = v.x; dst[4 * t + 1] = v.y; dst[4 * t + 2] = v.z; dst[4 * t + 3] = v.w;
+    };
+    unsigned idn[kWgChunk / 2];                            // ids of the next chunk, in flight
+    if (act[0]) {
+        const buffer_rsrc r0 = g_rows(0);
+        if constexpr (QUADS) static_for<kTileBatch / 4>([&](auto mc) { fetch_g_rows4(r0, (unsigned)__builtin_amdgcn_readfirstlane((int)jq[0]), mc); });
+        else static_for<kTileBatch>([&](auto bc) { fetch_g_row(r0, jq[0], bc); });
+#pragma unroll
+        for (int t = 0; t < kWgChunk / 8; ++t) fetch_ids_quarter(item[0], 0, t, idn);
+    }
+    const bool direct = (B % 4 == 0) && (N % 8 == 0) && (((uintptr_t)xT & 15) == 0);
+    for (int bt = 0; bt < nbt; ++bt) {
+        const int b0 = bt * kTileBatch;
+        __syncthreads();                                   // everyone is done with the previous tile
+        if (direct && b0 + kTileBatch <= B) {
+            stage_rows32_direct<kResThreads>(xs, xT, N, B, b0, wave, lane);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        } else {
+            stage_rows32<kResThreads, 8>(xs, xT, N, B, b0);
+        }
+        __syncthreads();
+        unsigned skew = (unsigned)(size_t)(lds_f32_ptr)xs + (unsigned)(lane & 7) * 16u;
+        asm volatile("" : "+v"(skew));                     // keep the LDS addresses out of loop-invariant hoisting
+#pragma unroll
+        for (int qq = 0; qq < kItems; ++qq) {
+            if (act[qq]) {
+                // what follows this item: the wavefront's next item of this batch tile, or its first of the next tile
+                const bool more = qq + 1 < kItems && act[qq + 1 < kItems ? qq + 1 : qq];
+                const int nbt_ = more ? bt : bt + 1;
+                const unsigned jn = more ? jq[qq + 1 < kItems ? qq + 1 : qq] : jq[0];
+                const long long itn = more ? item[qq + 1 < kItems ? qq + 1 : qq] : item[0];
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");          // the slice and idn have arrived
+                float gb[32];
+#pragma unroll
+                for (int c = 0; c < 8; ++c) {
+                    const lds_f32_ptr p = (lds_f32_ptr)(size_t)(gcol + (((unsigned)c << 10) ^ tsk));
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) gb[4 * c + i] = p[i * 64];
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");        // ... and has been read: refill it
+                // the next step's rows are requested one per connection of the walk below (a burst of 32 requests per
+                // wavefront finds the CU's memory queue full and stalls)
+                const buffer_rsrc rn = g_rows(nbt_);
+                const unsigned jn0 = (unsigned)__builtin_amdgcn_readfirstlane((int)jn);
+                if (bias_grad != nullptr) {
+                    float t = gsum[qq];
+#pragma unroll
+                    for (int b = 0; b < 32; ++b) t += gb[b];
+                    gsum[qq] = t;
+                }
+#pragma unroll
+                for (int c = 0; c < NCH; ++c) {
+                    if (c > 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    unsigned idp[kWgChunk / 2];
+#pragma unroll
+                    for (int t = 0; t < kWgChunk / 2; ++t) idp[t] = idn[t];
+                    // (no branch in here: the walk stays one basic block; behind the last step it fetches ids nobody uses
+                    // and zero rows from an empty buffer)
+                    static_for<kWgChunk>([&](auto kc) {
+                        constexpr int k = decltype(kc)::value;
+                        const unsigned e = (k & 1) ? (idp[k >> 1] >> 16) : idp[k >> 1];
+                        if constexpr (QUADS) {
+                            if (c == 0 && (k & 3) == 0) fetch_g_rows4(rn, jn0, std::integral_constant<int, k / 4>{});
+                        } else {
+                            if (c == 0) fetch_g_row(rn, jn, kc);
+                        }
+                        if ((k & 7) == 5) fetch_ids_quarter(c + 1 < NCH ? item[qq] : itn, c + 1 < NCH ? c + 1 : 0, k >> 3, idn);
+                        float4 xv[8];
+                        wgrad_reads(((e & kArrIdMask) << 7) + skew, xv);
+                        __builtin_amdgcn_sched_barrier(0);
+                        res[qq * NCH + c][k] = wgrad_dot(xv, gb, res[qq * NCH + c][k]);
+                        __builtin_amdgcn_sched_barrier(0);
+                    });
+                    asm volatile("" ::: "memory");
+                }
+            }
+        }
+    }
+    // Epilogue, each wavefront on its own: the sums go back into connection order through the wavefront's slice (128
+    // bytes per lane; the 16-byte groups of a lane's row are swizzled by lane bits 1-3 so that lanes which write the
+    // same connection number -- a lookup that already is in arranged order -- spread over the banks).
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // nothing is on its way into the slice any more
+    const unsigned srow = (unsigned)(size_t)gslice + (unsigned)lane * 128u;
+    const unsigned sw = ((unsigned)lane >> 1) & 7u;
+    const bool vec4 = (K % 4 == 0) && (((uintptr_t)gw & 15) == 0);
+    // (the entries of all the thread's units are requested before the first is used: one memory round trip, not one per unit)
+    unsigned ent[UNITS][kWgChunk / 2];
+#pragma unroll
+    for (int qq = 0; qq < kItems; ++qq)
+#pragma unroll
+        for (int cc = 0; cc < NCH; ++cc) {
+            const long long u = NCH == 1 ? item[qq] : (long long)cc * L + item[qq];
+#pragma unroll
+            for (int t = 0; t < kWgChunk / 8; ++t) {
+                uint4 v = make_uint4(0u, 0u, 0u, 0u);
+                if (act[qq]) v = *reinterpret_cast<const uint4*>(idx16 + arranged_quarter_offset(u, t));
+                ent[qq * NCH + cc][4 * t] = v.x; ent[qq * NCH + cc][4 * t + 1] = v.y;
+                ent[qq * NCH + cc][4 * t + 2] = v.z; ent[qq * NCH + cc][4 * t + 3] = v.w;
+            }
+        }
+#pragma unroll
+    for (int qq = 0; qq < kItems; ++qq) {
+        if (act[qq]) {
+            const long long it = i_begin + (long long)qq * kResThreads + threadIdx.x;
+            const bool mine = it < i_end;
+#pragma unroll
+            for (int cc = 0; cc < NCH; ++cc) {
+                const int c = NCH == 1 ? (int)(item[qq] / L) : cc;
+                const int j = NCH == 1 ? (int)(item[qq] - (long long)c * L) : (int)item[qq];
+                const int k0 = c * kWgChunk;
+                if (mine && bias_grad != nullptr && (NCH == 1 ? c == 0 : cc == 0)) bias_grad[j] = gsum[qq];
+#pragma unroll
+                for (int i = 0; i < kWgChunk; ++i) {
+                    const unsigned w = ent[qq * NCH + cc][i >> 1];
+                    const unsigned conn = ((i & 1) ? (w >> 16) : (w & 0xffffu)) >> kArrIdBits;
+                    *(lds_f32_ptr)(size_t)(srow + ((conn ^ (sw << 2)) << 2)) = res[qq * NCH + cc][i];
+                }
+                float* grow = gw + (size_t)j * K + k0;
+                if (QUADS && vec4 && k0 + kWgChunk <= K) {
+                    // lanes of consecutive labels: instruction t stores the rows of lanes 8 t ... 8 t + 7, eight lanes per row,
+                    // so that a store covers whole 128-byte rows (1 KB in one piece at fan-in 32) instead of 16 bytes of 64 rows
+                    const long long it0 = __builtin_amdgcn_readfirstlane((int)(it - lane));   // (the wavefront's first item, below 2^31: L < 2^25 labels)
+                    const int j0 = NCH == 1 ? (int)(it0 % L) : (int)it0;
+                    (void)j;
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) {
+                        const unsigned r = (unsigned)(8 * t) + ((unsigned)lane >> 3), q = (unsigned)lane & 7u;
+                        const unsigned rsw = (r >> 1) & 7u;
+                        const lds_v4f v = *(lds_v4f_ptr)(size_t)((unsigned)(size_t)gslice + r * 128u + ((q ^ rsw) << 4));
+                        if (it0 + (long long)r < i_end)
+                            *reinterpret_cast<float4*>(gw + (size_t)(j0 + (int)r) * K + k0 + 4 * q) = make_float4(v.x, v.y, v.z, v.w);
+                    }
+                } else if (vec4 && k0 + kWgChunk <= K) {
+#pragma unroll
+                    for (int t = 0; t < kWgChunk / 4; ++t) {
+                        const lds_v4f v = *(lds_v4f_ptr)(size_t)(srow + (((unsigned)t ^ sw) << 4));
+                        if (mine) *reinterpret_cast<float4*>(grow + 4 * t) = make_float4(v.x, v.y, v.z, v.w);
+                    }
+                } else {
+                    for (int k = 0; k < kWgChunk; ++k) {
+                        const float v = *(lds_f32_ptr)(size_t)(srow + (((unsigned)k ^ (sw << 2)) << 2));
+                        if (mine && k0 + k < K) grow[k] = v;
+                    }
                 }
             }
         }
@@ -337,15 +617,34 @@ int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float
         };
         if (plan != nullptr && plan->idx16 != nullptr) {
             // the unit slots of the final reordering need 144 bytes per thread
-            const size_t lds = std::max(tile_lds_bytes(d.N), (size_t)kResThreads * kSlotPitch * sizeof(float));
+            // with room for the wavefronts' out_grad slices behind the tile of x: the streaming kernel
+            // (and rows of out_grad of at least 256 bytes: the LDS-direct loads take their destination's offset inside the
+            // slice back out of the scalar offset of the row, which must not become negative)
+            const bool stream = tile_lds_bytes(d.N) + (size_t)(kResThreads / 64) * kSliceFloats * sizeof(float) <= kLdsPerWorkgroup &&
+                                d.L >= 64;
+            const size_t lds = std::max(tile_lds_bytes(d.N) + (stream ? (size_t)(kResThreads / 64) * kSliceFloats * sizeof(float) : 0),
+                                        (size_t)kResThreads * kSlotPitch * sizeof(float));
             // a label of two or four chunks: all its units in one thread (its out_grad values are loaded once per
             // batch tile instead of once per chunk); the work is then split by labels, not by units
 #define FFI_LAUNCH_ARRANGED(NCH, UNITS)                                                                                                \
             do {                                                                                                                       \
                 split(NCH == 1 ? (long long)d.L * nchunks : (long long)d.L, (long long)(UNITS / NCH) * kResThreads);                   \
-                FFI_HIP_TRY(hipFuncSetAttribute((const void*)wgrad_arranged_kernel<NCH, UNITS>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
-                hipLaunchKernelGGL((wgrad_arranged_kernel<NCH, UNITS>), dim3((unsigned)(n1 + n2)), dim3(kResThreads), lds, s, xT, plan->idx16, g, gw, \
-                                   bias_grad, d.B, d.N, d.L, d.K, nchunks, n1, ipb, ipb2);                                             \
+                if (stream) {                                                                                                          \
+                    constexpr bool kQuads = NCH > 1;   /* a wavefront's lanes hold consecutive labels */                               \
+                    if (kQuads || nchunks == 1) {                                                                                      \
+                        FFI_HIP_TRY(hipFuncSetAttribute((const void*)wgrad_stream_kernel<NCH, UNITS, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
+                        hipLaunchKernelGGL((wgrad_stream_kernel<NCH, UNITS, true>), dim3((unsigned)(n1 + n2)), dim3(kResThreads), lds, s, xT, plan->idx16, g, gw, \
+                                           bias_grad, d.B, d.N, d.L, d.K, nchunks, n1, ipb, ipb2);                                     \
+                    } else {                                                                                                           \
+                        FFI_HIP_TRY(hipFuncSetAttribute((const void*)wgrad_stream_kernel<NCH, UNITS, kQuads>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
+                        hipLaunchKernelGGL((wgrad_stream_kernel<NCH, UNITS, kQuads>), dim3((unsigned)(n1 + n2)), dim3(kResThreads), lds, s, xT, plan->idx16, g, gw, \
+                                           bias_grad, d.B, d.N, d.L, d.K, nchunks, n1, ipb, ipb2);                                     \
+                    }                                                                                                                  \
+                } else {                                                                                                               \
+                    FFI_HIP_TRY(hipFuncSetAttribute((const void*)wgrad_arranged_kernel<NCH, UNITS>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
+                    hipLaunchKernelGGL((wgrad_arranged_kernel<NCH, UNITS>), dim3((unsigned)(n1 + n2)), dim3(kResThreads), lds, s, xT, plan->idx16, g, gw, \
+                                       bias_grad, d.B, d.N, d.L, d.K, nchunks, n1, ipb, ipb2);                                         \
+                }                                                                                                                      \
             } while (0)
             if (nchunks == 2) FFI_LAUNCH_ARRANGED(2, 4);
             else if (nchunks == 4) FFI_LAUNCH_ARRANGED(4, 4);
@@ -374,3 +673,4 @@ int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float
 }
 
 }  // namespace ffi
+

@@ -181,7 +181,11 @@ def test_code_paths(ffi, shape, transposed):
                                    (48, 1300, 2000, 20),
                                    (96, 512, 20000, 64),     # two chunks per label, both held by one thread
                                    (64, 300, 2600, 128),      # four chunks per label
-                                   (32, 64, 360000, 32)])     # enough units per CU for the kernel that holds three units per thread
+                                   (32, 64, 360000, 32),      # enough units per CU for the kernel that holds three units per thread
+                                   (70, 768, 5000, 96),       # three chunks per label: unit numbers wrap inside a wavefront (row-by-row out_grad fetches)
+                                   (129, 763, 70, 32),        # one sample in the fifth batch tile, odd width (x staged through registers), 70 labels
+                                   (32, 768, 64, 8),          # the fewest labels the streaming kernel takes
+                                   (64, 776, 4000, 32)])      # x tile and out_grad slices do not fit the LDS together: the kernel without slices
 def test_planned_weight_grad_code_paths(ffi, shape):
     B, N, L, K = shape
     x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=B + K)
