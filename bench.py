@@ -31,7 +31,7 @@ PROFILE_DIR = os.path.join(ROOT, "profiles")
 # GPU kernels behind each pass (one C-ABI call)
 PASS_KERNELS = {
     "forward": "fwd_lane32_kernel",
-    "weight_grad": "wgrad_arranged_kernel",
+    "weight_grad": "wgrad_stream_kernel",
     "input_grad": "igrad_permute_weights_kernel + igrad_tile_kernel + igrad_reduce_kernel",
 }
 WIDE_PASS_KERNELS = {
@@ -57,6 +57,103 @@ def measured_traffic(config_name):
     return out, (f"profiles/{os.path.basename(path)}" + (f" ({stamp})" if stamp else "")) if out else None
 
 
+def measured_pipe_load(config_name):
+    """Per pass: VALU wavefront-instructions and LDS-busy cycles per launch, from the same counter summary (lines
+    `valu_insts <pass> <n>` = SQ_INSTS_VALU, `lds_busy_cycles <pass> <n>` = SQ_LDS_IDX_ACTIVE, summed over the pass's kernels)."""
+    path = os.path.join(PROFILE_DIR, f"ffi_{config_name}_counters.txt")
+    out = {"valu_insts": {}, "lds_busy_cycles": {}}
+    if os.path.exists(path):
+        for line in open(path):
+            f = line.split()
+            if len(f) >= 3 and f[0] in out:
+                out[f[0]][f[1]] = float(f[2])
+    return out
+
+
+def attainable(cfg, alg, config_name):
+    """What this design would reach if, in every pass, the slowest of its three resources ran without a gap: the VALU at
+    one instruction per 4 clocks and SIMD with the instruction counts the kernels have NOW (multiply-adds plus address,
+    unpacking and padding overhead, SQ_INSTS_VALU), the LDS with the cycles per read it shows NOW (bank conflicts
+    included, SQ_LDS_IDX_ACTIVE), HBM at its published peak.  Measured time above this is lost overlap (phases that wait
+    for each other); this figure above the HBM floor is the price of the instruction mix, the padding and the conflicts."""
+    load = measured_pipe_load(config_name)
+    if not load["valu_insts"]:
+        return None
+    simds, cus, clk = 1024.0, 256.0, 2.4e9
+    per_pass = {}
+    for k in ("forward", "weight_grad", "input_grad"):
+        if k not in load["valu_insts"] or k not in load["lds_busy_cycles"]:
+            return None
+        valu = load["valu_insts"][k] * 4.0 / simds / clk
+        lds = load["lds_busy_cycles"][k] / cus / clk
+        hbm = alg[k] / (HBM_PEAK_GBPS * 1e9)
+        per_pass[k] = {"valu_ms": round(valu * 1e3, 4), "lds_ms": round(lds * 1e3, 4), "hbm_ms": round(hbm * 1e3, 4),
+                       "bound_ms": round(max(valu, lds, hbm) * 1e3, 4)}
+    step = sum(v["bound_ms"] for v in per_pass.values())
+    return {"ms_per_step": round(step, 4), "samples_per_s": round(cfg.batch / (step * 1e-3), 1),
+            "frac_of_hbm_peak": round(alg["total"] / (step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4), "per_pass": per_pass,
+            "basis": f"SQ_INSTS_VALU and SQ_LDS_IDX_ACTIVE per launch from profiles/ffi_{config_name}_counters.txt, 1,024 SIMDs x 4 clocks per "
+                     "instruction, 256 CUs, 2.4 GHz, HBM 8 TB/s; per pass the largest of the three"}
+
+
+def rewire_costs(pkg, cfg, x, lookup, w, g, tp, stream):
+    """What a rewiring step costs the backward pass (the reference rewires every `rewire_interval` steps,
+    sparse/optimizer.py:68-74; tasks/amazon670k-cascade.json: 1000, also 100): the plan build alone, the first
+    ffi_backward_f32 after the library's own ffi_rewire_f32 (rebuilds the plan first), and after an edit of the lookup
+    by foreign code (served once by the kernels that read the lookup directly, then rebuilt).  Host-timed, each call
+    bracketed by synchronisations; on a copy of the lookup."""
+    import ctypes
+
+    import torch
+    B, N, L, K = cfg.batch, cfg.num_features, cfg.num_units, cfg.fan_in
+    lib, check, sh = pkg._lib.lib(), pkg._lib.check, stream.cuda_stream
+    ptr = lambda a: a.data_ptr()  # noqa: E731
+    lookup2 = lookup.clone()
+    gx, gw = torch.empty_like(x), torch.empty_like(w)
+
+    def timed(fn):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3
+
+    backward = lambda: check(lib.ffi_backward_f32(ptr(x), ptr(lookup2), ptr(w), ptr(g), ptr(gx), ptr(gw), B, N, L, K, int(tp), sh))  # noqa: E731
+    for _ in range(5):
+        backward()
+    normal = min(timed(backward) for _ in range(5))
+    plan = ctypes.c_void_p()
+    check(lib.ffi_plan_create(ptr(lookup2), L, K, N, B, sh, ctypes.byref(plan)))
+    build = min(timed(lambda: check(lib.ffi_plan_refresh(plan, ptr(lookup2), sh))) for _ in range(3))
+    check(lib.ffi_plan_destroy(plan))
+    thr = torch.empty(1, device="cuda")
+    gen = torch.Generator(device="cuda").manual_seed(11)
+
+    def rewire():
+        check(lib.ffi_select_threshold_f32(ptr(w), L * K, (L * K) // 100, ptr(thr), sh))
+        check(lib.ffi_rewire_f32(ptr(lookup2), ptr(w), None, 0, L * K, N, ptr(thr), 12345, None, sh))
+
+    rewire_ms = timed(rewire)
+    first_library = timed(backward)
+    after_library = timed(backward)
+    pos = torch.randint(0, L * K, ((L * K) // 100,), device="cuda", generator=gen)
+    lookup2.view(-1)[pos] = torch.randint(0, N, (pos.numel(),), device="cuda", generator=gen, dtype=torch.int32)
+    first_foreign = timed(backward)
+    second_foreign = timed(backward)
+    after_foreign = timed(backward)
+    out = {"backward_ms": round(normal, 4), "plan_build_ms": round(build, 4), "select_and_rewire_1pct_ms": round(rewire_ms, 4),
+           "first_backward_after_rewire_ms": {"library_rewire": round(first_library, 4), "foreign_in_place_edit": round(first_foreign, 4)},
+           "second_backward_after_rewire_ms": {"library_rewire": round(after_library, 4), "foreign_in_place_edit": round(second_foreign, 4)},
+           "third_backward_after_foreign_edit_ms": round(after_foreign, 4),
+           "note": "library route: ffi_rewire_f32 marks the cached plan outdated, the next backward rebuilds it and runs the plan-driven kernels; "
+                   "foreign route: the first backward runs the kernels that read the lookup directly (float atomics), the second rebuilds"}
+    extra_library = rewire_ms + first_library - normal
+    extra_foreign = (first_foreign - normal) + (second_foreign - normal)
+    out["amortised_ms_per_step"] = {f"rewire_interval_{i}": {"library_rewire": round(extra_library / i, 5), "foreign_in_place_edit": round(extra_foreign / i, 5)}
+                                    for i in (100, 1000)}
+    return out
+
+
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -75,6 +172,13 @@ def parse_args():
                     help="also time one training step of the layer (forward + squared-hinge loss gradient in one kernel, "
                          "backward over the non-zero gradients and Adam in one call) with the bias set so that this share of the loss "
                          "gradients is non-zero; reported under 'train_step' in the same JSON line")
+    ap.add_argument("--preload-ms", type=float, default=150.0,
+                    help="milliseconds of untimed steps in front of the warm-up: the GPU's clocks settle under load within tens of "
+                         "milliseconds, and a 20-step run (14 ms) would otherwise be timed on the ramp")
+    ap.add_argument("--no-rewire-costs", action="store_true", help="skip the plan-build / first-backward-after-rewiring timings")
+    ap.add_argument("--sweep", action="store_true",
+                    help="instead of the benchmark line: batch x width x labels x fan-in grid of the three passes, one CSV line each "
+                         "(gpurun_out/sweep.csv), in the manner of the reference's testing/detailed-bench.cpp:26-112")
     ap.add_argument("--copy-bytes", type=int, default=0,
                     help="also run one plain device copy kernel of this many bytes (read N, write N): the "
                          "known-size reference that rocprofv3 FETCH_SIZE/WRITE_SIZE readings are scaled by")
@@ -379,6 +483,14 @@ def main():
         check(lib.ffi_forward_f32(ptr(x), ptr(lookup), ptr(w), ptr(out), B, N, L, K, int(tp), sh))
         check(lib.ffi_backward_f32(ptr(x), ptr(lookup), ptr(w), ptr(g), ptr(gx), ptr(gw), B, N, L, K, int(tp), sh))
 
+    # untimed pre-load: steps until the GPU has been busy for --preload-ms (its clocks settle under load)
+    preload_steps, t_pre = 0, time.perf_counter()
+    while (time.perf_counter() - t_pre) * 1e3 < args.preload_ms:
+        for _ in range(10):
+            step()
+        torch.cuda.synchronize()
+        preload_steps += 10
+    preload_ms = (time.perf_counter() - t_pre) * 1e3
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -388,6 +500,16 @@ def main():
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed * 1e3 / args.steps
+    # spread of single steps, outside the timed region (an event between two steps costs a few microseconds)
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+    marks[0].record(stream)
+    for i in range(args.steps):
+        step()
+        marks[i + 1].record(stream)
+    marks[-1].synchronize()
+    singles = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
+    step_spread = {"min": round(singles[0], 4), "median": round(singles[len(singles) // 2], 4), "max": round(singles[-1], 4),
+                   "note": "per-step event timing in a second loop of the same length (includes the event records)"}
 
     # per-kernel durations with events on the launch stream (explicit plan: the kernel alone)
     import ctypes
@@ -400,6 +522,8 @@ def main():
         "input_grad": lambda: check(lib.ffi_input_grad_planned_f32(plan, ptr(w), ptr(g), ptr(gx), B, int(tp), sh)),
     }
     kernel_ms = {name: time_kernel(fn, stream, iters) for name, fn in kernels.items()}
+    plan_info = (ctypes.c_int64 * 8)()
+    check(lib.ffi_plan_info(plan, plan_info))
     check(lib.ffi_plan_destroy(plan))
     alg = synth.algorithmic_bytes(cfg)
     dominant = max(kernel_ms, key=kernel_ms.get)
@@ -409,10 +533,11 @@ def main():
     pass_kernels = dict(PASS_KERNELS if narrow else WIDE_PASS_KERNELS)
     if N <= 608 and B > 32:
         pass_kernels["forward"] = "fwd_lane64_kernel"       # batch tiles of 64 when the [N][64] tile fits in LDS
-    threads, nbt = (N + 63) // 64 * 64, (B + 31) // 32
-    if narrow and threads <= 768 and (nbt <= 2 or (nbt <= 4 and threads >= 704)) and K <= 32:
+    if narrow and plan_info[0] and plan_info[1]:
         # the plan's tiles are small enough for the walking kernel to keep the tile's weights in LDS: no permutation kernel
         pass_kernels["input_grad"] = "igrad_tile_kernel + igrad_reduce_kernel"
+    if narrow and not (N * 128 + 65536 <= 160 * 1024 and L >= 64):
+        pass_kernels["weight_grad"] = "wgrad_arranged_kernel"        # no room for the out_grad slices behind the tile of x
     flops = 2.0 * B * L * K
     roofline = {
         "bound": "hbm",
@@ -451,13 +576,21 @@ def main():
                                f"{L} labels, fan-in {K}, features [{'N,B' if tp else 'B,N'}]"
                                + (", connections of each label reordered by ffi_arrange_connections_f32" if args.arranged else ""),
                    "label_samples_per_s": round(B * L / (ms_per_step * 1e-3), 1)},
+        "preload_ms": round(preload_ms, 1),
+        "preload_steps": preload_steps,
+        "step_ms": step_spread,
         "roofline": roofline,
+        "attainable": attainable(cfg, alg, cfg.name) if narrow else None,
         "parity": parity,
         # device memory the library holds beside the caller's tensors after these steps (cached plan + workspaces),
         # and what ffi_workspace_bytes() predicts for this shape
         "library_bytes": int(lib.ffi_cache_bytes()),
         "library_bytes_estimate": int(lib.ffi_workspace_bytes(B, N, L, K, int(tp), 3)),
+        "plan": {"tiled": bool(plan_info[0]), "weights_in_lds": bool(plan_info[1]), "tile_labels": int(plan_info[2]), "tiles": int(plan_info[4]),
+                 "slots_per_connection": round(plan_info[5] * 64 / (L * K), 4) if plan_info[0] else None, "bytes": int(plan_info[6])},
     }
+    if narrow and not args.no_rewire_costs:
+        result["rewiring"] = rewire_costs(pkg, cfg, x, lookup, w, g, tp, stream)
     if args.train_step > 0:
         result["train_step"] = train_step(pkg, cfg, x, lookup, w, tp, args.train_step, stream, max(3, min(args.steps, 20)))
     if cpu_report is not None:

@@ -96,6 +96,22 @@ struct PlannedWeightGrad {
     float* bias_grad = nullptr;
 };
 
+// The library's own in-place editors of a lookup matrix (ffi_rewire_f32, ffi_arrange_connections_f32) tell the cache:
+// every cached plan built from that buffer on this device is marked outdated on the host, so the next backward call
+// rebuilds it before it enqueues anything (no walk of an outdated plan, no recomputing kernels, reproducible sums).
+// The device-side check stays for edits the library does not see (foreign kernels writing into the buffer).
+void mark_cached_plans_outdated(const int32_t* lookup) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) return;
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    for (ffi_plan* p : g_cache) {
+        if (p->device != dev || p->lookup == nullptr) continue;
+        // (an edit anywhere inside the buffer the plan was built from counts)
+        const int32_t* end = p->lookup + (size_t)p->L * (size_t)p->K;
+        if (lookup >= p->lookup && lookup < end) p->edited_by_library = true;
+    }
+}
+
 void drop_cached_plan(ffi_plan* p) {
     for (size_t i = 0; i < g_cache.size(); ++i)
         if (g_cache[i] == p) { g_cache.erase(g_cache.begin() + i); break; }
@@ -127,7 +143,7 @@ int input_grad_cached(const int32_t* lookup, const float* weights, const float* 
     bool seen = false, current = true;
     unsigned long long bad = 0;
     FFI_TRY(plan_guard_poll(p, &seen, &current, &bad));
-    if (seen && !current) {
+    if (p->edited_by_library || (seen && !current)) {
         // the lookup changed under the plan (the calls since then were served by the recomputing kernels);
         // the build fingerprints the present content, so this call needs no check
         const int st = plan_build(p, lookup, s);
@@ -476,6 +492,7 @@ int ffi_rewire_f32(int32_t* lookup, const float* weights, float* const* arrays, 
         if (!arrays[i]) return FFI_ERR_NULL_POINTER;
     if (count <= 0 || num_features <= 0) return FFI_ERR_BAD_SHAPE;
     if (num_features >= INT32_MAX) return FFI_ERR_TOO_LARGE;
+    mark_cached_plans_outdated(lookup);
     return launch_rewire(lookup, weights, arrays, n_arrays, (size_t)count, (unsigned)num_features, threshold,
                          (unsigned long long)seed, (long long*)rewired_count, (hipStream_t)stream);
 }
@@ -509,6 +526,19 @@ int ffi_plan_destroy(ffi_plan* plan) {
     if (!plan) return FFI_OK;
     plan_free(plan);
     delete plan;
+    return FFI_OK;
+}
+
+int ffi_plan_info(const ffi_plan* plan, int64_t info[8]) {
+    if (!plan || !info) return FFI_ERR_NULL_POINTER;
+    info[0] = plan->tiled ? 1 : 0;
+    info[1] = plan->w_in_lds ? 1 : 0;
+    info[2] = plan->tile_labels;
+    info[3] = plan->threads;
+    info[4] = plan->tiles;
+    info[5] = plan->total_rows;
+    info[6] = (int64_t)plan->bytes;
+    info[7] = plan->idx16 != nullptr ? 1 : 0;
     return FFI_OK;
 }
 
@@ -546,6 +576,7 @@ int ffi_arrange_connections_f32(int32_t* lookup, float* const* arrays, int n_arr
         if (!arrays[i]) return FFI_ERR_NULL_POINTER;
     Dims d;
     FFI_TRY(check_dims(1, 1, num_units, fan_in, 0, &d));
+    mark_cached_plans_outdated(lookup);
     return launch_arrange_in_place(lookup, arrays, n_arrays, d.L, d.K, (hipStream_t)stream);
 }
 
@@ -601,7 +632,7 @@ size_t ffi_workspace_bytes(int64_t batch, int64_t num_features, int64_t num_unit
             const size_t rows = (size_t)(mu + 2.6 * std::sqrt(mu) + 3.0);
             const size_t slots = tiles * slices * rows * 64;
             total += slots * 2 * 2 + (tiles * slices + 1) * 4 + L * 2;                  // 4 bytes per slot (lab16 + pos16, or slot32), slice_off, rowpos
-            if (tile_path_fits(d.N) && d.N < (1 << kArrIdBits)) total += L * ((K + 31) / 32) * 32 * 2;   // idx16
+            if (tile_path_fits(d.N) && d.N < (1 << kArrIdBits)) total += arranged_words((long long)(L * ((K + 31) / 32))) * 2;   // idx16
             if (!w_in_lds) features_slot = std::max(features_slot, slots * 4);         // weights in slot order
             const size_t nbt = (B + 31) / 32;
             const size_t per_cu = (size_t)tiled_workgroups_per_cu((int)threads, (int)TL, d.K, w_in_lds, (int)((B + 31) / 32));

@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 #include <cstdint>
 #include <cstddef>
+#include <vector>
 
 #include "ffi_hip.h"
 
@@ -238,8 +239,16 @@ struct ffi_plan {
     unsigned long long guard_seq = 0;         // checks enqueued so far
     unsigned long long guard_seen = 0;        // number of the last check whose result the host has looked at
     bool guard_stale = false;                 // such a look found the plan outdated and nobody has acted on it yet
+    bool edited_by_library = false;           // the library itself has enqueued an in-place edit of `lookup` since the plan was built
     hipStream_t guard_stream = nullptr;       // the stream of that check
     size_t bytes = 0;
+    // Device buffers behind the arrays above (`owned`) and buffers of an earlier build kept for the next one (`spare`):
+    // a rebuild after rewiring needs arrays of nearly the same sizes, and hipMalloc / hipFree of 100-MB buffers cost
+    // more than the kernels that fill them.
+    struct Buffer { void* ptr; size_t bytes; };
+    std::vector<Buffer> owned, spare;
+    hipStream_t helper_stream = nullptr;      // the arranged ids are built beside the tiled form (created on first use)
+    hipEvent_t helper_event = nullptr;
     int batch_hint = 0;                       // batch size the plan is expected to be used with (0 = unknown); steers layout choices only
     bool w_in_lds = false;                    // tiled form: tiles small enough for the walking kernel to keep the tile's weights in LDS too
 };

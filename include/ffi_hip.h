@@ -14,7 +14,10 @@
  *     result / out_grad are [batch, num_units]; feature_grad has the shape of features;
  *   - lookup holds column ids in [0, num_features); int32 and uint32 share the entry points
  *     (same bits for valid ids), duplicates inside a row are legal and accumulate.  The backward entry points
- *     reject ids outside that range (FFI_ERR_BAD_LOOKUP); the forward entry points do not look (neither does the
+ *     report ids outside that range as FFI_ERR_BAD_LOOKUP: at once when they build their view of the lookup (first
+ *     use, after ffi_rewire_f32 / ffi_arrange_connections_f32, ffi_plan_create / ffi_plan_refresh), and one call
+ *     late when foreign code wrote the id into a lookup they have already seen (the call that met it skipped the
+ *     connection and returned FFI_OK); the forward entry points do not look (neither does the
  *     reference in release builds, kernel_data.cu.h:211) and their results for such a lookup are undefined, not
  *     just for the offending connection: the narrow-input kernels keep two 16-bit ids per register, so an id of
  *     65,536 or more also changes its neighbour, and an id in [num_features, 65,536) reads whatever lies behind
@@ -99,8 +102,18 @@ int ffi_forward_noalloc_f32(const float* features, const int32_t* lookup, const 
  * Either output pointer may be NULL to skip that gradient.  The input gradient uses no float
  * atomics: results are bit-identical from run to run.  It needs a column-ordered view of `lookup`
  * which is built on the device on first use and cached inside the library, keyed on the lookup
- * pointer and shape and guarded by a content fingerprint that is re-checked on every call, so
- * in-place edits of lookup (rewiring, sparse/custom_layer.py:32-43) are picked up.
+ * pointer and shape, so in-place edits of lookup (rewiring, sparse/custom_layer.py:32-43) must be picked up:
+ *   - edits made through this library (ffi_rewire_f32, ffi_arrange_connections_f32) mark the cached view outdated
+ *     on the host, and the next backward call rebuilds it before it enqueues anything (that call synchronises
+ *     `stream` and takes the time of a plan build, about 3 ms at 670,091 x 32 connections; results stay
+ *     bit-reproducible);
+ *   - edits by foreign code are caught by a content fingerprint that a kernel re-checks on every call, on the
+ *     device, without a host wait: every call enqueued before the host has seen the verdict -- the first call after
+ *     the edit and as many more as the host runs ahead of the GPU -- computes correct results by kernels that read
+ *     the lookup directly (one thread per connection, float atomics for the input gradient: much slower, about
+ *     20 ms at that size, and with the atomics' summation order); the first call made after the verdict has reached
+ *     the host rebuilds the view.  Callers that edit the lookup themselves and care should hold an explicit plan
+ *     (ffi_plan_create / ffi_plan_refresh) or call ffi_arrange_connections_f32 afterwards.
  */
 int ffi_backward_f32(const float* features, const int32_t* lookup, const float* weights,
                      const float* out_grad, float* feature_grad, float* weight_grad,
@@ -133,6 +146,14 @@ int ffi_plan_create(const int32_t* lookup, int64_t num_units, int64_t fan_in, in
                     int64_t batch_hint, ffi_stream_t stream, ffi_plan** plan);
 int ffi_plan_refresh(ffi_plan* plan, const int32_t* lookup, ffi_stream_t stream);
 int ffi_plan_destroy(ffi_plan* plan);
+/*
+ * What a plan looks like (for benchmarks and logs; no counterpart in the reference).  info[0] = 1 for the tiled form
+ * (narrow inputs) or 0 for the blocked global form; [1] = 1 if the input-gradient kernel keeps a tile's weights in LDS;
+ * [2] labels per tile; [3] threads of the walking kernel; [4] tiles; [5] slot rows (64 slots each; slots / connections
+ * is the padding the walk pays); [6] bytes the plan holds on the device; [7] = 1 if it holds arranged column ids for
+ * the weight gradient.
+ */
+int ffi_plan_info(const ffi_plan* plan, int64_t info[8]);
 int ffi_input_grad_planned_f32(const ffi_plan* plan, const float* weights, const float* out_grad,
                                float* feature_grad, int64_t batch, int transposed, ffi_stream_t stream);
 
@@ -155,7 +176,8 @@ int ffi_weight_grad_planned_f32(const ffi_plan* plan, const float* features, con
  * place, per chunk of 32 connections, and applies the same permutation to up to four float matrices
  * of the same shape (weights, optimizer moments, ...; `arrays` is a HOST array of `n_arrays` device
  * pointers).  Results of all entry points are unchanged up to summation order; the call is
- * idempotent.  A caller that rewires (sparse/custom_layer.py:32-43) may call it again afterwards.
+ * idempotent.  A caller that rewires (sparse/custom_layer.py:32-43) may call it again afterwards.  Like
+ * ffi_rewire_f32 it marks any cached plan of `lookup` outdated.
  */
 int ffi_arrange_connections_f32(int32_t* lookup, float* const* arrays, int n_arrays,
                                 int64_t num_units, int64_t fan_in, ffi_stream_t stream);
@@ -386,8 +408,8 @@ int ffi_adam_step_f32(float* variable, float* m, float* v, const float* gradient
  * reference draws from TensorFlow's stream, which no other implementation reproduces -- and zeros in
  * arrays[0..n_arrays) (HOST array of up to four device pointers: the optimizer's moments,
  * sparse/optimizer.py:14-21).  Weights keep their values.  *rewired_count (device, may be NULL)
- * receives the number of positions changed.  Entry points that cache a plan of `lookup` notice the edit
- * through its fingerprint; an explicit plan needs ffi_plan_refresh.
+ * receives the number of positions changed.  The call marks any cached plan of `lookup` outdated: the next
+ * backward call through the stateless entry points rebuilds it first; an explicit plan needs ffi_plan_refresh.
  */
 int ffi_select_threshold_f32(const float* weights, int64_t count, int64_t k, float* threshold, ffi_stream_t stream);
 int ffi_rewire_f32(int32_t* lookup, const float* weights, float* const* arrays, int n_arrays, int64_t count,

@@ -222,6 +222,25 @@ def test_columns_fed_by_one_label_parity(ffi):
         assert rel_err(gw, o_gw) <= GRAD_RTOL
 
 
+def test_labels_that_list_a_column_twice(ffi):
+    # duplicates inside a row are legal and accumulate (backward.cpp:58-72 adds every connection).  The plan's fast slot
+    # placement works on a bitmap of (column, label) and hands tiles with such a label to the exact placement: here
+    # every third tile has some, the others none.
+    B, N, L, K = 48, 256, 6000, 16
+    x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=123)
+    rng = np.random.default_rng(9)
+    for j in rng.choice(L, 40, replace=False):
+        if (j // 256) % 3 == 0:
+            a, b = rng.choice(K, 2, replace=False)
+            lookup[j, a] = lookup[j, b]
+    lookup[17, :] = 5                                     # and one label that is a single column K times
+    gx, gw = hip_backward(ffi, x, lookup, w, g, False)
+    o_gx, o_gw = oracle.backward(x, lookup, w, g)
+    assert rel_err(gx, o_gx) <= GRAD_RTOL
+    assert rel_err(gw, o_gw) <= GRAD_RTOL
+    assert rel_err(hip_forward(ffi, x, lookup, w, False), oracle.forward(x, lookup, w)) <= FWD_RTOL
+
+
 def test_skewed_lookup_uses_the_global_plan(ffi):
     # every connection points at one of two columns: the padded tiled plan would explode, the
     # library must fall back to the global column order and still be exact to tolerance
@@ -328,6 +347,64 @@ def test_in_place_rewiring_is_picked_up(ffi):
     rebuilt = run()                                     # the host has seen the verdict: the plan is rebuilt
     assert rel_err(rebuilt, oracle.input_grad(x, lookup2, w, g)) <= GRAD_RTOL
     assert np.array_equal(rebuilt, run())               # plan-driven again: bit-identical from call to call
+
+
+def _label_sample_errors(lookup, w, g, x, gx, gw, B, N, K, labels):
+    """weight gradient of a label sample and the full input gradient against the oracle ([N,B] features)"""
+    o_gw = oracle.weight_grad(x, lookup[labels], w[labels], np.ascontiguousarray(g[:, labels]), transposed=True)
+    o_gx = oracle.input_grad(x, lookup, w, g, transposed=True)
+    return rel_err(gw[labels], o_gw), rel_err(gx, o_gx)
+
+
+@pytest.mark.parametrize("route", ["library", "foreign"])
+def test_rewiring_at_scale_both_routes(ffi, route):
+    # 262,144 labels x fan-in 32 over 768 columns, batch 64 (weights-in-LDS plan, streaming weight gradient).
+    # library: ffi_rewire_f32 edits the lookup and tells the plan cache -- the next backward rebuilds the plan first:
+    #   plan-driven kernels, bit-identical from call to call, never the recomputing kernels;
+    # foreign: a torch kernel edits the lookup -- the next backward is served by the recomputing kernels (correct up to
+    #   the atomics' summation order), the one after it rebuilds.
+    B, N, L, K = 64, 768, 262144, 32
+    rng = np.random.default_rng(5)
+    lookup = np.argsort(rng.random((L, N), dtype=np.float32), axis=1)[:, :K].astype(np.int32)
+    w = (rng.normal(size=(L, K)) / np.sqrt(K)).astype(np.float32)
+    x = np.maximum(rng.normal(size=(N, B)), 0).astype(np.float32)
+    g = (rng.normal(size=(B, L)) * 1e-2).astype(np.float32)
+    dx, dl, dw, dg = dev(x), dev(lookup), dev(w), dev(g)
+    gx, gw = torch.empty_like(dx), torch.empty_like(dw)
+    lib = ffi._lib.lib()
+
+    def run():
+        gx.fill_(float("nan")); gw.fill_(float("nan"))
+        ffi._lib.check(lib.ffi_backward_f32(dx.data_ptr(), dl.data_ptr(), dw.data_ptr(), dg.data_ptr(), gx.data_ptr(), gw.data_ptr(),
+                                            B, N, L, K, 1, stream()))
+        torch.cuda.synchronize()
+        return gx.cpu().numpy().copy(), gw.cpu().numpy().copy()
+
+    sample = rng.choice(L, 4096, replace=False)
+    a_gx, a_gw = run()
+    e = _label_sample_errors(lookup, w, g, x, a_gx, a_gw, B, N, K, sample)
+    assert max(e) <= GRAD_RTOL, e
+    if route == "library":
+        thr = ffi.fixed_fan_in_ops.select_threshold(dw.view(-1), (L * K) // 100)
+        ffi._lib.check(lib.ffi_rewire_f32(dl.data_ptr(), dw.data_ptr(), None, 0, L * K, N, thr.data_ptr(), 99, None, stream()))
+    else:
+        pos = torch.from_numpy(rng.choice(L * K, (L * K) // 100, replace=False)).cuda()
+        dl.view(-1)[pos] = torch.from_numpy(rng.integers(0, N, pos.numel()).astype(np.int32)).cuda()
+    torch.cuda.synchronize()
+    lookup2 = dl.cpu().numpy()
+    changed = int((lookup2 != lookup).sum())
+    assert changed > (L * K) // 200
+    b_gx, b_gw = run()                                   # the first backward after the edit
+    e = _label_sample_errors(lookup2, w, g, x, b_gx, b_gw, B, N, K, sample)
+    assert max(e) <= GRAD_RTOL, e
+    c_gx, c_gw = run()
+    e = _label_sample_errors(lookup2, w, g, x, c_gx, c_gw, B, N, K, sample)
+    assert max(e) <= GRAD_RTOL, e
+    d_gx, d_gw = run()
+    assert np.array_equal(c_gx, d_gx) and np.array_equal(c_gw, d_gw)      # plan-driven: bit-identical
+    if route == "library":
+        # the plan was rebuilt before the first backward enqueued anything: that call was plan-driven already
+        assert np.array_equal(b_gx, c_gx) and np.array_equal(b_gw, c_gw)
 
 
 @pytest.mark.parametrize("transposed", [False, True])
