@@ -75,8 +75,9 @@ int launch_transpose(const float* src, float* dst, int rows, int cols, hipStream
 int launch_forward(const float* x, const int32_t* idx, const float* w, const float* bias, float* out, const Dims& d,
                    hipStream_t s);
 // `plan` (may be null): a plan of the same lookup whose arranged copy of the column ids the kernel may use
+// `only_if_outdated` (may be null; without a plan only): device word of a lookup check -- the kernel returns at once unless it is 0
 int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float* gw, float* bias_grad, const Dims& d,
-                       hipStream_t s, const ffi_plan* plan = nullptr);
+                       hipStream_t s, const ffi_plan* plan = nullptr, const unsigned long long* only_if_outdated = nullptr);
 // any shape (the tile kernels cover narrow inputs only)
 int launch_forward_wide(const float* x, const int32_t* idx, const float* w, const float* bias, float* out, const Dims& d,
                         hipStream_t s);

@@ -321,8 +321,7 @@ constexpr int kFillChunk = 8192;
 __global__ void tile_fill_kernel(const int32_t* __restrict__ idx, const unsigned short* __restrict__ rowpos, int L, int K,
                                  int tile_labels, int zero_row, const unsigned* __restrict__ slice_off,
                                  unsigned short* __restrict__ lab16, unsigned short* __restrict__ pos16, unsigned pad_pos,
-                                 unsigned* __restrict__ slot32, const unsigned* __restrict__ only_flagged) {
-    if (only_flagged != nullptr && only_flagged[blockIdx.x] == 0u) return;     // (tiles the bitmap kernel has done)
+                                 unsigned* __restrict__ slot32) {
     __shared__ __align__(16) int keys[kFillChunk];
     __shared__ unsigned short rows_of[kPlanTileLabels];     // LDS row of each label of the tile
     const int t = blockIdx.x, nthreads = blockDim.x;
@@ -373,12 +372,12 @@ __global__ void tile_fill_kernel(const int32_t* __restrict__ idx, const unsigned
 // connections of the same bank half in ascending flat position: the order tile_fill_kernel produces), so the slots
 // are written by threads <-> connections, not by a column's thread scanning for them.  Padding goes to the slots no
 // connection takes (a column's thread knows them from its two totals).  A label that lists one column twice sets one
-// bit for two connections: such a tile is flagged and left to tile_fill_kernel, which the host runs afterwards for the
-// flagged tiles only.  Measured at 670,091 labels x fan-in 32 over 768 columns: 6.2 ms -> 0.1 ms.
+// bit for two connections: such a tile is placed by its columns' threads instead (see below), several times slower.
+// Measured at 670,091 labels x fan-in 32 over 768 columns: 6.2 ms -> 0.19 ms without such labels, 1.3 ms with some in every tile.
 __global__ void tile_fill_bitmap_kernel(const int32_t* __restrict__ idx, const unsigned short* __restrict__ rowpos, int L, int K,
                                         int tile_labels, int zero_row, const unsigned* __restrict__ slice_off,
                                         unsigned short* __restrict__ lab16, unsigned short* __restrict__ pos16, unsigned pad_pos,
-                                        unsigned* __restrict__ slot32, int words, unsigned* __restrict__ redo_flags) {
+                                        unsigned* __restrict__ slot32, int words) {
     extern __shared__ __align__(16) unsigned fill_lds[];
     const int t = blockIdx.x, nthreads = blockDim.x;
     unsigned* bm = fill_lds;                                                   // [nthreads][words] (words odd: no bank conflicts)
@@ -415,8 +414,41 @@ __global__ void tile_fill_bitmap_kernel(const int32_t* __restrict__ idx, const u
         }
     }
     __syncthreads();
-    if (duplicate) {                           // (uniform) left to the exact kernel
-        if (threadIdx.x == 0) redo_flags[t] = 1u;
+    if (duplicate) {
+        // (uniform) a label lists a column twice -- rewiring draws such labels all the time -- and the bitmap has one bit
+        // for the two connections: here the column's thread walks its bitmap row in ascending label order and scans each
+        // label found for the matching connections, which yields every connection, in ascending flat position
+        const unsigned mine = threadIdx.x;
+        const size_t sl = (size_t)t * nslices + (threadIdx.x >> 6);
+        const size_t row0 = slice_off[sl];
+        const unsigned rows = slice_off[sl + 1] - slice_off[sl];
+        const size_t at = row0 * 64 + (threadIdx.x & 63);
+        auto put = [&](size_t r, unsigned lab, unsigned pos) {
+            if (slot32 != nullptr) slot32[at + r * 64] = (pos << 17) | (lab << 7);
+            else { lab16[at + r * 64] = (unsigned short)lab; pos16[at + r * 64] = (unsigned short)pos; }
+        };
+        const unsigned first = parity_first(threadIdx.x);
+        // padding everywhere first; the thread's own slots are then overwritten (same thread: ordered)
+        for (unsigned r = 0; r < rows; ++r) put(r, (unsigned)zero_row + ((r & 1u) ^ first), pad_pos);
+        unsigned seen[2] = {0u, 0u};
+        const unsigned* my = bm + (size_t)mine * words;
+        for (int wd = 0; wd < words; ++wd) {
+            unsigned bits = my[wd];
+            while (bits) {
+                const unsigned b = (unsigned)__builtin_ctz(bits);
+                bits &= bits - 1u;
+                const unsigned l = 32u * (unsigned)wd + b;
+                const unsigned row = rows_of[l];
+                const unsigned par = row & 1u;
+                const unsigned short* lrow = ids + (size_t)l * K;
+                for (int k = 0; k < K; ++k) {
+                    if (lrow[k] == mine) {
+                        const unsigned t2 = par ? seen[1]++ : seen[0]++;
+                        put(2u * t2 + (par ^ first), row, l * (unsigned)K + (unsigned)k);
+                    }
+                }
+            }
+        }
         return;
     }
     // per column: labels in even / odd rows before each word; then the column's padding slots
@@ -643,21 +675,14 @@ int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
         int words = 0;
         const size_t fill_lds = tile_fill_bitmap_lds(threads, TL, p->K, &words);
         const unsigned pad_pos = w_in_lds ? (unsigned)TL * (unsigned)p->K : kPadPos;
-        unsigned* redo = nullptr;
-        if (fill_lds <= 160 * 1024 - 64 && dev_alloc(p, &redo, (size_t)tiles)) {
+        if (fill_lds <= 160 * 1024 - 64) {
             hipError_t ea = hipFuncSetAttribute((const void*)tile_fill_bitmap_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)fill_lds);
-            if (ea == hipSuccess) ea = hipMemsetAsync(redo, 0, (size_t)tiles * sizeof(unsigned), s);
             if (ea != hipSuccess) return hip_fail(ea);
             hipLaunchKernelGGL(tile_fill_bitmap_kernel, dim3(tiles), dim3(threads), fill_lds, s, lookup, p->rowpos, p->L, p->K, TL, 2 * cap,
-                               p->slice_off, p->lab16, p->pos16, pad_pos, p->slot32, words, redo);
-            // tiles in which a label lists a column twice (each exits at once otherwise)
-            hipLaunchKernelGGL(tile_fill_kernel, dim3(tiles), dim3(threads), 0, s, lookup, p->rowpos, p->L, p->K, TL, 2 * cap, p->slice_off,
-                               p->lab16, p->pos16, pad_pos, p->slot32, redo);
-            // (the flags are read by a kernel still in flight: back to the spare list only, not freed before the build's last wait)
-            dev_release(p, redo);
+                               p->slice_off, p->lab16, p->pos16, pad_pos, p->slot32, words);
         } else {
             hipLaunchKernelGGL(tile_fill_kernel, dim3(tiles), dim3(threads), 0, s, lookup, p->rowpos, p->L, p->K, TL, 2 * cap, p->slice_off,
-                               p->lab16, p->pos16, pad_pos, p->slot32, nullptr);
+                               p->lab16, p->pos16, pad_pos, p->slot32);
         }
     }
     e = hipGetLastError();

@@ -64,7 +64,8 @@ __global__ __launch_bounds__(kResThreads) void wgrad_resident_kernel(const float
                                                                      float* __restrict__ gw,
                                                                      float* __restrict__ bias_grad, int B, int N,
                                                                      int L, int K, int nchunks, int n1, int upb1,
-                                                                     int upb2) {
+                                                                     int upb2, const unsigned long long* __restrict__ only_if_outdated) {
+    if (only_if_outdated != nullptr && *only_if_outdated != 0) return;     // (enqueued as a fallback: the plan was current)
     extern __shared__ __align__(16) float xs[];
     const int lane = threadIdx.x & 63;
     const int blk = blockIdx.x;
@@ -588,7 +589,7 @@ bool three_units_cheaper(long long units, int N, int cus) {
 }
 
 int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float* gw, float* bias_grad, const Dims& d,
-                       hipStream_t s, const ffi_plan* plan) {
+                       hipStream_t s, const ffi_plan* plan, const unsigned long long* only_if_outdated) {
     // (32 rows of out_grad must be reachable through 32-bit byte offsets)
     if (tile_path_fits(d.N) && d.L < (1 << 25)) {
         const float* xT = x;
@@ -661,10 +662,10 @@ int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float
         const bool vec4 = (d.K % 4 == 0) && (((uintptr_t)gw | (uintptr_t)idx) % 16 == 0);
         if (vec4) {
             FFI_HIP_TRY(hipFuncSetAttribute((const void*)wgrad_resident_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-            hipLaunchKernelGGL(wgrad_resident_kernel<true>, dim3(blocks), dim3(kResThreads), lds, s, xT, idx, g, gw, bias_grad, d.B, d.N, d.L, d.K, nchunks, n1, upb, upb2);
+            hipLaunchKernelGGL(wgrad_resident_kernel<true>, dim3(blocks), dim3(kResThreads), lds, s, xT, idx, g, gw, bias_grad, d.B, d.N, d.L, d.K, nchunks, n1, upb, upb2, only_if_outdated);
         } else {
             FFI_HIP_TRY(hipFuncSetAttribute((const void*)wgrad_resident_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-            hipLaunchKernelGGL(wgrad_resident_kernel<false>, dim3(blocks), dim3(kResThreads), lds, s, xT, idx, g, gw, bias_grad, d.B, d.N, d.L, d.K, nchunks, n1, upb, upb2);
+            hipLaunchKernelGGL(wgrad_resident_kernel<false>, dim3(blocks), dim3(kResThreads), lds, s, xT, idx, g, gw, bias_grad, d.B, d.N, d.L, d.K, nchunks, n1, upb, upb2, only_if_outdated);
         }
         FFI_HIP_TRY(hipGetLastError());
         return FFI_OK;
