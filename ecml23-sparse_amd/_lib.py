@@ -27,6 +27,8 @@ SIGNATURES = {
     "ffi_plan_refresh": (_int, [_vp, _vp, _vp]),
     "ffi_plan_destroy": (_int, [_vp]),
     "ffi_plan_info": (_int, [_vp, ctypes.POINTER(_i64)]),
+    "ffi_host_forward_f32": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _i64, _i64]),
+    "ffi_host_backward_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _i64, _i64, _i64, _i64]),
     "ffi_input_grad_planned_f32": (_int, [_vp, _vp, _vp, _vp, _i64, _int, _vp]),
     "ffi_cache_clear": (_int, []),
     "ffi_cache_bytes": (ctypes.c_size_t, []),

@@ -31,6 +31,7 @@ SOURCES = [
     "ffi_optimizer.hip",
     "ffi_rewire.hip",
     "ffi_fallback.hip",
+    "host/ffi_host_kernels.cc",
 ]
 
 # gfx950 only.  Packed-fp32 VALU forms are switched off for all device code.
@@ -50,7 +51,7 @@ def hipcc() -> str:
 
 
 def _compile(src: str) -> str:
-    obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
+    obj = os.path.join(OBJ_DIR, os.path.splitext(os.path.basename(src))[0] + ".o")
     cmd = [hipcc(), *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:

@@ -6,12 +6,13 @@
 //
 // Built only when a TensorFlow installation is handed to CMake (see ../CMakeLists.txt: FFI_TF_INCLUDE_DIR,
 // FFI_TF_LIBRARY); this image has none, so the file is compiled by whoever integrates the library into a ROCm
-// TensorFlow.  The reference's CPU kernels (register.cpp:79-80,88-89,97-98,106-107) are its own functors
-// (forward.cpp, backward.cpp): list those two sources in FFI_TF_CPU_SOURCES to register them beside the GPU ones.
+// TensorFlow.  The eight DEVICE_CPU kernels of the same ops (register.cpp:79-80,88-89,97-98,106-107) are in
+// ffi_tf_cpu_ops.cc, part of the same CMake target: one `sparseops` library registers all sixteen.
+#define EIGEN_USE_GPU
 #include "tensorflow/core/framework/op.h"
 #include "tensorflow/core/framework/op_kernel.h"
 #include "tensorflow/core/framework/shape_inference.h"
-#include "tensorflow/core/platform/stream_executor.h"
+#include "third_party/eigen3/unsupported/Eigen/CXX11/Tensor"
 
 #include "ffi_hip.h"
 
@@ -53,10 +54,11 @@ template <bool Transposed>
     return ::tensorflow::OkStatus();
 }
 
-// TensorFlow's compute stream for this op, as the hipStream_t the C ABI takes (the reference enqueues on the same
-// stream: forward.cu:50-68, backward.cu:59-64)
+// TensorFlow's compute stream for this op, as the hipStream_t the C ABI takes: the stream of the op's Eigen GPU device,
+// which is what the reference launches on (forward.cu:50-68, backward.cu:59-64: device.stream()) and what every
+// TensorFlow 2.x has
 void* ComputeStream(OpKernelContext* ctx) {
-    return ctx->op_device_context()->stream()->platform_specific_handle().stream;
+    return static_cast<void*>(ctx->eigen_device<Eigen::GpuDevice>().stream());
 }
 
 struct LayerShape { int64_t batch, num_features, num_units, fan_in; };

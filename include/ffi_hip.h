@@ -416,6 +416,24 @@ int ffi_rewire_f32(int32_t* lookup, const float* weights, float* const* arrays, 
                    int64_t num_features, const float* threshold, uint64_t seed, int64_t* rewired_count,
                    ffi_stream_t stream);
 
+/*
+ * Host (CPU) implementation, for the DEVICE_CPU kernels an op library registers beside the GPU ones
+ * (tfsparse/cc/kernels/register.cpp:79-80,88-89,97-98,106-107; CPU functors forward.cpp:9-44, backward.cpp:8-73).
+ * All pointers are HOST pointers; nothing touches a GPU and nothing starts a thread: the caller splits the work
+ * over its own threads through the ranges -- ffi_host_forward_f32 writes result[:, unit_begin:unit_end);
+ * ffi_host_backward_f32 writes weight_grad rows [unit_begin, unit_end) (if weight_grad is given) and the
+ * feature_grad entries of batch rows [batch_begin, batch_end) (if feature_grad is given), as the reference splits
+ * its two halves (backward.cpp:26-35 by units, :58-72 by batch entries).  Ids outside [0, num_features) return
+ * FFI_ERR_BAD_LOOKUP.  These are not fallbacks of the GPU entry points, which never compute on the CPU.
+ */
+int ffi_host_forward_f32(const float* features, const int32_t* lookup, const float* weights, float* result,
+                         int64_t batch, int64_t num_features, int64_t num_units, int64_t fan_in, int transposed,
+                         int64_t unit_begin, int64_t unit_end);
+int ffi_host_backward_f32(const float* features, const int32_t* lookup, const float* weights, const float* out_grad,
+                          float* feature_grad, float* weight_grad, int64_t batch, int64_t num_features,
+                          int64_t num_units, int64_t fan_in, int transposed, int64_t unit_begin, int64_t unit_end,
+                          int64_t batch_begin, int64_t batch_end);
+
 #ifdef __cplusplus
 }
 #endif

@@ -104,8 +104,8 @@ def test_layer_constructor_arithmetic():
 def test_tensorflow_shim_declares_the_reference_ops():
     # The op library a maintainer builds against ROCm TensorFlow (csrc/tf/ffi_tf_ops.cc) must declare the four ops
     # exactly as tfsparse/cc/ops/fixed_fan_in_ops.cpp:55-93 does (names, attrs, inputs, outputs: the Python binding
-    # sparse/ops/fixed_fan_in_ops.py:9-40 is generated from them) and register the eight GPU kernels of
-    # tfsparse/cc/kernels/register.cpp:81-82,90-91,99-100,108-109.  TensorFlow is not in this image: the file is checked as text.
+    # sparse/ops/fixed_fan_in_ops.py:9-40 is generated from them) and register the sixteen kernels of
+    # tfsparse/cc/kernels/register.cpp:79-109 (eight GPU, eight CPU).  TensorFlow is not in this image: the files are checked as text.
     import os
     import re
 
@@ -127,14 +127,64 @@ def test_tensorflow_shim_declares_the_reference_ops():
                         ("GRAD", "FanInSparseMatmulGrad", "false"), ("GRAD", "FanInSparseMatmulGradTp", "true")]
     kernels = re.findall(r'FFI_REGISTER_GPU\("(\w+)", (\w+), (\w+), (true|false)\);', code)
     assert len(kernels) == 8
+    # ... and the eight CPU kernels of register.cpp:79-80,88-89,97-98,106-107, in the second source of the same target
+    cpu_src = open(os.path.join(ROOT, "ecml23-sparse_amd", "csrc", "tf", "ffi_tf_cpu_ops.cc")).read()
+    cpu_code = re.sub(r"//[^\n]*", "", cpu_src)
+    cpu_kernels = re.findall(r'FFI_REGISTER_CPU\("(\w+)", (\w+), (\w+), (true|false)\);', cpu_code)
+    assert len(cpu_kernels) == 8 and len(set(kernels)) + len(set(cpu_kernels)) == 16
     for op, transposed in (("FanInSparseMatmul", "false"), ("FanInSparseMatmulTp", "true"),
                            ("FanInSparseMatmulGrad", "false"), ("FanInSparseMatmulGradTp", "true")):
-        cls = "FanInSparseMatmulGradGpuOp" if "Grad" in op else "FanInSparseMatmulGpuOp"
         for ids in ("int32", "uint32"):
-            assert (op, cls, ids, transposed) in kernels
+            assert (op, "FanInSparseMatmulGradGpuOp" if "Grad" in op else "FanInSparseMatmulGpuOp", ids, transposed) in kernels
+            assert (op, "FanInSparseMatmulGradCpuOp" if "Grad" in op else "FanInSparseMatmulCpuOp", ids, transposed) in cpu_kernels
+    # the compute stream is taken as the reference takes it (forward.cu:50, backward.cu:63: the Eigen GPU device's stream,
+    # present in every TensorFlow 2.x), not through an accessor of recent releases only
+    assert "eigen_device<Eigen::GpuDevice>().stream()" in code
+    assert "platform_specific_handle" not in code and "op_device_context" not in code
+    # both sources are in the CMake target
+    cmake = open(os.path.join(ROOT, "ecml23-sparse_amd", "csrc", "CMakeLists.txt")).read()
+    assert re.search(r"add_library\(sparseops SHARED tf/ffi_tf_ops\.cc tf/ffi_tf_cpu_ops\.cc\)", cmake)
+    assert "host/ffi_host_kernels.cc" in cmake
     assert "DEVICE_GPU" in code and 'TypeConstraint<float>("T")' in code
     # no arithmetic in the shim: its Compute bodies end in exactly one C-ABI call each
     assert code.count("ffi_forward_f32(") == 1 and code.count("ffi_backward_f32(") == 1
     # and the default CMake build does not depend on TensorFlow
     cm = open(os.path.join(ROOT, "ecml23-sparse_amd", "csrc", "CMakeLists.txt")).read()
     assert "if(FFI_TF_INCLUDE_DIR AND FFI_TF_LIBRARY)" in cm and "tf/ffi_tf_ops.cc" in cm
+
+
+def test_host_kernels_match_the_oracle():
+    # the product's own CPU implementation behind the DEVICE_CPU kernels (csrc/host/ffi_host_kernels.cc, host pointers,
+    # no GPU): the reference's shape grid (testing/test.cpp:50-59), both layouts, work split into ranges the way an op's
+    # thread pool would split it; gates as for the GPU kernels (1e-5 forward, 1e-4 gradients)
+    import ctypes
+
+    import numpy as np
+
+    import oracle
+    from conftest import REFERENCE_SHAPES, load_package, reference_law_inputs, rel_err
+    lib = load_package()._lib.lib()
+    ptr = lambda a: a.ctypes.data_as(ctypes.c_void_p)  # noqa: E731
+    for (B, N, L, K) in [s for s in REFERENCE_SHAPES if s[2] <= 20000] + [(5, 7, 11, 3)]:
+        x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=L + K)
+        for tp in (0, 1):
+            xin = np.ascontiguousarray(x.T) if tp else x
+            out = np.full((B, L), np.nan, dtype=np.float32)
+            gx = np.full(xin.shape, np.nan, dtype=np.float32)
+            gw = np.full((L, K), np.nan, dtype=np.float32)
+            cuts = [0, L // 3, L]
+            for a, b in zip(cuts[:-1], cuts[1:]):
+                assert lib.ffi_host_forward_f32(ptr(xin), ptr(lookup), ptr(w), ptr(out), B, N, L, K, tp, a, b) == 0
+                assert lib.ffi_host_backward_f32(ptr(xin), ptr(lookup), ptr(w), ptr(g), None, ptr(gw), B, N, L, K, tp, a, b, 0, 0) == 0
+            bcuts = [0, B // 2, B]
+            for a, b in zip(bcuts[:-1], bcuts[1:]):
+                assert lib.ffi_host_backward_f32(ptr(xin), ptr(lookup), ptr(w), ptr(g), ptr(gx), None, B, N, L, K, tp, 0, 0, a, b) == 0
+            assert rel_err(out, oracle.forward(xin, lookup, w, transposed=bool(tp))) <= 1e-5
+            o_gx, o_gw = oracle.backward(xin, lookup, w, g, transposed=bool(tp))
+            assert rel_err(gw, o_gw) <= 1e-4 and rel_err(gx, o_gx) <= 1e-4
+    # argument checks
+    one = ctypes.c_void_p(16)
+    assert lib.ffi_host_forward_f32(None, one, one, one, 1, 1, 1, 1, 0, 0, 1) == -1
+    assert lib.ffi_host_forward_f32(one, one, one, one, 1, 1, 1, 1, 0, 0, 2) == -8
+    bad = np.array([[3]], dtype=np.int32); f1 = np.ones((1, 1), dtype=np.float32)
+    assert lib.ffi_host_forward_f32(ptr(f1), ptr(bad), ptr(f1), ptr(f1.copy()), 1, 1, 1, 1, 0, 0, 1) == -6
