@@ -182,9 +182,10 @@ def parse_args():
                     help="milliseconds of untimed steps in front of the warm-up: the GPU's clocks settle under load within tens of "
                          "milliseconds, and a 20-step run (14 ms) would otherwise be timed on the ramp")
     ap.add_argument("--no-rewire-costs", action="store_true", help="skip the plan-build / first-backward-after-rewiring timings")
-    ap.add_argument("--sweep", action="store_true",
-                    help="instead of the benchmark line: batch x width x labels x fan-in grid of the three passes, one CSV line each "
-                         "(gpurun_out/sweep.csv), in the manner of the reference's testing/detailed-bench.cpp:26-112")
+    ap.add_argument("--sweep", nargs="?", const="all", default=None, choices=["all", "reference", "layer", "layer_k64"],
+                    help="instead of the benchmark line: batch x width x labels x fan-in grids of the passes, one CSV line per "
+                         "timing (gpurun_out/sweep.csv): 'reference' = the grid of the reference's testing/detailed-bench.cpp:26-112, "
+                         "'layer' = the same axes around the headline workload, each pass also with the library's kernel choices overridden")
     ap.add_argument("--copy-bytes", type=int, default=0,
                     help="also run one plain device copy kernel of this many bytes (read N, write N): the "
                          "known-size reference that rocprofv3 FETCH_SIZE/WRITE_SIZE readings are scaled by")
@@ -420,9 +421,148 @@ def train_step(pkg, cfg, x, lookup, w, tp, density, stream, iters):
         check(lib.ffi_rewire_f32(ptr(lookup2), ptr(w), arrays, 2, L * K, N, ptr(thr), 12345, None, sh))
 
     out["rewire_1pct_ms"] = round(time_kernel(rewire, stream, iters), 4)
+    # the same step through the PyTorch binding: the fused loss as an autograd function, loss.backward() (the
+    # upstream factor arrives as a device scalar), gradients left in .grad; no optimizer
+    x_a, w_a, b_a = x.clone().requires_grad_(True), w.clone().requires_grad_(True), bias.clone().requires_grad_(True)
+    loss_fn, y_true = pkg.SparseSquaredHingeLoss(), (labels, None)
+
+    def autograd_step():
+        x_a.grad = w_a.grad = b_a.grad = None
+        loss_fn.fused(x_a, lookup, w_a, b_a, y_true, transposed=tp)[0].backward()
+
+    out["autograd_forward_loss_backward_ms"] = round(time_kernel(autograd_step, stream, iters), 4)
+
+    def c_abi_step():
+        fused_forward_loss()
+        check(lib.ffi_backward_sparse_f32(ptr(x), ptr(lookup), ptr(w), ptr(g), ptr(masks), 1 | 2, ctypes.c_float(0.0), ptr(gx), ptr(gw),
+                                          ptr(gb), ctypes.byref(taken), B, N, L, K, int(tp), sh))
+
+    out["c_abi_forward_loss_backward_ms"] = round(time_kernel(c_abi_step, stream, iters), 4)
     out["unfused_dense_route_ms"] = {"forward_bias+loss_grad": round(time_kernel(unfused_forward_loss, stream, iters), 4),
                                      "backward_dense": round(time_kernel(backward_dense, stream, iters), 4)}
     return out
+
+
+# Points of --sweep.  "reference": the grid of the reference's testing/detailed-bench.cpp:26-112 (forward pass, both
+# feature layouts, one axis varied around batch 32 / 32,768 inputs / 670,000 labels / fan-in 32).  "layer": the same
+# four axes around the headline workload, whose narrow input takes the LDS-tile kernels: all three passes, and each
+# pass also with the library's choices overridden (ffi_set_option), which is what re-checks those choices.
+SWEEP_GRIDS = {
+    "reference": {"base": (32, 32768, 670000, 32), "passes": ("forward",), "layouts": ("bn", "nb"), "distinct": False,
+                  "axes": {"batch": [4, 8, 10, 16, 25, 32, 50, 64, 100],
+                           "num_features": [768, 1024, 2048, 4096, 8192, 16384, 24576, 32768, 49152, 65536],
+                           "num_units": [4000, 10000, 32000, 64000, 100000, 256000, 670000, 1000000],
+                           "fan_in": [4, 8, 12, 16, 24, 32, 40, 48, 64, 80, 96, 128]}},
+    "layer": {"base": (128, 768, 670091, 32), "passes": ("forward", "weight_grad", "input_grad"), "layouts": ("nb",), "distinct": True,
+              "axes": {"batch": [32, 64, 96, 128, 160, 256, 512],
+                       "num_features": [64, 128, 256, 384, 512, 608, 640, 768, 1024, 1216],
+                       "num_units": [4000, 32000, 131072, 262144, 393216, 524288, 670091, 1000000, 3000000],
+                       "fan_in": [8, 16, 32, 64, 96, 128]}},
+}
+# (the second narrow workload of the benchmark set: 64 connections per label = two chunks per label, 512 columns)
+SWEEP_GRIDS["layer_k64"] = dict(SWEEP_GRIDS["layer"], base=(256, 512, 501070, 64),
+                                axes={"batch": [64, 128, 256, 512], "num_features": [256, 512, 608, 768],
+                                      "num_units": [131072, 501070, 1000000], "fan_in": [48, 64, 128]})
+SWEEP_VARIANTS = {
+    "forward": [("fwd_lane64", -1)],
+    "weight_grad": [("wgrad_units", 3), ("wgrad_units", 4), ("wgrad_stream", -1)],
+    "input_grad": [("plan_weights_in_lds", -1), ("plan_weights_in_lds", 1), ("workgroups_per_cu", 1)],
+}
+
+
+def sweep(args, pkg, synth):
+    """Times the passes over SWEEP_GRIDS and writes one CSV line per (point, layout, pass, variant) to
+    gpurun_out/sweep.csv; prints one JSON line that lists where an override beat the library's own choice."""
+    import csv
+    import ctypes
+
+    import torch
+    lib, check = pkg._lib.lib(), pkg._lib.check
+    stream = torch.cuda.current_stream()
+    sh = stream.cuda_stream
+    ptr = lambda a: a.data_ptr()  # noqa: E731
+    os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
+    path = os.path.join(ROOT, "gpurun_out", "sweep.csv")
+    rows, beaten, points = [], [], 0
+    names = ("batch", "num_features", "num_units", "fan_in")
+    grids = [g for g in SWEEP_GRIDS if args.sweep in ("all", g)]
+    for grid in grids:
+        spec = SWEEP_GRIDS[grid]
+        seen = set()
+        for axis, values in spec["axes"].items():
+            for v in values:
+                dims = list(spec["base"])
+                dims[names.index(axis)] = v
+                B, N, L, K = dims
+                if (B, N, L, K) in seen and axis != "batch":
+                    continue                      # the base point is on every axis: timed once
+                seen.add((B, N, L, K))
+                points += 1
+                gen = torch.Generator(device="cuda").manual_seed(args.seed)
+                lookup = synth.make_lookup(L, K, N, distinct=spec["distinct"], generator=gen, device="cuda")
+                w = torch.randn((L, K), generator=gen, device="cuda") * K ** -0.5
+                g = torch.randn((B, L), generator=gen, device="cuda") * 0.1
+                out, gw = torch.empty_like(g), torch.empty_like(w)
+                for layout in spec["layouts"]:
+                    tp = layout == "nb"
+                    x = torch.relu(torch.randn((N, B) if tp else (B, N), generator=gen, device="cuda"))
+                    gx = torch.empty_like(x)
+                    plan = ctypes.c_void_p()
+                    iters = max(3, min(30, int(2.0e10 / (B * L * K))))
+
+                    def settled(fn):
+                        # 25 ms of the same kernel in front of the timed launches: the clocks follow the load
+                        t0 = time.perf_counter()
+                        while time.perf_counter() - t0 < 0.025:
+                            for _ in range(iters):
+                                fn()
+                            torch.cuda.synchronize()
+                        return time_kernel(fn, stream, iters)
+
+                    def timed(name):
+                        # the gradient passes through an explicit plan (built under the options in force), created here
+                        # and destroyed after the timing
+                        if name == "forward":
+                            return settled(lambda: check(lib.ffi_forward_f32(ptr(x), ptr(lookup), ptr(w), ptr(out), B, N, L, K, int(tp), sh)))
+                        check(lib.ffi_plan_create(ptr(lookup), L, K, N, B, sh, ctypes.byref(plan)))
+                        if name == "weight_grad":
+                            ms = settled(lambda: check(lib.ffi_weight_grad_planned_f32(plan, ptr(x), ptr(lookup), ptr(g), ptr(gw), B, int(tp), sh)))
+                        else:
+                            ms = settled(lambda: check(lib.ffi_input_grad_planned_f32(plan, ptr(w), ptr(g), ptr(gx), B, int(tp), sh)))
+                        check(lib.ffi_plan_destroy(plan))
+                        return ms
+
+                    for name in spec["passes"]:
+                        narrow = grid != "reference"
+                        variants = [("auto", 0)] + (SWEEP_VARIANTS[name] if narrow else [])
+                        # two rounds over the variants, the smaller time of each: the clocks drift by several percent
+                        # with the load of the preceding milliseconds, in both directions
+                        results = {}
+                        for _ in range(2 if narrow else 1):
+                            for option, value in variants:
+                                if value:
+                                    check(lib.ffi_set_option(option.encode(), value))
+                                ms = timed(name)
+                                if value:
+                                    check(lib.ffi_set_option(option.encode(), 0))
+                                label = option if not value else f"{option}={value}"
+                                results[label] = min(ms, results.get(label, ms))
+                        for label, ms in results.items():
+                            rows.append([grid, axis, B, N, L, K, layout, name, label, f"{ms:.5f}"])
+                            if label != "auto" and ms < 0.97 * results["auto"]:
+                                beaten.append({"point": [B, N, L, K], "pass": name, "override": label,
+                                               "auto_ms": round(results["auto"], 4), "override_ms": round(ms, 4)})
+                    del x, gx
+                del lookup, w, g, out, gw
+                check(lib.ffi_cache_clear())
+                torch.cuda.empty_cache()
+                print(f"sweep: {grid} {axis}={v} done", file=sys.stderr, flush=True)
+    with open(path, "w", newline="") as f:
+        wr = csv.writer(f)
+        wr.writerow(["grid", "axis", "batch", "num_features", "num_units", "fan_in", "layout", "pass", "variant", "ms"])
+        wr.writerows(rows)
+    print(json.dumps({"sweep": grids, "points": points, "timings": len(rows), "csv": os.path.relpath(path, ROOT),
+                      "overrides_faster_than_the_library_by_3_percent": beaten}))
 
 
 def main():
@@ -451,6 +591,9 @@ def main():
         torch.mul(src, 1.0, out=dst)
         torch.cuda.synchronize()
         del src, dst
+    if args.sweep:
+        sweep(args, pkg, synth)
+        return
     cfg = synth.CONFIGS[args.config]
     if cfg.name == "c5":
         print(json.dumps(bench_inference(args, pkg, synth, cfg)))

@@ -6,11 +6,14 @@
 #include <algorithm>
 #include <climits>
 #include <cmath>
+#include <cstring>
 #include <mutex>
 #include <new>
 #include <vector>
 
 namespace ffi {
+
+Options g_options;
 
 static thread_local int g_last_hip_error = 0;
 
@@ -597,6 +600,28 @@ int ffi_cache_clear(void) {
     workspace_clear(dev);
     nonzero_count_forget(dev);
     return FFI_OK;
+}
+
+int ffi_set_option(const char* name, int value) {
+    if (name == nullptr) return FFI_ERR_BAD_ARGUMENT;
+    static const struct { const char* name; int ffi::Options::*field; int lo, hi; } table[] = {
+        {"wgrad_units", &ffi::Options::wgrad_units, 0, 4},
+        {"wgrad_stream", &ffi::Options::wgrad_stream, -1, 0},
+        {"fwd_lane64", &ffi::Options::fwd_lane64, -1, 0},
+        {"plan_weights_in_lds", &ffi::Options::plan_weights_in_lds, -1, 1},
+        {"workgroups_per_cu", &ffi::Options::workgroups_per_cu, 0, 16},
+    };
+    for (const auto& t : table) {
+        if (std::strcmp(name, t.name) != 0) continue;
+        if (value < t.lo || value > t.hi || (t.field == &ffi::Options::wgrad_units && value != 0 && value != 3 && value != 4))
+            return FFI_ERR_BAD_ARGUMENT;
+        // cached plans were laid out under the old choice
+        const int status = ffi_cache_clear();
+        if (status != FFI_OK && status != FFI_ERR_NO_DEVICE) return status;
+        ffi::g_options.*(t.field) = value;
+        return FFI_OK;
+    }
+    return FFI_ERR_BAD_ARGUMENT;
 }
 
 size_t ffi_cache_bytes(void) {

@@ -108,7 +108,10 @@ __device__ __forceinline__ void loss_epilogue(float (&acc)[32], bool all_rows, u
     mask = m;
 }
 
-template <bool VEC4, int EPI, bool TOPK>
+// VEC: how a label's column ids and weights are loaded.  0: one by one (any fan-in, any alignment); 1: by 16-byte quads
+// (fan-in a multiple of four, 16-byte aligned arrays), a partly filled last chunk one by one; 2: by quads, for a fan-in
+// below one chunk of 32 (a build of its own: the same code inside the general loop costs the full chunks 25 %).
+template <int VEC, int EPI, bool TOPK>
 __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* __restrict__ xT,
                                                                   const int32_t* __restrict__ idx,
                                                                   const float* __restrict__ w,
@@ -142,6 +145,8 @@ __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* _
     if (EPI == kEpiLossGradAndScores) grsrc = make_rsrc(fl.gout + (size_t)b0 * (size_t)L, (size_t)nrows * (size_t)L * sizeof(float));
     float lsum = 0.f;
 
+    constexpr bool VEC4 = VEC >= 1;
+    constexpr bool SHORT = VEC == 2;
     constexpr bool SKEW = EPI == kEpiLossGradSkewed;
     constexpr bool LOSS = EPI == kEpiLossGrad || EPI == kEpiLossGradAndScores || SKEW;
     static_assert(!(SKEW && TOPK), "the top-k tests need the natural order");
@@ -161,10 +166,23 @@ __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* _
         for (int i = 0; i < 32; ++i) acc[i] = 0.f;
         for (int ch = 0; ch < nchunks; ++ch) {
             const int k0 = ch * 32;
-            const bool full = VEC4 && k0 + 32 <= K;
+            const bool full = VEC4 && !SHORT && k0 + 32 <= K;
             unsigned idp[16];
             float wv[32];
-            if (full) {
+            if (SHORT) {
+                // the one, partly filled chunk: the quads behind its end re-read its first quad, so that the loads stay
+                // unconditional; their connections are skipped below
+                const int quads = K >> 2;
+#pragma unroll
+                for (int q = 0; q < 8; ++q) {
+                    const int at = 4 * (q < quads ? q : 0);
+                    const int4 v = *reinterpret_cast<const int4*>(irow + at);
+                    idp[2 * q + 0] = (unsigned)v.x | ((unsigned)v.y << 16);
+                    idp[2 * q + 1] = (unsigned)v.z | ((unsigned)v.w << 16);
+                    const float4 f = *reinterpret_cast<const float4*>(wrow + at);
+                    wv[4 * q] = f.x; wv[4 * q + 1] = f.y; wv[4 * q + 2] = f.z; wv[4 * q + 3] = f.w;
+                }
+            } else if (full) {
 #pragma unroll
                 for (int q = 0; q < 8; ++q) {
                     const int4 v = *reinterpret_cast<const int4*>(irow + k0 + 4 * q);
@@ -479,7 +497,14 @@ int launch_lane64(const float* xT, const int32_t* idx, const float* w, const flo
 }
 
 // (64 rows of out of a batch tile are reached through 32-bit byte offsets)
-bool lane64_fits(const Dims& d) { return d.N <= kLane64MaxN && d.B > kTileBatch && d.L < (1 << 24); }
+// Where the tile of 64 samples fits, and where it pays.  Measured against the 32-sample kernel at 501,070 labels, 256-608
+// columns: +2...+10 % from 192 samples up at every fan-in, -3...-14 % at 64-160 samples with a fan-in up to 40; +5...+12 %
+// from 128 samples up with a fan-in of 64 or more; +20...+37 % at fan-in 48 at every batch size (a last chunk of 16
+// connections is a full chunk here, and loaded one by one there).
+bool lane64_fits(const Dims& d) {
+    if (d.N > kLane64MaxN || d.B <= kTileBatch || d.L >= (1 << 24) || g_options.fwd_lane64 < 0) return false;
+    return d.B >= 192 || (d.K >= 64 && d.B >= 128) || (d.K > 32 && d.K % 32 != 0 && d.K % 16 == 0);
+}
 
 }  // namespace
 
@@ -511,11 +536,11 @@ __global__ __launch_bounds__(256) void fwd_sample_kernel(const float* __restrict
     }
 }
 
-template <bool VEC4, int EPI, bool TOPK>
+template <int VEC, int EPI, bool TOPK>
 int launch_lane32(const float* xT, const int32_t* idx, const float* w, const float* bias, float* out, const Dims& d, int nbt,
                   int per_stream, int blocks, size_t lds, const FwdLoss& fl, const FwdTopk& ft, hipStream_t s) {
-    FFI_HIP_TRY(hipFuncSetAttribute((const void*)fwd_lane32_kernel<VEC4, EPI, TOPK>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL((fwd_lane32_kernel<VEC4, EPI, TOPK>), dim3(blocks), dim3(kTileThreads), lds, s, xT, idx, w, bias, out, d.B, d.N,
+    FFI_HIP_TRY(hipFuncSetAttribute((const void*)fwd_lane32_kernel<VEC, EPI, TOPK>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL((fwd_lane32_kernel<VEC, EPI, TOPK>), dim3(blocks), dim3(kTileThreads), lds, s, xT, idx, w, bias, out, d.B, d.N,
                        d.L, d.K, nbt, per_stream, fl, ft);
     FFI_HIP_TRY(hipGetLastError());
     return FFI_OK;
@@ -525,14 +550,16 @@ template <int EPI>
 int launch_lane32_any(bool vec4, bool topk, const float* xT, const int32_t* idx, const float* w, const float* bias, float* out,
                       const Dims& d, int nbt, int per_stream, int blocks, size_t lds, const FwdLoss& fl, const FwdTopk& ft,
                       hipStream_t s) {
+    // (see fwd_lane32_kernel: 2 = quads, fan-in below one chunk)
+    const int vec = !vec4 ? 0 : d.K < 32 ? 2 : 1;
+#define FFI_LANE32(VEC, E, T) launch_lane32<VEC, E, T>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, ft, s)
     if constexpr (EPI != kEpiLossGradSkewed) {              // (that epilogue has no top-k form)
-        if (topk)
-            return vec4 ? launch_lane32<true, EPI, true>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, ft, s)
-                        : launch_lane32<false, EPI, true>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, ft, s);
+        if (topk) return vec == 2 ? FFI_LANE32(2, EPI, true) : vec == 1 ? FFI_LANE32(1, EPI, true) : FFI_LANE32(0, EPI, true);
     }
     if (EPI == kEpiNone) return FFI_OK;                     // nothing to compute
-    return vec4 ? launch_lane32<true, EPI == kEpiNone ? kEpiScores : EPI, false>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, ft, s)
-                : launch_lane32<false, EPI == kEpiNone ? kEpiScores : EPI, false>(xT, idx, w, bias, out, d, nbt, per_stream, blocks, lds, fl, ft, s);
+    constexpr int E = EPI == kEpiNone ? kEpiScores : EPI;
+    return vec == 2 ? FFI_LANE32(2, E, false) : vec == 1 ? FFI_LANE32(1, E, false) : FFI_LANE32(0, E, false);
+#undef FFI_LANE32
 }
 
 // Narrow-input forward pass with the given epilogue; `la` is needed for the loss epilogues only, `tk` (may be

@@ -22,6 +22,17 @@ struct Dims {
     bool tp; // features / feature_grad are [N,B]
 };
 
+// Overrides of the launchers' choices, set through ffi_set_option (benchmark sweeps re-check each choice against its
+// alternative with them); all zero = the library decides.
+struct Options {
+    int wgrad_units = 0;            // 3 or 4 units per thread of the arranged weight-gradient kernels
+    int wgrad_stream = 0;           // -1: never the streaming weight-gradient kernel
+    int fwd_lane64 = 0;             // -1: never the 64-sample forward kernel
+    int plan_weights_in_lds = 0;    // -1: never / 1: whenever the tile fits
+    int workgroups_per_cu = 0;      // upper limit for the kernel that walks a tiled plan
+};
+extern Options g_options;
+
 // Records a failing HIP call for ffi_last_hip_error() and maps it to FFI_ERR_HIP.
 int hip_fail(hipError_t e);
 
@@ -281,7 +292,8 @@ inline int tiled_workgroups_per_cu(int threads, int tile_labels, int K, bool wit
     const size_t lds = tiled_lds_bytes(tile_labels, K, with_weights);
     const int by_lds = (int)((size_t)160 * 1024 / (lds > 0 ? lds : 1));
     const int by_waves = (with_weights ? 768 : 1024) / (threads > 0 ? threads : 1);
-    const int n = by_lds < by_waves ? by_lds : by_waves;
+    int n = by_lds < by_waves ? by_lds : by_waves;
+    if (g_options.workgroups_per_cu > 0 && n > g_options.workgroups_per_cu) n = g_options.workgroups_per_cu;
     return n < 1 ? 1 : n;
 }
 constexpr int kArrIdBits = 11;            // column-id field of an arranged entry (narrow inputs: ids < 1216)

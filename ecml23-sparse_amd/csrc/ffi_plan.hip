@@ -601,16 +601,18 @@ int plan_tile_labels(int N, int K, int L, int batch_hint, bool* weights_in_lds) 
     // tiles and workgroups per CU that suit each form (tiled_workgroups_per_cu): with up to four batch tiles the form is
     // 5-60 % faster (most where the fan-in exceeds 32 or the layer has at most 256 columns); with five to eight batch
     // tiles the tile's weights are staged that many times per tile: at fan-in 32 and below still -5...-30 % with at
-    // most 256 columns (several workgroups per CU overlap the staging) and -1...-8 % with 512 or 768, but +1 % at fan-in
+    // most 256 columns (several workgroups per CU overlap the staging) and -1...-8 % with 512 or 768; with 576 to 768
+    // columns -5...-13 % at every fan-in from 40 to 128 (one workgroup per CU either way); but +12 % at fan-in
     // 64 / 512 columns against the two-workgroup slot-ordered form, which also wins at 320-448 columns; with sixteen
-    // batch tiles -7...+4 %: not taken.
+    // batch tiles -7...+6 %: not taken.
     // The tile: as many labels as fit the LDS with their weights, one label per thread to stage; a thread carries
     // 8 x 16 bytes of the tile's weights in registers across the barrier, what exceeds that is copied behind it.
     // A slot's position inside the tile's weights has 15 bits (the zero word that padding slots read included).
     bool w_in_lds = false;
     const int nbt_hint = (batch_hint + 31) / 32;
-    const bool wanted = batch_hint > 0 &&
-                        (nbt_hint <= 4 || (nbt_hint <= 8 && K <= 32 && (threads >= 512 || threads <= 256)));   // (unknown batch size: the form for large batches)
+    const bool wanted = batch_hint > 0 && g_options.plan_weights_in_lds >= 0 &&
+                        (g_options.plan_weights_in_lds > 0 || nbt_hint <= 4 ||
+                         (nbt_hint <= 8 && (threads > 512 || (K <= 32 && (threads == 512 || threads <= 256)))));   // (unknown batch size: the form for large batches)
     if (wanted && threads <= 768) {
         int tw = std::min(TL, threads & ~1);
         // (workgroups of at most 256 threads share a CU when there are batch tiles to overlap: tiled_workgroups_per_cu)

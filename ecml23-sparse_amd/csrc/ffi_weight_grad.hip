@@ -622,7 +622,7 @@ int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float
             // (and rows of out_grad of at least 256 bytes: the LDS-direct loads take their destination's offset inside the
             // slice back out of the scalar offset of the row, which must not become negative)
             const bool stream = tile_lds_bytes(d.N) + (size_t)(kResThreads / 64) * kSliceFloats * sizeof(float) <= kLdsPerWorkgroup &&
-                                d.L >= 64;
+                                d.L >= 64 && g_options.wgrad_stream >= 0;
             const size_t lds = std::max(tile_lds_bytes(d.N) + (stream ? (size_t)(kResThreads / 64) * kSliceFloats * sizeof(float) : 0),
                                         (size_t)kResThreads * kSlotPitch * sizeof(float));
             // a label of two or four chunks: all its units in one thread (its out_grad values are loaded once per
@@ -649,7 +649,10 @@ int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float
             } while (0)
             if (nchunks == 2) FFI_LAUNCH_ARRANGED(2, 4);
             else if (nchunks == 4) FFI_LAUNCH_ARRANGED(4, 4);
-            else if (three_units_cheaper((long long)d.L * nchunks, d.N, cus)) FFI_LAUNCH_ARRANGED(1, 3);
+            // the streaming kernel: three units per thread wherever measured (4,000 to 3,000,000 labels, batch 32-512, 64-768
+            // columns, fan-in 8-32 and 96: 3-15 % under four units); the kernel without slices: by the model above
+            else if (g_options.wgrad_units == 3 ||
+                     (g_options.wgrad_units != 4 && (stream || three_units_cheaper((long long)d.L * nchunks, d.N, cus)))) FFI_LAUNCH_ARRANGED(1, 3);
             else FFI_LAUNCH_ARRANGED(1, 4);
 #undef FFI_LAUNCH_ARRANGED
             FFI_HIP_TRY(hipGetLastError());

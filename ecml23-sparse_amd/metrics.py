@@ -106,14 +106,18 @@ def forward_loss(features, lookup, weights, bias, y_true, kind, grad_scale=None,
     return result + (top,) if topk else result
 
 
-def _scaled(out_grad, upstream):
-    # multiplied on the device, whatever the factor: reading it on the host would make every training step wait
-    # for the GPU (a host-side scalar equal to 1 is the one case that can be skipped without looking at the device)
+def _upstream_is_one(upstream):
+    """True where the factor autograd hands to ``backward`` is known ON THE HOST to be 1: reading a device scalar
+    here would make every training step wait for the GPU."""
     if not isinstance(upstream, torch.Tensor):
-        return out_grad if float(upstream) == 1.0 else out_grad * upstream
-    if upstream.device.type == "cpu" and upstream.numel() == 1 and float(upstream) == 1.0:
-        return out_grad
-    return out_grad * upstream
+        return float(upstream) == 1.0
+    return upstream.device.type == "cpu" and upstream.numel() == 1 and float(upstream) == 1.0
+
+
+def _scaled(out_grad, upstream):
+    # multiplied on the device, whatever the factor (a host-side scalar equal to 1 is the one case that can be
+    # skipped without looking at the device); out of place, since a retained graph may run backward again
+    return out_grad if _upstream_is_one(upstream) else out_grad * upstream
 
 
 class _SparseLossFn(torch.autograd.Function):
@@ -150,13 +154,22 @@ class _LayerLossFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad, _grad_scores):
         features, lookup, weights, out_grad, masks = ctx.saved_tensors
-        g = _scaled(out_grad, grad)
+        # The upstream factor never touches the [B,L] gradient matrix (mostly unwritten entries, hundreds of MB):
+        # all three results are linear in it, so the factor goes on the small operands instead.  The weight
+        # gradient is linear in the features ([B,N]); the feature and bias gradients are scaled as results.
+        one = _upstream_is_one(grad)
         # the masks say where the gradient is not zero: the backward pass skips the rest when they are few
-        feature_grad, weight_grad, bias_grad, _ = backward_sparse(features, lookup, weights, g, nz_words=masks,
+        feature_grad, weight_grad, bias_grad, _ = backward_sparse(features if one else features * grad, lookup, weights,
+                                                                  out_grad, nz_words=masks,
                                                                   transposed=ctx.transposed,
                                                                   need_feature_grad=ctx.needs_input_grad[0],
                                                                   need_bias_grad=ctx.has_bias, grad_is_partial=True,
                                                                   decide_from_previous=True)
+        if not one:
+            if feature_grad is not None:
+                feature_grad.mul_(grad)
+            if bias_grad is not None:
+                bias_grad.mul_(grad)
         return feature_grad, None, weight_grad, bias_grad, None, None, None, None, None
 
 

@@ -182,6 +182,19 @@ int ffi_weight_grad_planned_f32(const ffi_plan* plan, const float* features, con
 int ffi_arrange_connections_f32(int32_t* lookup, float* const* arrays, int n_arrays,
                                 int64_t num_units, int64_t fan_in, ffi_stream_t stream);
 
+/*
+ * Overrides one of the library's kernel choices, process-wide (for benchmark sweeps that re-check a choice against its
+ * alternative; no counterpart in the reference).  0 always means "the library decides".
+ *   "wgrad_units"          3 or 4: units per thread of the weight-gradient kernels that read arranged column ids
+ *   "wgrad_stream"         -1: never the weight-gradient kernel that streams out_grad through LDS
+ *   "fwd_lane64"           -1: never the forward kernel that holds 64 samples per workgroup
+ *   "plan_weights_in_lds"  -1: never / 1: whenever it fits: the input-gradient form that keeps a tile's weights in LDS
+ *   "workgroups_per_cu"    n > 0: at most n workgroups per CU for the kernel that walks a tiled plan
+ * Drops the cached plans and workspaces of the current device first (as ffi_cache_clear, with its rule about calls in
+ * flight).  Unknown names and values outside the ranges above return FFI_ERR_BAD_ARGUMENT and change nothing.
+ */
+int ffi_set_option(const char* name, int value);
+
 /* Drops every cached plan and workspace of the calling thread's current device.  Waits for the device first; no other
    call of this library may be in flight on that device (from another thread) while it runs. */
 int ffi_cache_clear(void);

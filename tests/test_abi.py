@@ -60,3 +60,17 @@ def test_argument_checks_run_before_any_device_work():
     assert lib.ffi_plan_destroy(None) == 0
     with pytest.raises(pkg._lib.FfiError):
         pkg._lib.check(-2)
+
+
+def test_option_names_and_ranges_are_checked():
+    # without a GPU there is nothing cached to drop: the setter still validates and stores
+    pkg = load_package()
+    lib = pkg._lib.lib()
+    assert lib.ffi_set_option(None, 0) == -8
+    assert lib.ffi_set_option(b"no_such_option", 0) == -8
+    assert lib.ffi_set_option(b"wgrad_units", 5) == -8 and lib.ffi_set_option(b"wgrad_units", 2) == -8
+    assert lib.ffi_set_option(b"fwd_lane64", 1) == -8
+    for name, value in ((b"wgrad_units", 3), (b"wgrad_stream", -1), (b"fwd_lane64", -1), (b"plan_weights_in_lds", 1),
+                        (b"workgroups_per_cu", 2)):
+        assert lib.ffi_set_option(name, value) == 0
+        assert lib.ffi_set_option(name, 0) == 0

@@ -206,6 +206,37 @@ def test_fused_loss_trains_like_the_unfused_ops(ffi):
     assert abs(l0 - losses.mean(axis=-1).mean()) <= 1e-5 * losses.mean()
 
 
+@pytest.mark.parametrize("fused", [False, True])
+def test_upstream_factor_scales_every_gradient(ffi, fused):
+    # (factor * loss).backward(): autograd hands the factor to the loss op as a device scalar; all gradients
+    # carry it, checked against the oracle's backward pass of the oracle's loss gradient
+    B, N, L, K, factor = 48, 200, 2500, 12, 3.5
+    g = torch.Generator(device="cuda").manual_seed(9)
+    x = torch.rand((B, N), device="cuda", generator=g)
+    lookup = torch.randint(0, N, (L, K), device="cuda", generator=g, dtype=torch.int64).to(torch.int32)
+    rng = np.random.default_rng(4)
+    indices, _ = label_list(rng, B, L, values=False)
+    y = (torch.from_numpy(indices).cuda(), None)
+    w = ((torch.arange(L * K, device="cuda", dtype=torch.float32).reshape(L, K) % 11) / 11 - 0.5).requires_grad_(True)
+    bias = torch.full((L,), -0.2, device="cuda", requires_grad=True)
+    xin = x.clone().requires_grad_(True)
+    loss_fn = ffi.SparseSquaredHingeLoss()
+    if fused:
+        loss, _ = loss_fn.fused(xin, lookup, w, bias, y)
+    else:
+        loss = loss_fn(y, ffi.fan_in_sparse_matmul_bias(xin, lookup, w, bias))
+    (loss * factor).backward()
+    torch.cuda.synchronize()
+    xn, ln, wn = x.cpu().numpy(), lookup.cpu().numpy(), w.detach().cpu().numpy()
+    scores = oracle.forward(xn, ln, wn) - 0.2
+    _, grad = oracle.sparse_loss(scores, indices, None, oracle.LOSS_SQUARED_HINGE)
+    out_grad = (grad * (factor / (B * L))).astype(np.float32)
+    ref_gx, ref_gw = oracle.backward(xn, ln, wn, out_grad)
+    assert rel_err(w.grad.cpu().numpy(), ref_gw) <= 1e-4
+    assert rel_err(xin.grad.cpu().numpy(), ref_gx) <= 1e-4
+    assert rel_err(bias.grad.cpu().numpy(), out_grad.sum(axis=0)) <= 1e-4
+
+
 def test_loss_sum_is_reproducible(ffi):
     B, L = 128, 20000
     rng = np.random.default_rng(2)

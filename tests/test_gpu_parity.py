@@ -154,11 +154,14 @@ PATH_SHAPES = [
     (96, 128, 12000, 16),      # three batch tiles, weights in LDS: six workgroups of 128 threads, a share of the LDS each
     (160, 256, 9000, 32),      # five batch tiles, weights in LDS: three workgroups of 256 threads
     (288, 64, 20000, 8),       # nine batch tiles, weights in slot order: sixteen workgroups of 64 threads
-    # forward over batch tiles of 64 (N <= 608 and more than 32 samples):
+    # forward over batch tiles of 64 (N <= 608; from 192 samples, from 128 with a fan-in of 64 or more, fan-in 48 / 80 / 112):
     (256, 512, 5000, 64),      # whole tiles, vector loads
-    (100, 608, 3100, 21),      # the widest input of that path, second tile partly filled, odd fan-in (scalar loads)
-    (33, 40, 2100, 24),        # one sample beyond a 32-tile; fan-in with a tail of 8 behind a half chunk of 16
-    (65, 300, 1500, 8),        # one sample in the second 64-tile; fan-in below a half chunk
+    (200, 608, 3100, 21),      # the widest input of that path, fourth tile partly filled, odd fan-in (scalar loads)
+    (33, 40, 2100, 48),        # one sample beyond a 32-tile; three half chunks of 16
+    (193, 300, 1500, 8),       # one sample in the fourth 64-tile; fan-in below a half chunk
+    (130, 256, 2000, 72),      # fan-in with a tail of 8 behind four half chunks
+    # the 32-sample kernel's build for a fan-in below one chunk (loads by quads):
+    (100, 608, 3100, 24), (65, 300, 1500, 8), (128, 768, 5000, 16), (50, 1000, 700, 28), (40, 640, 900, 4),
 ]
 
 
@@ -175,6 +178,50 @@ def test_code_paths(ffi, shape, transposed):
     o_gx, o_gw = oracle.backward(xin, lookup, w, g, transposed=transposed)
     assert rel_err(gw, o_gw) <= GRAD_RTOL
     assert rel_err(gx, o_gx) <= GRAD_RTOL
+
+
+@pytest.mark.parametrize("shape", [(100, 608, 3100, 21),     # 32-sample tiles, the fourth holds 4 samples; loads one by one
+                                   (100, 608, 3100, 24),     # the same with loads by quads (fan-in below one chunk)
+                                   (200, 608, 3100, 21),     # 64-sample tiles, the fourth holds 8 samples
+                                   (70, 768, 2000, 32),      # 32-sample tiles, full chunks
+                                   (70, 2000, 900, 32)])     # wide input
+@pytest.mark.parametrize("transposed", [False, True])
+def test_partly_filled_batch_tiles_write_nothing_behind_the_result(ffi, shape, transposed):
+    # the rows of a batch tile that lie past the batch must not be stored: the result is a view of a larger buffer whose
+    # rows behind it (and a guard row in front) hold a sentinel
+    B, N, L, K = shape
+    x, lookup, w, _ = reference_law_inputs(B, N, L, K, seed=B + K)
+    xin = np.ascontiguousarray(x.T) if transposed else x
+    dx, dl, dw = dev(xin), dev(lookup), dev(w)
+    sentinel = 12345.0
+    whole = torch.full((1 + B + 64, L), sentinel, device="cuda")
+    out = whole[1:1 + B]
+    print(f"case shape={shape} transposed={transposed}", flush=True)
+    ffi._lib.check(ffi._lib.lib().ffi_forward_f32(dx.data_ptr(), dl.data_ptr(), dw.data_ptr(), out.data_ptr(), B, N, L, K,
+                                                  int(transposed), stream()))
+    torch.cuda.synchronize()
+    assert bool((whole[0] == sentinel).all()) and bool((whole[1 + B:] == sentinel).all())
+    assert rel_err(out.cpu().numpy(), oracle.forward(xin, lookup, w, transposed=transposed)) <= FWD_RTOL
+
+
+@pytest.mark.parametrize("option", [("wgrad_units", 3), ("wgrad_units", 4), ("wgrad_stream", -1), ("fwd_lane64", -1),
+                                    ("plan_weights_in_lds", -1), ("plan_weights_in_lds", 1), ("workgroups_per_cu", 1)])
+@pytest.mark.parametrize("shape", [(128, 512, 9000, 32), (64, 768, 5000, 16), (256, 256, 6000, 32)])
+def test_overridden_kernel_choices_keep_parity(ffi, option, shape):
+    # every alternative a benchmark sweep can force computes the same layer
+    B, N, L, K = shape
+    x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=N + K)
+    lib = ffi._lib.lib()
+    print(f"case option={option} shape={shape}", flush=True)
+    ffi._lib.check(lib.ffi_set_option(option[0].encode(), option[1]))
+    try:
+        out = hip_forward(ffi, x, lookup, w, False)
+        gx, gw = hip_backward(ffi, x, lookup, w, g, False)
+    finally:
+        ffi._lib.check(lib.ffi_set_option(option[0].encode(), 0))
+    assert rel_err(out, oracle.forward(x, lookup, w)) <= FWD_RTOL
+    o_gx, o_gw = oracle.backward(x, lookup, w, g)
+    assert rel_err(gw, o_gw) <= GRAD_RTOL and rel_err(gx, o_gx) <= GRAD_RTOL
 
 
 @pytest.mark.parametrize("shape", [(300, 700, 5000, 32), (33, 96, 9, 5), (128, 512, 4100, 100), (40, 1216, 2500, 36), (64, 1100, 3000, 12),
