@@ -27,6 +27,7 @@ from .fixed_fan_in_ops import (  # noqa: E402
     arrange_connections,
     backward_sparse,
     fan_in_sparse_topk,
+    lookup_edited,
 )
 from . import custom_layer, metrics, optimizer  # noqa: E402
 from .optimizer import SparseAdam, SparseOptWrapper, RewireCallback  # noqa: E402
@@ -56,6 +57,7 @@ __all__ = [
     "arrange_connections",
     "backward_sparse",
     "fan_in_sparse_topk",
+    "lookup_edited",
     "StratifiedRewireLayerV2",
     "StratifiedRewireLayer",
     "RewireSelector",

@@ -31,6 +31,7 @@ SIGNATURES = {
     "ffi_host_backward_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _i64, _i64, _i64, _i64]),
     "ffi_input_grad_planned_f32": (_int, [_vp, _vp, _vp, _vp, _i64, _int, _vp]),
     "ffi_cache_clear": (_int, []),
+    "ffi_lookup_edited": (_int, [_vp]),
     "ffi_set_option": (_int, [ctypes.c_char_p, _int]),
     "ffi_cache_bytes": (ctypes.c_size_t, []),
     "ffi_workspace_bytes": (ctypes.c_size_t, [_i64, _i64, _i64, _i64, _int, _int]),

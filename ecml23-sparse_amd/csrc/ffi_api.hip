@@ -583,6 +583,12 @@ int ffi_arrange_connections_f32(int32_t* lookup, float* const* arrays, int n_arr
     return launch_arrange_in_place(lookup, arrays, n_arrays, d.L, d.K, (hipStream_t)stream);
 }
 
+int ffi_lookup_edited(const int32_t* lookup) {
+    if (!lookup) return FFI_ERR_NULL_POINTER;
+    mark_cached_plans_outdated(lookup);
+    return FFI_OK;
+}
+
 int ffi_cache_clear(void) {
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     int dev = -1;

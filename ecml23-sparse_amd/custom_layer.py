@@ -188,8 +188,8 @@ class StratifiedRewireLayerV2(torch.nn.Module):
     def rewire(self, other_vars=None):
         """Gives the selected connections new random sources (weights keep their values) and
         returns ``other_vars`` (e.g. Adam moments, sparse/optimizer.py:14-23) with the entries at
-        the rewired locations set to zero.  The index buffer is edited in place; the library
-        notices through the lookup fingerprint and rebuilds its plan on the next backward call."""
+        the rewired locations set to zero.  The index buffer is edited in place and the library is
+        told so: it rebuilds its plan before the next backward call."""
         other_vars = [] if other_vars is None else list(other_vars)
         self._rewire_count += 1
         if hasattr(self.rewire_selector, "threshold_tensor"):
@@ -203,6 +203,8 @@ class StratifiedRewireLayerV2(torch.nn.Module):
             locations = torch.nonzero(self.rewire_selector.select(self.kernel_weights.detach())).reshape(-1)
             if locations.numel():
                 self.kernel_indices[locations] = self._random_sources(locations.numel(), self.kernel_indices.device)
+            if self.kernel_indices.is_cuda:
+                ops.lookup_edited(self.kernel_indices)
             outputs = []
             for other in other_vars:
                 new_v = other.clone()
@@ -233,6 +235,8 @@ class StratifiedRewireLayer(StratifiedRewireLayerV2):
         idx = self.kernel_indices.view(-1, self.fan_in)
         order = torch.argsort(idx.to(torch.int64), dim=1, stable=True)
         self.kernel_indices.copy_(torch.gather(idx, 1, order).reshape(-1))
+        if self.kernel_indices.is_cuda:
+            ops.lookup_edited(self.kernel_indices)
         self.kernel_weights.data.copy_(torch.gather(self.kernel_weights.data.view(-1, self.fan_in), 1, order).reshape(-1))
         return [torch.gather(o.reshape(-1, self.fan_in), 1, order).reshape(o.shape) for o in other_vars]
 

@@ -370,6 +370,12 @@ def rewire_connections(lookup, weights, arrays, num_features, threshold, seed):
     return changed
 
 
+def lookup_edited(lookup):
+    """Call after editing ``lookup`` in place with torch operations: the library then rebuilds its cached view of the
+    connections before the next backward pass, instead of finding the edit on the device one call late."""
+    _lib.check(_lib.lib().ffi_lookup_edited(lookup.data_ptr()))
+
+
 def fan_in_sparse_topk(features, lookup, weights, bias=None, k=5, transposed=False, want_scores=False):
     """``(values [B,k], labels [B,k] int32)`` of the k best fp32 scores per sample (best first, equal scores
     by ascending label), and the score matrix as a third result if ``want_scores``.  Without

@@ -183,6 +183,16 @@ int ffi_arrange_connections_f32(int32_t* lookup, float* const* arrays, int n_arr
                                 int64_t num_units, int64_t fan_in, ffi_stream_t stream);
 
 /*
+ * Tells the library that the caller has edited (or is about to edit, on the stream of its next backward call) the
+ * lookup at this address in place with code of its own: cached plans of that buffer are marked outdated, and the next
+ * backward call rebuilds before it runs, as after ffi_rewire_f32.  Optional: without it the device-side check
+ * described at the top finds the edit, at the price of one backward call through the recomputing kernels.  No
+ * counterpart in the reference, whose TensorFlow variables are simply read anew by every kernel.  Host-side only;
+ * enqueues nothing.
+ */
+int ffi_lookup_edited(const int32_t* lookup);
+
+/*
  * Overrides one of the library's kernel choices, process-wide (for benchmark sweeps that re-check a choice against its
  * alternative; no counterpart in the reference).  0 always means "the library decides".
  *   "wgrad_units"          3 or 4: units per thread of the weight-gradient kernels that read arranged column ids

@@ -403,13 +403,14 @@ def _label_sample_errors(lookup, w, g, x, gx, gw, B, N, K, labels):
     return rel_err(gw[labels], o_gw), rel_err(gx, o_gx)
 
 
-@pytest.mark.parametrize("route", ["library", "foreign"])
+@pytest.mark.parametrize("route", ["library", "foreign", "foreign_announced"])
 def test_rewiring_at_scale_both_routes(ffi, route):
     # 262,144 labels x fan-in 32 over 768 columns, batch 64 (weights-in-LDS plan, streaming weight gradient).
     # library: ffi_rewire_f32 edits the lookup and tells the plan cache -- the next backward rebuilds the plan first:
     #   plan-driven kernels, bit-identical from call to call, never the recomputing kernels;
     # foreign: a torch kernel edits the lookup -- the next backward is served by the recomputing kernels (correct up to
-    #   the atomics' summation order), the one after it rebuilds.
+    #   the atomics' summation order), the one after it rebuilds;
+    # foreign_announced: the same edit followed by ffi_lookup_edited -- as the library route.
     B, N, L, K = 64, 768, 262144, 32
     rng = np.random.default_rng(5)
     lookup = np.argsort(rng.random((L, N), dtype=np.float32), axis=1)[:, :K].astype(np.int32)
@@ -437,6 +438,8 @@ def test_rewiring_at_scale_both_routes(ffi, route):
     else:
         pos = torch.from_numpy(rng.choice(L * K, (L * K) // 100, replace=False)).cuda()
         dl.view(-1)[pos] = torch.from_numpy(rng.integers(0, N, pos.numel()).astype(np.int32)).cuda()
+        if route == "foreign_announced":
+            ffi._lib.check(lib.ffi_lookup_edited(dl.data_ptr()))
     torch.cuda.synchronize()
     lookup2 = dl.cpu().numpy()
     changed = int((lookup2 != lookup).sum())
@@ -449,7 +452,7 @@ def test_rewiring_at_scale_both_routes(ffi, route):
     assert max(e) <= GRAD_RTOL, e
     d_gx, d_gw = run()
     assert np.array_equal(c_gx, d_gx) and np.array_equal(c_gw, d_gw)      # plan-driven: bit-identical
-    if route == "library":
+    if route != "foreign":
         # the plan was rebuilt before the first backward enqueued anything: that call was plan-driven already
         assert np.array_equal(b_gx, c_gx) and np.array_equal(b_gw, c_gw)
 

@@ -18,30 +18,59 @@ def _inputs(B, N, L, K, seed):
     return x, lookup, w
 
 
-def _run(lib, check, name, x, lookup, w, transposed):
-    B, N = x.shape
-    L, K = lookup.shape
+def _device_inputs(x, lookup, w, transposed):
     feats = np.ascontiguousarray(x.T) if transposed else x
-    dx, dl, dw = (torch.from_numpy(a).cuda() for a in (feats, lookup, w))
-    out = torch.full((B, L), float("nan"), device="cuda")
+    return tuple(torch.from_numpy(a).cuda() for a in (feats, lookup, w))
+
+
+def _call(lib, check, name, dx, dl, dw, out, transposed):
+    B, L = out.shape
+    N = dx.shape[0] if transposed else dx.shape[1]
+    K = dl.shape[1]
     sh = torch.cuda.current_stream().cuda_stream
     check(getattr(lib, name)(dx.data_ptr(), dl.data_ptr(), dw.data_ptr(), out.data_ptr(), B, N, L, K, int(transposed), sh))
     torch.cuda.synchronize()
-    return out.cpu().numpy()
+
+
+def _free_bytes():
+    free, _total = torch.cuda.mem_get_info()
+    return free
 
 
 @pytest.mark.parametrize("transposed", [False, True])
 def test_two_calls_in_a_row_match_the_allocating_entry_point(transposed):
+    import oracle
+
     pkg = load_package()
     assert torch.cuda.is_available()
     lib, check = pkg._lib.lib(), pkg._lib.check
-    # the second call is smaller: it must not see what the first left in the shared array
-    for seed, (B, N, L, K) in enumerate([(128, 768, 20000, 32), (37, 254, 513, 12)]):
+    shapes = [(128, 768, 20000, 32), (37, 254, 513, 12)]      # the second call is smaller: it must not see what the first
+    cases = []                                                # left in the shared array
+    # the allocating entry point first, for every shape: its results are stored and its workspaces dropped again
+    for seed, (B, N, L, K) in enumerate(shapes):
         x, lookup, w = _inputs(B, N, L, K, seed)
-        want = _run(lib, check, "ffi_forward_f32", x, lookup, w, transposed)
-        got = _run(lib, check, "ffi_forward_noalloc_f32", x, lookup, w, transposed)
+        dx, dl, dw = _device_inputs(x, lookup, w, transposed)
+        want = torch.full((B, L), float("nan"), device="cuda")
+        _call(lib, check, "ffi_forward_f32", dx, dl, dw, want, transposed)
+        got = torch.full((B, L), float("nan"), device="cuda")
+        cases.append((x, lookup, w, dx, dl, dw, want.cpu().numpy(), got))
+    check(lib.ffi_cache_clear())
+    assert lib.ffi_cache_bytes() == 0
+    torch.cuda.synchronize()
+    free_before = _free_bytes()
+    for x, lookup, w, dx, dl, dw, want, got in cases:
+        _call(lib, check, "ffi_forward_noalloc_f32", dx, dl, dw, got, transposed)
+        # nothing was allocated: the library holds no workspace, and the device's free memory has not moved (the
+        # outputs were allocated beforehand; torch's allocator is not called in between)
+        assert lib.ffi_cache_bytes() == 0
+        assert _free_bytes() == free_before
+    for x, lookup, w, dx, dl, dw, want, got in cases:
+        got = got.cpu().numpy()
         assert not np.isnan(got).any()
-        assert np.array_equal(got, want), f"shape {(B, N, L, K)}"       # same kernels: bit for bit
+        assert np.array_equal(got, want), f"shape {x.shape} {lookup.shape}"       # same kernels: bit for bit
+        feats = np.ascontiguousarray(x.T) if transposed else x
+        ref = oracle.forward(feats, lookup, w, transposed=transposed)
+        assert np.abs(got - ref).max() <= 1e-5 * np.abs(ref).max()
 
 
 def test_sizes_beyond_the_fixed_array_are_rejected():
