@@ -670,7 +670,22 @@ def main():
         "weight_grad": lambda: check(lib.ffi_weight_grad_planned_f32(plan, ptr(x), ptr(lookup), ptr(g), ptr(gw), B, int(tp), sh)),
         "input_grad": lambda: check(lib.ffi_input_grad_planned_f32(plan, ptr(w), ptr(g), ptr(gx), B, int(tp), sh)),
     }
-    kernel_ms = {name: time_kernel(fn, stream, iters) for name, fn in kernels.items()}
+    back_to_back_ms = {name: time_kernel(fn, stream, iters) for name, fn in kernels.items()}
+    # the same three launches in the order of a step, an event between them: each pass behind the pass it follows in a
+    # step (a pass launched back to back follows its own stores instead, which the forward pass in particular feels)
+    order = ("forward", "weight_grad", "input_grad")
+    rounds = max(20, min(args.steps, 100))
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(rounds)]
+    for _ in range(5):
+        for name in order:
+            kernels[name]()
+    for r in range(rounds):
+        ev[r][0].record(stream)
+        for i, name in enumerate(order):
+            kernels[name]()
+            ev[r][i + 1].record(stream)
+    ev[-1][3].synchronize()
+    kernel_ms = {name: sum(ev[r][i].elapsed_time(ev[r][i + 1]) for r in range(rounds)) / rounds for i, name in enumerate(order)}
     plan_info = (ctypes.c_int64 * 8)()
     check(lib.ffi_plan_info(plan, plan_info))
     check(lib.ffi_plan_destroy(plan))
@@ -680,8 +695,8 @@ def main():
     traffic, traffic_source = measured_traffic(cfg.name)
     narrow = N <= 1216
     pass_kernels = dict(PASS_KERNELS if narrow else WIDE_PASS_KERNELS)
-    if N <= 608 and B > 32:
-        pass_kernels["forward"] = "fwd_lane64_kernel"       # batch tiles of 64 when the [N][64] tile fits in LDS
+    if N <= 608 and B > 32 and (B >= 192 or (K >= 64 and B >= 128) or (K > 32 and K % 32 != 0 and K % 16 == 0)):
+        pass_kernels["forward"] = "fwd_lane64_kernel"       # batch tiles of 64 where the [N][64] tile fits in LDS and pays
     if narrow and plan_info[0] and plan_info[1]:
         # the plan's tiles are small enough for the walking kernel to keep the tile's weights in LDS: no permutation kernel
         pass_kernels["input_grad"] = "igrad_tile_kernel + igrad_reduce_kernel"
@@ -699,6 +714,8 @@ def main():
         "traffic_source": traffic_source,
         "algorithmic_bytes": alg[dominant],
         "kernel_ms": {k: round(v, 4) for k, v in kernel_ms.items()},
+        "kernel_ms_note": f"HIP events around each pass, the passes launched in the order of a step, mean of {rounds} rounds",
+        "kernel_ms_back_to_back": {k: round(v, 4) for k, v in back_to_back_ms.items()},
         "all_kernels_gbps": {k: round(alg[k] / (v * 1e-3) / 1e9, 1) for k, v in kernel_ms.items()},
         "three_pass_gbps": round(alg["total"] / (sum(kernel_ms.values()) * 1e-3) / 1e9, 1),
         # what one pass cannot go below on the two other resources it uses for every multiply-add (published peaks):
