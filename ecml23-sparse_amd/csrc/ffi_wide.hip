@@ -73,11 +73,26 @@ __global__ __launch_bounds__(kWideThreads) void fwd_wide_kernel(const float* __r
                         if (TWO) acc1 = fmaf(ws[u], x1[u], acc1);
                     }
                 }
-                for (; k < kn; ++k) {
-                    const unsigned n = (unsigned)__builtin_amdgcn_readlane((int)iv, k);
-                    const float wk = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wv), k));
-                    acc0 = fmaf(wk, buffer_load_f32(xr, lane_off0, n * row_bytes), acc0);
-                    if (TWO) acc1 = fmaf(wk, buffer_load_f32(xr, lane_off1, n * row_bytes), acc1);
+                if (k < kn) {
+                    // the last, partly filled group, its gathers in flight together like the others: connections behind
+                    // the end repeat the last one and are left out of the sum (one gather at a time cost 40 % at fan-in 12)
+                    float x0[kWideInflight], x1[kWideInflight], ws[kWideInflight];
+#pragma unroll
+                    for (int u = 0; u < kWideInflight; ++u) {
+                        const int kk = min(k + u, kn - 1);
+                        const unsigned n = (unsigned)__builtin_amdgcn_readlane((int)iv, kk);
+                        const float wk = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wv), kk));
+                        ws[u] = wk;
+                        x0[u] = buffer_load_f32(xr, lane_off0, n * row_bytes);
+                        x1[u] = TWO ? buffer_load_f32(xr, lane_off1, n * row_bytes) : 0.f;
+                    }
+#pragma unroll
+                    for (int u = 0; u < kWideInflight; ++u) {
+                        if (k + u < kn) {                       // wave-uniform
+                            acc0 = fmaf(ws[u], x0[u], acc0);
+                            if (TWO) acc1 = fmaf(ws[u], x1[u], acc1);
+                        }
+                    }
                 }
             }
         }
@@ -164,12 +179,24 @@ __global__ __launch_bounds__(kWideThreads) void wgrad_wide_kernel(const float* _
                         if (lane == k + u) mine = s;
                     }
                 }
-                for (; k < kn; ++k) {
-                    const unsigned n = (unsigned)__builtin_amdgcn_readlane((int)iv, k);
-                    const float a = buffer_load_f32(xr, lane_off0, n * row_bytes);
-                    const float b = TWO ? buffer_load_f32(xr, lane_off1, n * row_bytes) : 0.f;
-                    const float s = wave_sum(TWO ? fmaf(in1 ? b : 0.f, g1, (in0 ? a : 0.f) * g0) : (in0 ? a : 0.f) * g0);
-                    if (lane == k) mine = s;
+                if (k < kn) {
+                    // (the last, partly filled group: gathers in flight together, the connections behind the end repeat
+                    // the last one and are not kept)
+                    float x0[kWideInflight], x1[kWideInflight];
+#pragma unroll
+                    for (int u = 0; u < kWideInflight; ++u) {
+                        const unsigned n = (unsigned)__builtin_amdgcn_readlane((int)iv, min(k + u, kn - 1));
+                        x0[u] = buffer_load_f32(xr, lane_off0, n * row_bytes);
+                        x1[u] = TWO ? buffer_load_f32(xr, lane_off1, n * row_bytes) : 0.f;
+                    }
+#pragma unroll
+                    for (int u = 0; u < kWideInflight; ++u) {
+                        if (k + u < kn) {                       // wave-uniform
+                            const float p = TWO ? fmaf(in1 ? x1[u] : 0.f, g1, (in0 ? x0[u] : 0.f) * g0) : (in0 ? x0[u] : 0.f) * g0;
+                            const float s = wave_sum(p);
+                            if (lane == k + u) mine = s;
+                        }
+                    }
                 }
                 if (lane < kn) res[jl * K + k0 + lane] += mine;
             }
@@ -229,11 +256,25 @@ __global__ __launch_bounds__(kWideThreads) void igrad_wide_kernel(const int32_t*
                     if (TWO) acc1 = fmaf(ws[u], b[u], acc1);
                 }
             }
-            for (; i < cnt; ++i) {
-                const unsigned j = (unsigned)__builtin_amdgcn_readlane((int)jv, i);
-                const float wk = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wv), i));
-                acc0 = fmaf(wk, buffer_load_f32(gr, lane_off0, j * (unsigned)ldb * 4u), acc0);
-                if (TWO) acc1 = fmaf(wk, buffer_load_f32(gr, lane_off1, j * (unsigned)ldb * 4u), acc1);
+            if (i < cnt) {
+                // (the last, partly filled group: in flight together, what lies behind the end is left out of the sum)
+                float a[kWideInflight], b[kWideInflight], ws[kWideInflight];
+#pragma unroll
+                for (int u = 0; u < kWideInflight; ++u) {
+                    const int ii = min(i + u, cnt - 1);
+                    const unsigned j = (unsigned)__builtin_amdgcn_readlane((int)jv, ii);
+                    const float wk = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wv), ii));
+                    ws[u] = wk;
+                    a[u] = buffer_load_f32(gr, lane_off0, j * (unsigned)ldb * 4u);
+                    b[u] = TWO ? buffer_load_f32(gr, lane_off1, j * (unsigned)ldb * 4u) : 0.f;
+                }
+#pragma unroll
+                for (int u = 0; u < kWideInflight; ++u) {
+                    if (i + u < cnt) {                          // wave-uniform
+                        acc0 = fmaf(ws[u], a[u], acc0);
+                        if (TWO) acc1 = fmaf(ws[u], b[u], acc1);
+                    }
+                }
             }
         }
     }
