@@ -647,7 +647,10 @@ int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float
                                        bias_grad, d.B, d.N, d.L, d.K, nchunks, n1, ipb, ipb2);                                         \
                 }                                                                                                                      \
             } while (0)
-            if (nchunks == 2) FFI_LAUNCH_ARRANGED(2, 4);
+            // (two chunks per label: one label per thread, 64 sums, measured 2-4 % under two labels per thread, whose 128 sums
+            // leave the streaming kernel 92 bytes of spills per lane)
+            if (nchunks == 2 && (g_options.wgrad_units == 4 || !stream)) FFI_LAUNCH_ARRANGED(2, 4);
+            else if (nchunks == 2) FFI_LAUNCH_ARRANGED(2, 2);
             else if (nchunks == 4) FFI_LAUNCH_ARRANGED(4, 4);
             // the streaming kernel: three units per thread wherever measured (4,000 to 3,000,000 labels, batch 32-512, 64-768
             // columns, fan-in 8-32 and 96: 3-15 % under four units); the kernel without slices: by the model above
