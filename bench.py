@@ -671,21 +671,33 @@ def main():
         "input_grad": lambda: check(lib.ffi_input_grad_planned_f32(plan, ptr(w), ptr(g), ptr(gx), B, int(tp), sh)),
     }
     back_to_back_ms = {name: time_kernel(fn, stream, iters) for name, fn in kernels.items()}
-    # the same three launches in the order of a step, an event between them: each pass behind the pass it follows in a
-    # step (a pass launched back to back follows its own stores instead, which the forward pass in particular feels)
+    # What a pass costs inside a step: the three launches in the order of a step, timed as whole rounds with all three
+    # and with one of them left out; a pass's figure is the difference per round.  (No event inside a round: a record
+    # between two kernels opens a gap of several microseconds; and a pass launched back to back follows its own stores
+    # instead of the pass it follows in a step, which the forward pass in particular feels.)
     order = ("forward", "weight_grad", "input_grad")
     rounds = max(20, min(args.steps, 100))
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(rounds)]
-    for _ in range(5):
-        for name in order:
-            kernels[name]()
-    for r in range(rounds):
-        ev[r][0].record(stream)
-        for i, name in enumerate(order):
-            kernels[name]()
-            ev[r][i + 1].record(stream)
-    ev[-1][3].synchronize()
-    kernel_ms = {name: sum(ev[r][i].elapsed_time(ev[r][i + 1]) for r in range(rounds)) / rounds for i, name in enumerate(order)}
+
+    def rounds_ms(names):
+        for _ in range(5):
+            for name in names:
+                kernels[name]()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record(stream)
+        for _ in range(rounds):
+            for name in names:
+                kernels[name]()
+        b.record(stream)
+        b.synchronize()
+        return a.elapsed_time(b) / rounds
+
+    whole, without = [], {}
+    for left_out in order:
+        whole.append(rounds_ms(order))
+        without[left_out] = rounds_ms(tuple(n for n in order if n != left_out))
+    whole.append(rounds_ms(order))
+    whole_ms = sum(whole) / len(whole)
+    kernel_ms = {name: whole_ms - without[name] for name in order}
     plan_info = (ctypes.c_int64 * 8)()
     check(lib.ffi_plan_info(plan, plan_info))
     check(lib.ffi_plan_destroy(plan))
@@ -714,7 +726,8 @@ def main():
         "traffic_source": traffic_source,
         "algorithmic_bytes": alg[dominant],
         "kernel_ms": {k: round(v, 4) for k, v in kernel_ms.items()},
-        "kernel_ms_note": f"HIP events around each pass, the passes launched in the order of a step, mean of {rounds} rounds",
+        "kernel_ms_note": f"cost of each pass inside a round of the three passes in step order: {rounds} rounds with all three minus {rounds} rounds "
+                          f"without it, HIP events around the {rounds} rounds (whole round {whole_ms:.4f} ms)",
         "kernel_ms_back_to_back": {k: round(v, 4) for k, v in back_to_back_ms.items()},
         "all_kernels_gbps": {k: round(alg[k] / (v * 1e-3) / 1e9, 1) for k, v in kernel_ms.items()},
         "three_pass_gbps": round(alg["total"] / (sum(kernel_ms.values()) * 1e-3) / 1e9, 1),
