@@ -184,8 +184,9 @@ def parse_args():
     ap.add_argument("--no-rewire-costs", action="store_true", help="skip the plan-build / first-backward-after-rewiring timings")
     ap.add_argument("--sweep", nargs="?", const="all", default=None, choices=["all", "reference", "layer", "layer_k64"],
                     help="instead of the benchmark line: batch x width x labels x fan-in grids of the passes, one CSV line per "
-                         "timing (gpurun_out/sweep.csv): 'reference' = the grid of the reference's testing/detailed-bench.cpp:26-112, "
+                         "timing (file: --sweep-csv): 'reference' = the grid of the reference's testing/detailed-bench.cpp:26-112, "
                          "'layer' = the same axes around the headline workload, each pass also with the library's kernel choices overridden")
+    ap.add_argument("--sweep-csv", default=os.path.join("gpurun_out", "sweep.csv"), help="where --sweep writes its timings (relative to this file)")
     ap.add_argument("--copy-bytes", type=int, default=0,
                     help="also run one plain device copy kernel of this many bytes (read N, write N): the "
                          "known-size reference that rocprofv3 FETCH_SIZE/WRITE_SIZE readings are scaled by")
@@ -472,7 +473,7 @@ SWEEP_VARIANTS = {
 
 def sweep(args, pkg, synth):
     """Times the passes over SWEEP_GRIDS and writes one CSV line per (point, layout, pass, variant) to
-    gpurun_out/sweep.csv; prints one JSON line that lists where an override beat the library's own choice."""
+    the file named by --sweep-csv; prints one JSON line that lists where an override beat the library's own choice."""
     import csv
     import ctypes
 
@@ -481,8 +482,8 @@ def sweep(args, pkg, synth):
     stream = torch.cuda.current_stream()
     sh = stream.cuda_stream
     ptr = lambda a: a.data_ptr()  # noqa: E731
-    os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
-    path = os.path.join(ROOT, "gpurun_out", "sweep.csv")
+    path = os.path.join(ROOT, args.sweep_csv)
+    os.makedirs(os.path.dirname(path), exist_ok=True)
     rows, beaten, points = [], [], 0
     names = ("batch", "num_features", "num_units", "fan_in")
     grids = [g for g in SWEEP_GRIDS if args.sweep in ("all", g)]
