@@ -338,7 +338,10 @@ __device__ __forceinline__ void stage_rows32_direct(float* xs, const float* __re
     }
 }
 
-template <int NCH, int UNITS, bool QUADS>
+// WALK: connections walked in a label's last chunk.  A fan-in that is not a multiple of 32 leaves that chunk partly
+// filled, and the arranged order puts the real connections first: such launches walk its first 8, 16 or 24 entries only
+// (labels of one, two or four chunks, i.e. the launches in which a thread holds whole labels).
+template <int NCH, int UNITS, bool QUADS, int WALK = kWgChunk>
 __global__ __launch_bounds__(kResThreads) void wgrad_stream_kernel(const float* __restrict__ xT,
                                                                    const unsigned short* __restrict__ idx16,
                                                                    const float* __restrict__ g,
@@ -351,6 +354,7 @@ __global__ __launch_bounds__(kResThreads) void wgrad_stream_kernel(const float* 
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int blk = blockIdx.x;
     static_assert(UNITS % NCH == 0 && UNITS <= kResUnits, "whole labels per thread");
+    static_assert(WALK == kWgChunk || (QUADS && WALK % 8 == 0 && WALK > 0 && WALK < kWgChunk), "short walks: a thread's units must all end in the same chunk");
     constexpr int kItems = UNITS / NCH;
     const long long total_items = NCH == 1 ? (long long)L * nchunks : (long long)L;
     const long long i_begin = blk < n1 ? (long long)blk * ipb1 : (long long)n1 * ipb1 + (long long)(blk - n1) * ipb2;
@@ -461,23 +465,31 @@ __global__ __launch_bounds__(kResThreads) void wgrad_stream_kernel(const float* 
                     for (int b = 0; b < 32; ++b) t += gb[b];
                     gsum[qq] = t;
                 }
-#pragma unroll
-                for (int c = 0; c < NCH; ++c) {
+                static_for<NCH>([&](auto cc) {
+                    constexpr int c = decltype(cc)::value;
+                    // connections walked in this chunk (the label's last chunk may be partly filled), and in the walk that follows it
+                    constexpr int kWalk = c == NCH - 1 ? WALK : kWgChunk;
+                    constexpr int kNextWalk = c + 1 < NCH ? (c + 1 == NCH - 1 ? WALK : kWgChunk) : (NCH == 1 ? WALK : kWgChunk);
+                    // the quarters of that walk's entries are requested at even distances, each a few connections before its stretch ends
+                    constexpr int kQuarters = kNextWalk / 8, kStep = kWalk / kQuarters, kAt = kStep > 3 ? kStep - 3 : 0;
                     if (c > 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                     unsigned idp[kWgChunk / 2];
 #pragma unroll
                     for (int t = 0; t < kWgChunk / 2; ++t) idp[t] = idn[t];
                     // (no branch in here: the walk stays one basic block; behind the last step it fetches ids nobody uses
                     // and zero rows from an empty buffer)
-                    static_for<kWgChunk>([&](auto kc) {
+                    static_for<kWalk>([&](auto kc) {
                         constexpr int k = decltype(kc)::value;
                         const unsigned e = (k & 1) ? (idp[k >> 1] >> 16) : idp[k >> 1];
                         if constexpr (QUADS) {
-                            if (c == 0 && (k & 3) == 0) fetch_g_rows4(rn, jn0, std::integral_constant<int, k / 4>{});
+                            // (the eight four-row requests of the next step, spread evenly over the walk of the first chunk)
+                            constexpr int kPer = kWalk / 8;
+                            if constexpr (c == 0 && k % kPer == 0) fetch_g_rows4(rn, jn0, std::integral_constant<int, k / kPer>{});
                         } else {
-                            if (c == 0) fetch_g_row(rn, jn, kc);
+                            if constexpr (c == 0) fetch_g_row(rn, jn, kc);
                         }
-                        if ((k & 7) == 5) fetch_ids_quarter(c + 1 < NCH ? item[qq] : itn, c + 1 < NCH ? c + 1 : 0, k >> 3, idn);
+                        if constexpr (k % kStep == kAt && k / kStep < kQuarters)
+                            fetch_ids_quarter(c + 1 < NCH ? item[qq] : itn, c + 1 < NCH ? c + 1 : 0, k / kStep, idn);
                         float4 xv[8];
                         wgrad_reads(((e & kArrIdMask) << 7) + skew, xv);
                         __builtin_amdgcn_sched_barrier(0);
@@ -485,7 +497,7 @@ __global__ __launch_bounds__(kResThreads) void wgrad_stream_kernel(const float* 
                         __builtin_amdgcn_sched_barrier(0);
                     });
                     asm volatile("" ::: "memory");
-                }
+                });
             }
         }
     }
@@ -543,11 +555,12 @@ __global__ __launch_bounds__(kResThreads) void wgrad_stream_kernel(const float* 
                         if (it0 + (long long)r < i_end)
                             *reinterpret_cast<float4*>(gw + (size_t)(j0 + (int)r) * K + k0 + 4 * q) = make_float4(v.x, v.y, v.z, v.w);
                     }
-                } else if (vec4 && k0 + kWgChunk <= K) {
+                } else if (vec4) {
+                    // (a partly filled chunk of a fan-in that is a multiple of four: its first quads)
 #pragma unroll
                     for (int t = 0; t < kWgChunk / 4; ++t) {
                         const lds_v4f v = *(lds_v4f_ptr)(size_t)(srow + (((unsigned)t ^ sw) << 4));
-                        if (mine) *reinterpret_cast<float4*>(grow + 4 * t) = make_float4(v.x, v.y, v.z, v.w);
+                        if (mine && k0 + 4 * t < K) *reinterpret_cast<float4*>(grow + 4 * t) = make_float4(v.x, v.y, v.z, v.w);
                     }
                 } else {
                     for (int k = 0; k < kWgChunk; ++k) {
@@ -627,12 +640,25 @@ int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float
                                         (size_t)kResThreads * kSlotPitch * sizeof(float));
             // a label of two or four chunks: all its units in one thread (its out_grad values are loaded once per
             // batch tile instead of once per chunk); the work is then split by labels, not by units
+            // connections in a label's last chunk, rounded up to the eights the walk is cut in
+            const int last_walk = (d.K - (nchunks - 1) * kWgChunk + 7) / 8 * 8;
+#define FFI_LAUNCH_STREAM_WALK(NCH, UNITS, WALK)                                                                                       \
+            do {                                                                                                                       \
+                FFI_HIP_TRY(hipFuncSetAttribute((const void*)wgrad_stream_kernel<NCH, UNITS, true, WALK>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
+                hipLaunchKernelGGL((wgrad_stream_kernel<NCH, UNITS, true, WALK>), dim3((unsigned)(n1 + n2)), dim3(kResThreads), lds, s, xT, plan->idx16, g, gw, \
+                                   bias_grad, d.B, d.N, d.L, d.K, nchunks, n1, ipb, ipb2);                                             \
+            } while (0)
 #define FFI_LAUNCH_ARRANGED(NCH, UNITS)                                                                                                \
             do {                                                                                                                       \
                 split(NCH == 1 ? (long long)d.L * nchunks : (long long)d.L, (long long)(UNITS / NCH) * kResThreads);                   \
                 if (stream) {                                                                                                          \
                     constexpr bool kQuads = NCH > 1;   /* a wavefront's lanes hold consecutive labels */                               \
-                    if (kQuads || nchunks == 1) {                                                                                      \
+                    if ((kQuads || nchunks == 1) && last_walk < kWgChunk) {                                                            \
+                        /* the last chunk of every label is partly filled: its walk covers the filled part only */                     \
+                        if (last_walk == 8) FFI_LAUNCH_STREAM_WALK(NCH, UNITS, 8);                                                     \
+                        else if (last_walk == 16) FFI_LAUNCH_STREAM_WALK(NCH, UNITS, 16);                                              \
+                        else FFI_LAUNCH_STREAM_WALK(NCH, UNITS, 24);                                                                   \
+                    } else if (kQuads || nchunks == 1) {                                                                               \
                         FFI_HIP_TRY(hipFuncSetAttribute((const void*)wgrad_stream_kernel<NCH, UNITS, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
                         hipLaunchKernelGGL((wgrad_stream_kernel<NCH, UNITS, true>), dim3((unsigned)(n1 + n2)), dim3(kResThreads), lds, s, xT, plan->idx16, g, gw, \
                                            bias_grad, d.B, d.N, d.L, d.K, nchunks, n1, ipb, ipb2);                                     \
@@ -658,6 +684,7 @@ int launch_weight_grad(const float* x, const int32_t* idx, const float* g, float
                      (g_options.wgrad_units != 4 && (stream || three_units_cheaper((long long)d.L * nchunks, d.N, cus)))) FFI_LAUNCH_ARRANGED(1, 3);
             else FFI_LAUNCH_ARRANGED(1, 4);
 #undef FFI_LAUNCH_ARRANGED
+#undef FFI_LAUNCH_STREAM_WALK
             FFI_HIP_TRY(hipGetLastError());
             return FFI_OK;
         }

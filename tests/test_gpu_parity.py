@@ -232,7 +232,11 @@ def test_overridden_kernel_choices_keep_parity(ffi, option, shape):
                                    (70, 768, 5000, 96),       # three chunks per label: unit numbers wrap inside a wavefront (row-by-row out_grad fetches)
                                    (129, 763, 70, 32),        # one sample in the fifth batch tile, odd width (x staged through registers), 70 labels
                                    (32, 768, 64, 8),          # the fewest labels the streaming kernel takes
-                                   (64, 776, 4000, 32)])      # x tile and out_grad slices do not fit the LDS together: the kernel without slices
+                                   (64, 776, 4000, 32),       # x tile and out_grad slices do not fit the LDS together: the kernel without slices
+                                   # a last chunk that is partly filled is walked as far as it is filled (8, 16 or 24 connections):
+                                   (64, 768, 4000, 8), (64, 768, 4000, 12), (100, 512, 3000, 20), (33, 640, 5000, 24), (64, 256, 3000, 3),
+                                   (96, 512, 3000, 40), (64, 512, 3000, 52), (40, 300, 2600, 63),        # two chunks
+                                   (64, 300, 2600, 104), (32, 256, 2000, 97), (48, 200, 1500, 120)])    # four chunks
 def test_planned_weight_grad_code_paths(ffi, shape):
     B, N, L, K = shape
     x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=B + K)
