@@ -271,8 +271,8 @@ constexpr unsigned kPadPos = 0xffffu;      // pos16 of a padding slot; real posi
 // LDS of the kernel that walks the tiled form: the tile's rows of out_grad (per bank half: half the tile plus some room
 // for the balancing) and two all-zero rows, 128 bytes each; with the tile's weights behind them, tile_labels * K floats
 // and one zero word that padding slots read.
-constexpr size_t kPlanLdsBudget = 160000;
-inline int tiled_rows_per_half(int tile_labels) { return tile_labels / 2 + (tile_labels / 16 < 64 ? tile_labels / 16 : 64); }
+constexpr size_t kPlanLdsBudget = 163700;      // of the 163,840 bytes a workgroup can have (the walking kernel has no other LDS)
+inline int tiled_rows_per_half(int tile_labels) { return tile_labels / 2 + (tile_labels / 32 < 64 ? tile_labels / 32 : 64); }
 inline size_t tiled_lds_bytes(int tile_labels, int K, bool with_weights) {
     return (size_t)(2 * tiled_rows_per_half(tile_labels) + 2) * 128 + (with_weights ? ((size_t)tile_labels * K + 4) * 4 : 0);
 }
