@@ -502,7 +502,8 @@ __global__ void tile_fill_bitmap_kernel(const int32_t* __restrict__ idx, const u
     }
 }
 
-// LDS the bitmap form needs
+// LDS the bitmap form needs, and may have
+constexpr size_t kFillLdsLimit = 160 * 1024 - 64;
 inline size_t tile_fill_bitmap_lds(int threads, int tile_labels, int K, int* words_out) {
     const int words = ((tile_labels + 31) / 32) | 1;
     *words_out = words;
@@ -619,6 +620,13 @@ int plan_tile_labels(int N, int K, int L, int batch_hint, bool* weights_in_lds) 
         const size_t budget = (threads <= 256 && nbt_hint >= 2) ? kPlanLdsBudget / (size_t)(768 / threads) : kPlanLdsBudget;
         while (tw >= 64 && tiled_lds_bytes(tw, K, true) > budget) tw -= 2;
         while (tw >= 64 && (long long)tw * K >= 32768) tw -= 2;
+        // a tile the bitmap fill has the LDS for (its bitmaps grow by whole words of 32 labels) builds five times faster
+        // than one it has not; take the next smaller such tile where that costs at most a twentieth of the tile
+        int words = 0;
+        if (tw >= 64 && tile_fill_bitmap_lds(threads, tw, K, &words) > kFillLdsLimit) {
+            const int fits = tw & ~31;
+            if (fits >= 64 && fits * 20 >= tw * 19 && tile_fill_bitmap_lds(threads, fits, K, &words) <= kFillLdsLimit) tw = fits;
+        }
         if (tw >= 64) { TL = tw; w_in_lds = true; }
     }
     // the forms with weights in slot order, workgroups of at most 512 threads: one label per thread, so that two or more
@@ -677,7 +685,7 @@ int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
         int words = 0;
         const size_t fill_lds = tile_fill_bitmap_lds(threads, TL, p->K, &words);
         const unsigned pad_pos = w_in_lds ? (unsigned)TL * (unsigned)p->K : kPadPos;
-        if (fill_lds <= 160 * 1024 - 64) {
+        if (fill_lds <= kFillLdsLimit) {
             hipError_t ea = hipFuncSetAttribute((const void*)tile_fill_bitmap_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)fill_lds);
             if (ea != hipSuccess) return hip_fail(ea);
             hipLaunchKernelGGL(tile_fill_bitmap_kernel, dim3(tiles), dim3(threads), fill_lds, s, lookup, p->rowpos, p->L, p->K, TL, 2 * cap,
