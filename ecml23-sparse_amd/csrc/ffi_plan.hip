@@ -627,6 +627,22 @@ int plan_tile_labels(int N, int K, int L, int batch_hint, bool* weights_in_lds) 
             const int fits = tw & ~31;
             if (fits >= 64 && fits * 20 >= tw * 19 && tile_fill_bitmap_lds(threads, fits, K, &words) <= kFillLdsLimit) tw = fits;
         }
+        // Tiles per workgroup come in whole numbers: the walking kernel runs cus / batch tiles label streams of
+        // ceil(tiles / streams) tiles each, and the largest tile can leave the last stream nearly empty, or whole CUs
+        // without a stream (670,091 labels in 608-label tiles: 62 streams of 18 tiles on 64 CUs' worth of workgroups).
+        // The tile shrinks to what fills every stream with that same number of tiles (582 labels there: 64 x 18); a
+        // smaller tile pads a little more per connection, which costs less than the idle streams.  (Workgroups that share
+        // a CU are left alone: there the streams outnumber the CUs.)
+        if (tw >= 64 && (threads > 256 || nbt_hint < 2)) {
+            const long long streams = std::max(1, device_cu_count() / std::max(1, nbt_hint));
+            const long long tiles = ((long long)L + tw - 1) / tw;
+            if (tiles > streams) {
+                const long long per_stream = (tiles + streams - 1) / streams;
+                int even = (int)(((long long)L + streams * per_stream - 1) / (streams * per_stream));
+                even = (even + 1) & ~1;
+                if (even >= 64 && even <= tw && even * 10 >= tw * 9) tw = even;
+            }
+        }
         if (tw >= 64) { TL = tw; w_in_lds = true; }
     }
     // the forms with weights in slot order, workgroups of at most 512 threads: one label per thread, so that two or more
