@@ -160,6 +160,8 @@ PATH_SHAPES = [
     (33, 40, 2100, 48),        # one sample beyond a 32-tile; three half chunks of 16
     (193, 300, 1500, 8),       # one sample in the fourth 64-tile; fan-in below a half chunk
     (130, 256, 2000, 72),      # fan-in with a tail of 8 behind four half chunks
+    # full chunks loaded by quads from rows that are only 4-byte aligned (fan-in no multiple of four), last chunk one by one:
+    (64, 768, 3000, 33), (40, 512, 2000, 63), (200, 300, 1500, 35), (130, 256, 2000, 67),
     # the 32-sample kernel's build for a fan-in below one chunk (loads by quads):
     (100, 608, 3100, 24), (65, 300, 1500, 8), (128, 768, 5000, 16), (50, 1000, 700, 28), (40, 640, 900, 4),
 ]
