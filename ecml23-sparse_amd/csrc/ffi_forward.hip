@@ -39,6 +39,33 @@ __device__ __forceinline__ void fwd_lane_step(unsigned base, float wv, float (&a
     acc[4 * C + 3] = fmaf(wv, v.w, acc[4 * C + 3]);
 }
 
+// One connection of the lane's label: the eight 16-byte reads of row `rb` (chunk order skewed per lane) and their 32
+// multiply-adds, in a pinned order -- two reads in flight; a read's registers are refilled as soon as its four values
+// are used, under the multiply-adds of the other read.  Left to itself the scheduler finds this order or one that
+// waits for each read in turn (13 % slower over the whole kernel), depending on code far away from here.
+__device__ __forceinline__ void fwd_lane_connection(unsigned rb, float wv, float (&acc)[32]) {
+    lds_v4f a = *(lds_v4f_ptr)(size_t)rb;
+    lds_v4f b = *(lds_v4f_ptr)(size_t)(rb ^ 16u);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        acc[8 * p + 0] = fmaf(wv, a.x, acc[8 * p + 0]);
+        acc[8 * p + 4] = fmaf(wv, b.x, acc[8 * p + 4]);
+        acc[8 * p + 1] = fmaf(wv, a.y, acc[8 * p + 1]);
+        acc[8 * p + 2] = fmaf(wv, a.z, acc[8 * p + 2]);
+        acc[8 * p + 3] = fmaf(wv, a.w, acc[8 * p + 3]);
+        acc[8 * p + 5] = fmaf(wv, b.y, acc[8 * p + 5]);
+        __builtin_amdgcn_sched_barrier(0);
+        if (p < 3) a = *(lds_v4f_ptr)(size_t)(rb ^ (unsigned)(32 * p + 32));
+        __builtin_amdgcn_sched_barrier(0);
+        acc[8 * p + 6] = fmaf(wv, b.z, acc[8 * p + 6]);
+        acc[8 * p + 7] = fmaf(wv, b.w, acc[8 * p + 7]);
+        __builtin_amdgcn_sched_barrier(0);
+        if (p < 3) b = *(lds_v4f_ptr)(size_t)(rb ^ (unsigned)(32 * p + 48));
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
 // What the kernel does with a finished score s (after the bias):
 //   kEpiScores       out = s
 //   kEpiLossGrad     out = scale * dloss(s, 0)/ds, the loss gradient of a position that is not a listed label
@@ -207,10 +234,7 @@ __global__ __launch_bounds__(kTileThreads) void fwd_lane32_kernel(const float* _
                 if (full || k < kn) {
                     const unsigned id = (k & 1) ? (idp[k >> 1] >> 16) : (idp[k >> 1] & 0xffffu);
                     const unsigned rb = (id << 7) + skewbase;
-                    fwd_lane_step<0>(rb, wv[k], acc); fwd_lane_step<1>(rb, wv[k], acc);
-                    fwd_lane_step<2>(rb, wv[k], acc); fwd_lane_step<3>(rb, wv[k], acc);
-                    fwd_lane_step<4>(rb, wv[k], acc); fwd_lane_step<5>(rb, wv[k], acc);
-                    fwd_lane_step<6>(rb, wv[k], acc); fwd_lane_step<7>(rb, wv[k], acc);
+                    fwd_lane_connection(rb, wv[k], acc);
                 }
             }
         }
