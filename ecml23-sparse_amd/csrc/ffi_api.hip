@@ -539,7 +539,7 @@ int ffi_plan_info(const ffi_plan* plan, int64_t info[8]) {
     info[2] = plan->tile_labels;
     info[3] = plan->threads;
     info[4] = plan->tiles;
-    info[5] = plan->total_rows;
+    info[5] = plan->total_rows + (plan->upper ? plan->upper->total_rows : 0);   // (both column windows of a wide input)
     info[6] = (int64_t)plan->bytes;
     info[7] = plan->idx16 != nullptr ? 1 : 0;
     return FFI_OK;
@@ -652,25 +652,31 @@ size_t ffi_workspace_bytes(int64_t batch, int64_t num_features, int64_t num_unit
     else features_slot = (d.tp && ldw == B) ? 0 : N * ldw * 4;
     size_t total = 0, partial_slot = 0;
     if (passes & FFI_PASS_BACKWARD) {
-        if (d.N <= 1024 && d.K <= 1024 && d.L < (1 << 25)) {
+        const bool one_window = d.N <= 1024, two_windows = !one_window && tile_path_fits(d.N) && d.N <= 2048;
+        if ((one_window || two_windows) && d.K <= 1024 && d.L < (1 << 25)) {
             // tiled plan: the geometry of ffi_plan.hip, the slot rows of a slice estimated for column ids drawn uniformly
-            // (longest of 64 columns whose lengths scatter like Poisson counts around tile_labels * fan_in / num_features)
-            const size_t threads = (N + 63) / 64 * 64;
-            bool w_in_lds = false;
-            const size_t TL = (size_t)plan_tile_labels(d.N, d.K, d.L, d.B, &w_in_lds);
-            const size_t tiles = (L + TL - 1) / TL, slices = threads / 64;
-            const double mu = (double)TL * (double)K / (double)N;
-            const size_t rows = (size_t)(mu + 2.6 * std::sqrt(mu) + 3.0);
-            const size_t slots = tiles * slices * rows * 64;
-            total += slots * 2 * 2 + (tiles * slices + 1) * 4 + L * 2;                  // 4 bytes per slot (lab16 + pos16, or slot32), slice_off, rowpos
+            // (longest of 64 columns whose lengths scatter like Poisson counts around tile_labels * fan_in / num_features);
+            // inputs wider than 1,024 columns have one such form per half of the columns, walked one after the other
+            const size_t lower = one_window ? N : ((N + 1) / 2 + 63) / 64 * 64;
+            for (int win = 0; win < (one_window ? 1 : 2); ++win) {
+                const size_t cols = win == 0 ? lower : N - lower;
+                const size_t threads = (cols + 63) / 64 * 64;
+                bool w_in_lds = false;
+                const size_t TL = (size_t)plan_tile_labels((int)cols, d.K, d.L, d.B, &w_in_lds);
+                const size_t tiles = (L + TL - 1) / TL, slices = threads / 64;
+                const double mu = (double)TL * (double)K / (double)N;
+                const size_t rows = (size_t)(mu + 2.6 * std::sqrt(mu) + 3.0);
+                const size_t slots = tiles * slices * rows * 64;
+                total += slots * 2 * 2 + (tiles * slices + 1) * 4 + L * 2;              // 4 bytes per slot (lab16 + pos16, or slot32), slice_off, rowpos
+                if (!w_in_lds) features_slot = std::max(features_slot, slots * 4);     // weights in slot order
+                const size_t nbt = (B + 31) / 32;
+                const size_t per_cu = (size_t)tiled_workgroups_per_cu((int)threads, (int)TL, d.K, w_in_lds, (int)((B + 31) / 32));
+                size_t streams = std::max<size_t>(1, std::min<size_t>(tiles, per_cu * (size_t)device_cu_count() / std::max<size_t>(1, nbt)));
+                const size_t tiles_per_stream = (tiles + streams - 1) / streams;        // (as the launcher evens them out)
+                streams = (tiles + tiles_per_stream - 1) / tiles_per_stream;
+                partial_slot = std::max(partial_slot, streams * threads * nbt * 32 * 4);
+            }
             if (tile_path_fits(d.N) && d.N < (1 << kArrIdBits)) total += arranged_words((long long)(L * ((K + 31) / 32))) * 2;   // idx16
-            if (!w_in_lds) features_slot = std::max(features_slot, slots * 4);         // weights in slot order
-            const size_t nbt = (B + 31) / 32;
-            const size_t per_cu = (size_t)tiled_workgroups_per_cu((int)threads, (int)TL, d.K, w_in_lds, (int)((B + 31) / 32));
-            size_t streams = std::max<size_t>(1, std::min<size_t>(tiles, per_cu * (size_t)device_cu_count() / std::max<size_t>(1, nbt)));
-            const size_t tiles_per_stream = (tiles + streams - 1) / streams;            // (as the launcher evens them out)
-            streams = (tiles + tiles_per_stream - 1) / tiles_per_stream;
-            partial_slot = streams * threads * nbt * 32 * 4;
         } else {
             const size_t nblocks = (L + 65535) / 65536;
             total += L * K * 4 + (nblocks * N + 1) * 4;                                 // perm, col_ptr

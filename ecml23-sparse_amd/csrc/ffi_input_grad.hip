@@ -297,10 +297,11 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
 template <bool TP>
 __global__ __launch_bounds__(256) void igrad_reduce_kernel(const float* __restrict__ partial, float* __restrict__ gx,
                                                            int B, int N, int streams, int nthreads, int bpad,
-                                                           const unsigned long long* __restrict__ verdict) {
+                                                           const unsigned long long* __restrict__ verdict, int col_lo) {
     const int b = blockIdx.x * 256 + threadIdx.x;
-    const int n = blockIdx.y;
+    const int n = blockIdx.y;                          // column inside the plan's window; gx column n + col_lo
     if (b >= B) return;
+    gx += TP ? (size_t)col_lo * B : (size_t)col_lo;
     // the plan is known to be outdated: zeros, for the kernel that recomputes the gradient from the lookup to add to
     if (verdict != nullptr && *verdict == 0) {
         if (TP) gx[(size_t)n * B + b] = 0.f; else gx[(size_t)b * N + n] = 0.f;
@@ -367,11 +368,11 @@ int launch_tiled(const ffi_plan* p, const float* w, const float* g, float* gx, i
         FFI_LAUNCH_TILE(1024, 1, false);
     }
 #undef FFI_LAUNCH_TILE
-    dim3 rgrid((B + 255) / 256, p->N);
+    dim3 rgrid((B + 255) / 256, p->col_n ? p->col_n : p->N);
     if (tp)
-        hipLaunchKernelGGL(igrad_reduce_kernel<true>, rgrid, dim3(256), 0, s, partial, gx, B, p->N, streams, p->threads, bpad, verdict);
+        hipLaunchKernelGGL(igrad_reduce_kernel<true>, rgrid, dim3(256), 0, s, partial, gx, B, p->N, streams, p->threads, bpad, verdict, p->col_lo);
     else
-        hipLaunchKernelGGL(igrad_reduce_kernel<false>, rgrid, dim3(256), 0, s, partial, gx, B, p->N, streams, p->threads, bpad, verdict);
+        hipLaunchKernelGGL(igrad_reduce_kernel<false>, rgrid, dim3(256), 0, s, partial, gx, B, p->N, streams, p->threads, bpad, verdict, p->col_lo);
     FFI_HIP_TRY(hipGetLastError());
     return FFI_OK;
 }
@@ -386,7 +387,14 @@ int launch_input_grad(const ffi_plan* p, const float* w, const float* g, float* 
     if (p->tiled) {
         if (!p->slice_off || !p->rowpos || (p->w_in_lds ? !p->slot32 : (!p->lab16 || !p->pos16))) return FFI_ERR_BAD_ARGUMENT;
         if (zeroed_if_outdated) *zeroed_if_outdated = verdict != nullptr;
-        return launch_tiled(p, w, g, gx, B, tp, s, verdict);
+        FFI_TRY(launch_tiled(p, w, g, gx, B, tp, s, verdict));
+        // inputs wider than one workgroup has threads: the second half of the columns has a tiled form of its own
+        if (p->upper != nullptr) {
+            const ffi_plan* u = p->upper;
+            if (!u->tiled || !u->slice_off || !u->rowpos || (u->w_in_lds ? !u->slot32 : (!u->lab16 || !u->pos16))) return FFI_ERR_BAD_ARGUMENT;
+            return launch_tiled(u, w, g, gx, B, tp, s, verdict);
+        }
+        return FFI_OK;
     }
     if (!p->perm || !p->col_ptr) return FFI_ERR_BAD_ARGUMENT;
     return launch_input_grad_wide(p, w, g, gx, B, tp, s);

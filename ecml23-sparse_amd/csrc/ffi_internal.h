@@ -263,6 +263,11 @@ struct ffi_plan {
     hipEvent_t helper_event = nullptr;
     int batch_hint = 0;                       // batch size the plan is expected to be used with (0 = unknown); steers layout choices only
     bool w_in_lds = false;                    // tiled form: tiles small enough for the walking kernel to keep the tile's weights in LDS too
+    // Inputs of 1,025 to 1,216 columns (the LDS tile holds them, a workgroup of one thread per column does not): the tiled
+    // form is built twice, for the lower and the upper half of the columns.  This plan's tiled arrays then cover columns
+    // [col_lo, col_lo + col_n) = the lower half, and `upper` (tiled arrays only; everything else of it is unused) the rest.
+    int col_lo = 0, col_n = 0;                // col_n == 0: all N columns
+    ffi_plan* upper = nullptr;
 };
 
 namespace ffi {

@@ -189,8 +189,9 @@ __device__ __forceinline__ unsigned column_slots(unsigned thread, unsigned even,
 // of even-count minus odd-count of the column), which keeps the columns that matter close to an even split.
 // Rows of a half are handed out in ascending order, at most `cap` per half.  One workgroup per tile; the tile's
 // column ids are staged in LDS, one wavefront then decides label after label (lane <-> connection).
+// (`col_lo`: the plan covers the columns [col_lo, col_lo + ncols) only; connections into other columns are left out)
 __global__ __launch_bounds__(256) void tile_color_kernel(const int32_t* __restrict__ idx, int L, int K, int tile_labels, int cap,
-                                                         int ncols, unsigned short* __restrict__ rowpos) {
+                                                         int ncols, unsigned short* __restrict__ rowpos, int col_lo) {
     extern __shared__ int color_lds[];
     int* imb = color_lds;                                                        // [ncols] even minus odd labels per column
     int* wt = color_lds + ncols;                                                 // [ncols] weight of the column's balance
@@ -202,9 +203,10 @@ __global__ __launch_bounds__(256) void tile_color_kernel(const int32_t* __restri
     for (int i = threadIdx.x; i < ncols; i += 256) { imb[i] = 0; wt[i] = 0; }
     __syncthreads();
     for (int e = threadIdx.x; e < nl * K; e += 256) {
-        const int c = src[e];
-        ids[e] = (unsigned short)c;
-        atomicAdd(&wt[c], 1);                                                    // column lengths first
+        const unsigned c = (unsigned)(src[e] - col_lo);
+        const bool in = c < (unsigned)ncols;
+        ids[e] = in ? (unsigned short)c : (unsigned short)0xffffu;              // (ncols <= 1024)
+        if (in) atomicAdd(&wt[c], 1);                                            // column lengths first
     }
     __syncthreads();
     // Only the longest columns of a slice (64 columns, one wavefront of the walking kernel) set its number of slot
@@ -225,13 +227,13 @@ __global__ __launch_bounds__(256) void tile_color_kernel(const int32_t* __restri
     int placed[2] = {0, 0};
     for (int jl = 0; jl < nl; ++jl) {
         int sum = 0;
-        for (int k = lane; k < K; k += 64) { const int c = ids[jl * K + k]; sum += wt[c] * imb[c]; }
+        for (int k = lane; k < K; k += 64) { const int c = ids[jl * K + k]; if (c < ncols) sum += wt[c] * imb[c]; }
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
         int color = sum > 0 ? 1 : (sum < 0 ? 0 : (placed[1] < placed[0] ? 1 : 0));
         if (placed[color] >= cap) color ^= 1;
         const int delta = color ? -1 : 1;
-        for (int k = lane; k < K; k += 64) atomicAdd(&imb[ids[jl * K + k]], delta);     // a column may occur twice in a label
+        for (int k = lane; k < K; k += 64) { const int c = ids[jl * K + k]; if (c < ncols) atomicAdd(&imb[c], delta); }   // a column may occur twice in a label
         if (lane == 0) half[jl] = (unsigned char)color;
         ++placed[color];
     }
@@ -241,15 +243,15 @@ __global__ __launch_bounds__(256) void tile_color_kernel(const int32_t* __restri
     for (int jl = 0; jl < nl; ++jl) {
         const int old = half[jl];                         // (written by lane 0 above; LDS accesses of a wavefront are in order)
         const int back = old ? 1 : -1;
-        for (int k = lane; k < K; k += 64) atomicAdd(&imb[ids[jl * K + k]], back);
+        for (int k = lane; k < K; k += 64) { const int c = ids[jl * K + k]; if (c < ncols) atomicAdd(&imb[c], back); }
         int sum = 0;
-        for (int k = lane; k < K; k += 64) { const int c = ids[jl * K + k]; sum += wt[c] * imb[c]; }
+        for (int k = lane; k < K; k += 64) { const int c = ids[jl * K + k]; if (c < ncols) sum += wt[c] * imb[c]; }
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
         int color = sum > 0 ? 1 : (sum < 0 ? 0 : old);
         if (color != old && placed[color] >= cap) color = old;
         const int delta = color ? -1 : 1;
-        for (int k = lane; k < K; k += 64) atomicAdd(&imb[ids[jl * K + k]], delta);
+        for (int k = lane; k < K; k += 64) { const int c = ids[jl * K + k]; if (c < ncols) atomicAdd(&imb[c], delta); }
         if (color != old) { --placed[old]; ++placed[color]; if (lane == 0) half[jl] = (unsigned char)color; }
     }
     // rows of a half are handed out in ascending label order
@@ -267,7 +269,7 @@ __global__ __launch_bounds__(256) void tile_color_kernel(const int32_t* __restri
 // and bank half of the label's row (integer LDS atomics: order-independent), stores the slot count of the
 // longest column of each slice.
 __global__ void tile_count_kernel(const int32_t* __restrict__ idx, const unsigned short* __restrict__ rowpos, int L, int K,
-                                  int tile_labels, unsigned* __restrict__ slice_len) {
+                                  int tile_labels, unsigned* __restrict__ slice_len, int col_lo) {
     extern __shared__ unsigned cnt[];          // [2][threads]: labels in even rows, labels in odd rows
     const int t = blockIdx.x, nthreads = blockDim.x;
     cnt[threadIdx.x] = 0;
@@ -277,8 +279,10 @@ __global__ void tile_count_kernel(const int32_t* __restrict__ idx, const unsigne
     const int nl = min(tile_labels, L - j0);
     const int* src = idx + (size_t)j0 * K;
     const int total = nl * K;
-    for (int e = threadIdx.x; e < total; e += nthreads)
-        atomicAdd(&cnt[(rowpos[j0 + e / K] & 1u) * nthreads + (unsigned)src[e]], 1u);
+    for (int e = threadIdx.x; e < total; e += nthreads) {
+        const unsigned c = (unsigned)(src[e] - col_lo);
+        if (c < (unsigned)nthreads) atomicAdd(&cnt[(rowpos[j0 + e / K] & 1u) * nthreads + c], 1u);
+    }
     __syncthreads();
     const unsigned even = cnt[threadIdx.x], odd = cnt[nthreads + threadIdx.x];
     unsigned c = column_slots(threadIdx.x, even, odd);
@@ -321,7 +325,7 @@ constexpr int kFillChunk = 8192;
 __global__ void tile_fill_kernel(const int32_t* __restrict__ idx, const unsigned short* __restrict__ rowpos, int L, int K,
                                  int tile_labels, int zero_row, const unsigned* __restrict__ slice_off,
                                  unsigned short* __restrict__ lab16, unsigned short* __restrict__ pos16, unsigned pad_pos,
-                                 unsigned* __restrict__ slot32) {
+                                 unsigned* __restrict__ slot32, int col_lo) {
     __shared__ __align__(16) int keys[kFillChunk];
     __shared__ unsigned short rows_of[kPlanTileLabels];     // LDS row of each label of the tile
     const int t = blockIdx.x, nthreads = blockDim.x;
@@ -329,7 +333,7 @@ __global__ void tile_fill_kernel(const int32_t* __restrict__ idx, const unsigned
     const int nl = min(tile_labels, L - j0);
     const int* src = idx + (size_t)j0 * K;
     const int total = nl * K;
-    const int mine = threadIdx.x;
+    const int mine = (int)threadIdx.x + col_lo;
     const size_t sl = (size_t)t * (nthreads >> 6) + (threadIdx.x >> 6);
     const size_t row0 = slice_off[sl];
     const unsigned rows = slice_off[sl + 1] - slice_off[sl];
@@ -377,7 +381,7 @@ __global__ void tile_fill_kernel(const int32_t* __restrict__ idx, const unsigned
 __global__ void tile_fill_bitmap_kernel(const int32_t* __restrict__ idx, const unsigned short* __restrict__ rowpos, int L, int K,
                                         int tile_labels, int zero_row, const unsigned* __restrict__ slice_off,
                                         unsigned short* __restrict__ lab16, unsigned short* __restrict__ pos16, unsigned pad_pos,
-                                        unsigned* __restrict__ slot32, int words) {
+                                        unsigned* __restrict__ slot32, int words, int col_lo) {
     extern __shared__ __align__(16) unsigned fill_lds[];
     const int t = blockIdx.x, nthreads = blockDim.x;
     unsigned* bm = fill_lds;                                                   // [nthreads][words] (words odd: no bank conflicts)
@@ -395,7 +399,10 @@ __global__ void tile_fill_bitmap_kernel(const int32_t* __restrict__ idx, const u
     for (int i = threadIdx.x; i < nthreads * words; i += nthreads) bm[i] = 0u;
     for (int i = threadIdx.x; i < words; i += nthreads) pm[i] = 0u;
     for (int i = threadIdx.x; i < nl; i += nthreads) rows_of[i] = rowpos[j0 + i];
-    for (int e = threadIdx.x; e < total; e += nthreads) ids[e] = (unsigned short)src[e];
+    for (int e = threadIdx.x; e < total; e += nthreads) {
+        const unsigned c = (unsigned)(src[e] - col_lo);                       // (columns outside the plan's window: never matched)
+        ids[e] = c < (unsigned)nthreads ? (unsigned short)c : (unsigned short)0xffffu;
+    }
     __syncthreads();
     for (int i = threadIdx.x; i < nl; i += nthreads)
         if (rows_of[i] & 1u) atomicOr(&pm[i >> 5], 1u << (i & 31));
@@ -534,7 +541,16 @@ int bits_for(unsigned max_value) {
 }
 
 // Detaches the arrays from the plan.  keep == true (a rebuild follows): their buffers go to the spare list.
+void free_spares(ffi_plan* p);
 void free_arrays(ffi_plan* p, bool keep = false) {
+    if (p->upper != nullptr) {
+        // (the second column window's arrays: freed, never kept -- inputs that wide are rare and their plans small)
+        free_arrays(p->upper, false);
+        free_spares(p->upper);
+        delete p->upper;
+        p->upper = nullptr;
+    }
+    p->col_lo = 0; p->col_n = 0;
     for (const ffi_plan::Buffer& b : p->owned) {
         if (keep) p->spare.push_back(b);
         else (void)hipFree(b.ptr);
@@ -658,13 +674,14 @@ namespace {
 // three times the connection count (heavily skewed column usage): the caller then builds the
 // global form instead.
 int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
-    const int threads = ((p->N + 63) / 64) * 64;
+    const int cols = p->col_n ? p->col_n : p->N;           // the columns this plan's tiled form covers, from col_lo on
+    const int threads = ((cols + 63) / 64) * 64;
     // every thread of the kernel that walks the plan stages at most two labels of a tile (one when
     // the workgroup is larger than 768 threads and registers are scarcer)
     // (even, so that label parity inside a tile is the parity of the LDS row)
     // and small enough for the positions inside a tile to fit 16 bits
     bool w_in_lds = false;
-    const int TL = plan_tile_labels(p->N, p->K, p->L, p->batch_hint, &w_in_lds);
+    const int TL = plan_tile_labels(cols, p->K, p->L, p->batch_hint, &w_in_lds);
     const int slices = threads / 64;
     const int tiles = (p->L + TL - 1) / TL;
     const size_t nslices = (size_t)tiles * slices;
@@ -677,10 +694,10 @@ int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
         const size_t lds = 2 * (size_t)threads * sizeof(int) + (size_t)TL * p->K * sizeof(unsigned short) + (size_t)TL;
         hipError_t ea = hipFuncSetAttribute((const void*)tile_color_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (ea != hipSuccess) return hip_fail(ea);
-        hipLaunchKernelGGL(tile_color_kernel, dim3(tiles), dim3(256), lds, s, lookup, p->L, p->K, TL, cap, threads, p->rowpos);
+        hipLaunchKernelGGL(tile_color_kernel, dim3(tiles), dim3(256), lds, s, lookup, p->L, p->K, TL, cap, threads, p->rowpos, p->col_lo);
     }
     hipLaunchKernelGGL(tile_count_kernel, dim3(tiles), dim3(threads), 2 * threads * sizeof(unsigned), s, lookup, p->rowpos, p->L,
-                       p->K, TL, slice_len);
+                       p->K, TL, slice_len, p->col_lo);
     hipLaunchKernelGGL(slice_scan_kernel, dim3(1), dim3(1024), 0, s, slice_len, p->slice_off, (int)nslices,
                        p->d_scratch + 2);
     hipError_t e = hipGetLastError();
@@ -690,8 +707,10 @@ int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     if (e != hipSuccess) return hip_fail(e);
     const unsigned long long rows = p->h_scratch[2];
     const unsigned long long connections = (unsigned long long)p->L * p->K;
-    // too skewed, or beyond what the walking kernel's 32-bit buffer offsets reach (256 bytes per row)
-    if (rows * 64ull > 3ull * connections + 64ull * nslices || rows >= (1ull << 24)) return FFI_OK;
+    // too skewed (a window of the columns may have two slots per connection of the layer: how many of them fall into
+    // it is not counted), or beyond what the walking kernel's 32-bit buffer offsets reach (256 bytes per row)
+    const unsigned long long allowed = p->col_n ? 2ull : 3ull;
+    if (rows * 64ull > allowed * connections + 64ull * nslices || rows >= (1ull << 24)) return FFI_OK;
     if (w_in_lds) {
         if (!dev_alloc(p, &p->slot32, (size_t)rows * 64)) return FFI_ERR_OUT_OF_MEMORY;
     } else if (!dev_alloc(p, &p->lab16, (size_t)rows * 64) || !dev_alloc(p, &p->pos16, (size_t)rows * 64)) {
@@ -705,10 +724,10 @@ int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
             hipError_t ea = hipFuncSetAttribute((const void*)tile_fill_bitmap_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)fill_lds);
             if (ea != hipSuccess) return hip_fail(ea);
             hipLaunchKernelGGL(tile_fill_bitmap_kernel, dim3(tiles), dim3(threads), fill_lds, s, lookup, p->rowpos, p->L, p->K, TL, 2 * cap,
-                               p->slice_off, p->lab16, p->pos16, pad_pos, p->slot32, words);
+                               p->slice_off, p->lab16, p->pos16, pad_pos, p->slot32, words, p->col_lo);
         } else {
             hipLaunchKernelGGL(tile_fill_kernel, dim3(tiles), dim3(threads), 0, s, lookup, p->rowpos, p->L, p->K, TL, 2 * cap, p->slice_off,
-                               p->lab16, p->pos16, pad_pos, p->slot32);
+                               p->lab16, p->pos16, pad_pos, p->slot32, p->col_lo);
         }
     }
     e = hipGetLastError();
@@ -1027,6 +1046,35 @@ int plan_build_arrays(ffi_plan* p, const int32_t* lookup, hipStream_t s, unsigne
     if (p->N <= 1024 && p->K <= 1024 && p->L < (1 << 25)) {
         int st = build_tiled(p, lookup, s);
         if (st != FFI_OK) { (void)join(); free_arrays(p); return st; }
+    } else if (tile_path_fits(p->N) && p->N <= 2048 && p->K <= 1024 && p->L < (1 << 25)) {
+        // 1,025 to 1,216 columns: the LDS tile of the other two passes holds them, a workgroup of one thread per column
+        // does not.  Two tiled forms, one per half of the columns; each walk stages the tile's out_grad itself, which costs
+        // far less than the cache-bound global form (measured at 1,216 columns, c2's other dimensions: 1.58 ms).
+        const int lower = ((p->N + 1) / 2 + 63) / 64 * 64;
+        p->col_lo = 0; p->col_n = lower;
+        int st = build_tiled(p, lookup, s);
+        if (st == FFI_OK && p->tiled) {
+            ffi_plan* u = new (std::nothrow) ffi_plan();
+            if (u == nullptr) st = FFI_ERR_OUT_OF_MEMORY;
+            else {
+                u->device = p->device; u->L = p->L; u->K = p->K; u->N = p->N; u->batch_hint = p->batch_hint;
+                u->col_lo = lower; u->col_n = p->N - lower;
+                u->d_scratch = p->d_scratch; u->h_scratch = p->h_scratch;      // (borrowed for the build; never freed through `u`)
+                p->upper = u;
+                st = build_tiled(u, lookup, s);
+                u->d_scratch = nullptr; u->h_scratch = nullptr;
+                if (st == FFI_OK && u->tiled) p->bytes += u->bytes;
+            }
+        }
+        if (st != FFI_OK) { (void)join(); free_arrays(p); return st; }
+        if (!p->tiled || !p->upper || !p->upper->tiled) {
+            // too skewed for the tiled form in one of the halves: both go, the global form serves all columns
+            ffi_plan* u = p->upper;
+            p->upper = nullptr;
+            if (u) { free_arrays(u, false); free_spares(u); delete u; }
+            p->tiled = false;
+            p->col_lo = 0; p->col_n = 0;
+        }
     }
     if (!p->tiled) {
         // (the tiled form's arrays, if any were made, go back to the spare list; the arranged ids stay)

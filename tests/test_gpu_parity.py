@@ -134,12 +134,12 @@ def test_layouts_agree(ffi, shape):
 # shapes that steer the library through each of its code paths:
 #   narrow inputs (LDS tile kernels), wide inputs (generic kernels), the tiled and the global plan,
 #   partly filled batch tiles, fan-ins below / across / beyond the 32-connection register chunk,
-#   fewer labels than one tile, more than 1024 columns (global plan with tile forward/weight-grad),
+#   fewer labels than one tile, more than 1024 columns (one tiled plan per half of the columns, tile forward/weight-grad),
 #   the forward kernel over batch tiles of 64
 PATH_SHAPES = [
     (300, 700, 5000, 32),      # 10 batch tiles, the last one partly filled
     (33, 96, 9, 5),            # fewer labels than lanes, odd fan-in
-    (64, 1100, 3000, 12),      # N > 1024: tile forward / weight-grad, global plan
+    (64, 1100, 3000, 12),      # N > 1024: tile forward / weight-grad, a tiled plan for each half of the columns
     (40, 1216, 2500, 36),      # largest N that still fits the LDS tile
     (48, 1300, 2000, 20),      # wide: generic kernels, one batch entry per lane, rows padded to 128 bytes
     (64, 1400, 700, 16),       # wide, rows already aligned: [N,B] features used in place
@@ -306,6 +306,58 @@ def test_skewed_lookup_uses_the_global_plan(ffi):
     assert np.array_equal(gx[:, [0, 1, 2, 4, 149, 151]], np.zeros((B, 6), dtype=np.float32))
     assert rel_err(gw, oracle.weight_grad(x, lookup, w, g)) <= GRAD_RTOL
     assert rel_err(hip_forward(ffi, x, lookup, w, False), oracle.forward(x, lookup, w)) <= FWD_RTOL
+
+
+@pytest.mark.parametrize("case", ["uniform", "upper_half_unused", "lower_half_skewed", "upper_half_skewed", "rewired"])
+def test_inputs_of_more_than_1024_columns_take_one_plan_per_half(ffi, case):
+    # 1,025 to 1,216 columns: the input gradient walks two tiled plans, one per half of the columns (a workgroup has at
+    # most 1,024 threads, one per column).  Either half may be unused, or too skewed for the tiled form (then the global
+    # column order serves all columns), and a lookup edited in place must be noticed for both.
+    B, N, L, K = 70, 1100, 5000, 16
+    x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=55)
+    split = ((N + 1) // 2 + 63) // 64 * 64
+    if case == "upper_half_unused":
+        lookup = (lookup % split).astype(np.int32)
+    elif case == "lower_half_skewed":
+        lookup = np.where(lookup < split, 7, lookup).astype(np.int32)
+    elif case == "upper_half_skewed":
+        lookup = np.where(lookup >= split, N - 1, lookup).astype(np.int32)
+    lib = ffi._lib.lib()
+    dx, dl, dw, dg = dev(x), dev(lookup), dev(w), dev(g)
+    plan = ctypes.c_void_p()
+    ffi._lib.check(lib.ffi_plan_create(dl.data_ptr(), L, K, N, B, stream(), ctypes.byref(plan)))
+    info = (ctypes.c_int64 * 8)()
+    ffi._lib.check(lib.ffi_plan_info(plan, info))
+    assert info[0] == (0 if case.endswith("skewed") else 1)
+    gx = torch.full_like(dx, float("nan"))
+    ffi._lib.check(lib.ffi_input_grad_planned_f32(plan, dw.data_ptr(), dg.data_ptr(), gx.data_ptr(), B, 0, stream()))
+    torch.cuda.synchronize()
+    ffi._lib.check(lib.ffi_plan_destroy(plan))
+    assert rel_err(gx.cpu().numpy(), oracle.input_grad(x, lookup, w, g)) <= GRAD_RTOL
+    if case == "upper_half_unused":
+        assert not gx[:, split:].any()
+    # the cached route, both layouts; then an edit of the lookup in place that moves connections between the halves
+    for transposed in (False, True):
+        xin = np.ascontiguousarray(x.T) if transposed else x
+        got_gx, got_gw = hip_backward(ffi, xin, lookup, w, g, transposed)
+        o_gx, o_gw = oracle.backward(xin, lookup, w, g, transposed=transposed)
+        assert rel_err(got_gx, o_gx) <= GRAD_RTOL and rel_err(got_gw, o_gw) <= GRAD_RTOL
+    if case == "rewired":
+        gx2 = torch.empty_like(dx)
+
+        def run():
+            ffi._lib.check(lib.ffi_input_grad_f32(dl.data_ptr(), dw.data_ptr(), dg.data_ptr(), gx2.data_ptr(), B, N, L, K, 0, stream()))
+            torch.cuda.synchronize()
+            return gx2.cpu().numpy().copy()
+
+        assert rel_err(run(), oracle.input_grad(x, lookup, w, g)) <= GRAD_RTOL
+        rng = np.random.default_rng(8)
+        lookup2 = lookup.copy()
+        lookup2[rng.integers(0, L, 700), rng.integers(0, K, 700)] = rng.integers(0, N, 700)
+        dl.copy_(dev(lookup2))
+        for _ in range(3):                                   # recomputed from the lookup, then from the rebuilt plans
+            assert rel_err(run(), oracle.input_grad(x, lookup2, w, g)) <= GRAD_RTOL
+        assert np.array_equal(run(), run())
 
 
 def test_unaligned_buffers(ffi):
