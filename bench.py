@@ -152,7 +152,7 @@ def rewire_costs(pkg, cfg, x, lookup, w, g, tp, stream):
            "second_backward_after_rewire_ms": {"library_rewire": round(after_library, 4), "foreign_in_place_edit": round(second_foreign, 4)},
            "third_backward_after_foreign_edit_ms": round(after_foreign, 4),
            "note": "library route: ffi_rewire_f32 marks the cached plan outdated, the next backward rebuilds it and runs the plan-driven kernels; "
-                   "foreign route: the first backward runs the kernels that read the lookup directly (float atomics), the second rebuilds"}
+                   "foreign route: the first backward runs the kernels that read the lookup directly (the input gradient sorts every label tile by column on the fly), the second rebuilds"}
     extra_library = rewire_ms + first_library - normal
     extra_foreign = (first_foreign - normal) + (second_foreign - normal)
     out["amortised_ms_per_step"] = {f"rewire_interval_{i}": {"library_rewire": round(extra_library / i, 5), "foreign_in_place_edit": round(extra_foreign / i, 5)}

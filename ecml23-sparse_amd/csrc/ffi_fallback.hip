@@ -5,7 +5,8 @@
 // tfsparse/cc/kernels/backward.cpp:8-36 (weight gradient) and :39-73 (input gradient); the input gradient scatters
 // with float atomics here, as the reference's GPU kernels do (backward.cu.h:119,139,161,182), so this one call is
 // not reproducible bit for bit.  Ids outside [0, num_features) are skipped.  Narrow inputs take the weight-gradient kernel
-// that reads the lookup itself and an input-gradient kernel that sums in LDS (float atomics there too).
+// that reads the lookup itself and an input-gradient kernel that sorts each label tile's connections by column in LDS
+// (ffi_input_grad.hip; float atomics only where the workgroups add their sums to gx).
 #include "ffi_internal.h"
 #include "ffi_lds_tile.h"
 
@@ -51,43 +52,6 @@ __global__ __launch_bounds__(kFbBlock) void fallback_backward_kernel(const unsig
     }
 }
 
-// Narrow inputs: the input gradient of one batch tile (32 samples) and a range of labels summed in LDS -- acc[b][n],
-// so that the lanes of a wavefront (one label each) spread over the banks by their column ids -- and added to gx with
-// one global atomic per (column, sample) and workgroup.  At 670,091 labels x fan-in 32, batch 128, this takes the
-// place of 2.7 G global float atomics onto 98,304 addresses (138 ms) with as many LDS atomics (about a tenth of that).
-constexpr int kFbLdsThreads = 1024;
-template <bool TP>
-__global__ __launch_bounds__(kFbLdsThreads) void fallback_input_grad_lds_kernel(const unsigned long long* __restrict__ verdict,
-                                                                                const int32_t* __restrict__ idx, const float* __restrict__ w,
-                                                                                const float* __restrict__ g, float* __restrict__ gx, int B,
-                                                                                int N, int L, int K, int labels_per_block) {
-    if (*verdict != 0) return;
-    extern __shared__ float fb_acc[];                     // [32][N]
-    const int b0 = blockIdx.y * kTileBatch;
-    const int j_begin = blockIdx.x * labels_per_block, j_end = min(j_begin + labels_per_block, L);
-    for (int i = threadIdx.x; i < kTileBatch * N; i += kFbLdsThreads) fb_acc[i] = 0.f;
-    __syncthreads();
-    for (int j = j_begin + (int)threadIdx.x; j < j_end; j += kFbLdsThreads) {
-        float gb[32];
-        load_rows32(g, L, b0, B, (unsigned)j, gb);
-        const int32_t* irow = idx + (size_t)j * K;
-        const float* wrow = w + (size_t)j * K;
-        for (int k = 0; k < K; ++k) {
-            const unsigned id = (unsigned)irow[k];
-            const float wv = wrow[k];
-            if (id < (unsigned)N) {
-#pragma unroll
-                for (int b = 0; b < 32; ++b) atomicAdd(&fb_acc[b * N + (int)id], wv * gb[b]);
-            }
-        }
-    }
-    __syncthreads();
-    for (int i = threadIdx.x; i < kTileBatch * N; i += kFbLdsThreads) {
-        const int b = i / N, n = i - b * N;
-        if (b0 + b < B) atomicAdd(&gx[TP ? (size_t)n * B + (b0 + b) : (size_t)(b0 + b) * N + n], fb_acc[i]);
-    }
-}
-
 }  // namespace
 
 int launch_backward_if_outdated(const unsigned long long* verdict, const float* features, const int32_t* lookup,
@@ -100,27 +64,11 @@ int launch_backward_if_outdated(const unsigned long long* verdict, const float* 
     }
     float* gw = features != nullptr ? weight_grad : nullptr;
     float* gb = features != nullptr ? bias_grad : nullptr;
-    if (tile_path_fits(d.N) && d.L < (1 << 25)) {
+    if (tile_path_fits(d.N) && d.L < (1 << 25) && input_grad_unplanned_fits(d.N, d.K)) {
         // narrow inputs: the weight gradient by the kernel that needs no plan (it returns at once unless the verdict says
-        // "outdated"), the input gradient through LDS
+        // "outdated"), the input gradient by the kernel that sorts each label tile's connections by column in LDS
         if (gw != nullptr) FFI_TRY(launch_weight_grad(features, lookup, out_grad, gw, gb, d, s, nullptr, verdict));
-        if (feature_grad != nullptr) {
-            const int nbt = (d.B + kTileBatch - 1) / kTileBatch;
-            const int per_tile = std::max(1, 4 * cus / nbt);
-            const int lpb = std::max(kFbLdsThreads, (d.L + per_tile - 1) / per_tile);
-            const dim3 grid((unsigned)((d.L + lpb - 1) / lpb), (unsigned)nbt);
-            const size_t lds = tile_lds_bytes(d.N);
-            if (d.tp) {
-                FFI_HIP_TRY(hipFuncSetAttribute((const void*)fallback_input_grad_lds_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-                hipLaunchKernelGGL(fallback_input_grad_lds_kernel<true>, grid, dim3(kFbLdsThreads), lds, s, verdict, lookup, weights, out_grad,
-                                   feature_grad, d.B, d.N, d.L, d.K, lpb);
-            } else {
-                FFI_HIP_TRY(hipFuncSetAttribute((const void*)fallback_input_grad_lds_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-                hipLaunchKernelGGL(fallback_input_grad_lds_kernel<false>, grid, dim3(kFbLdsThreads), lds, s, verdict, lookup, weights, out_grad,
-                                   feature_grad, d.B, d.N, d.L, d.K, lpb);
-            }
-            FFI_HIP_TRY(hipGetLastError());
-        }
+        if (feature_grad != nullptr) FFI_TRY(launch_input_grad_unplanned(verdict, lookup, weights, out_grad, feature_grad, d, s));
         return FFI_OK;
     }
     if (d.tp)

@@ -337,6 +337,11 @@ void plan_free(ffi_plan* p);
 // when it says the plan is outdated (*zeroed_if_outdated tells whether they could)
 int launch_input_grad(const ffi_plan* p, const float* w, const float* g, float* gx, int B, bool tp,
                       hipStream_t s, const unsigned long long* verdict = nullptr, bool* zeroed_if_outdated = nullptr);
+// The input gradient straight from the lookup (no plan), added into a zeroed gx by a kernel that runs only if *verdict == 0;
+// for inputs that fit the LDS tile and fan-ins whose tile of one label fits beside it (input_grad_unplanned_fits).
+bool input_grad_unplanned_fits(int N, int K);
+int launch_input_grad_unplanned(const unsigned long long* verdict, const int32_t* idx, const float* w, const float* g, float* gx,
+                                const Dims& d, hipStream_t s);
 int launch_input_grad_wide(const ffi_plan* p, const float* w, const float* g, float* gx, int B, bool tp, hipStream_t s);
 }  // namespace ffi
 

@@ -193,19 +193,20 @@ __device__ __forceinline__ unsigned column_slots(unsigned thread, unsigned even,
 __global__ __launch_bounds__(256) void tile_color_kernel(const int32_t* __restrict__ idx, int L, int K, int tile_labels, int cap,
                                                          int ncols, unsigned short* __restrict__ rowpos, int col_lo) {
     extern __shared__ int color_lds[];
-    int* imb = color_lds;                                                        // [ncols] even minus odd labels per column
-    int* wt = color_lds + ncols;                                                 // [ncols] weight of the column's balance
-    unsigned short* ids = reinterpret_cast<unsigned short*>(color_lds + 2 * ncols);  // [tile_labels * K] column ids
+    // (entry `ncols` of both: where connections into columns outside the window go -- weight 0, so they never count)
+    int* imb = color_lds;                                                        // [ncols + 1] even minus odd labels per column
+    int* wt = color_lds + ncols + 1;                                             // [ncols + 1] weight of the column's balance
+    unsigned short* ids = reinterpret_cast<unsigned short*>(color_lds + 2 * (ncols + 1));  // [tile_labels * K] column ids
     const int t = blockIdx.x;
     const int j0 = t * tile_labels;
     const int nl = min(tile_labels, L - j0);
     const int* src = idx + (size_t)j0 * K;
-    for (int i = threadIdx.x; i < ncols; i += 256) { imb[i] = 0; wt[i] = 0; }
+    for (int i = threadIdx.x; i <= ncols; i += 256) { imb[i] = 0; wt[i] = 0; }
     __syncthreads();
     for (int e = threadIdx.x; e < nl * K; e += 256) {
         const unsigned c = (unsigned)(src[e] - col_lo);
         const bool in = c < (unsigned)ncols;
-        ids[e] = in ? (unsigned short)c : (unsigned short)0xffffu;              // (ncols <= 1024)
+        ids[e] = in ? (unsigned short)c : (unsigned short)ncols;                // (ncols <= 1024)
         if (in) atomicAdd(&wt[c], 1);                                            // column lengths first
     }
     __syncthreads();
@@ -227,13 +228,13 @@ __global__ __launch_bounds__(256) void tile_color_kernel(const int32_t* __restri
     int placed[2] = {0, 0};
     for (int jl = 0; jl < nl; ++jl) {
         int sum = 0;
-        for (int k = lane; k < K; k += 64) { const int c = ids[jl * K + k]; if (c < ncols) sum += wt[c] * imb[c]; }
+        for (int k = lane; k < K; k += 64) { const int c = ids[jl * K + k]; sum += wt[c] * imb[c]; }
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
         int color = sum > 0 ? 1 : (sum < 0 ? 0 : (placed[1] < placed[0] ? 1 : 0));
         if (placed[color] >= cap) color ^= 1;
         const int delta = color ? -1 : 1;
-        for (int k = lane; k < K; k += 64) { const int c = ids[jl * K + k]; if (c < ncols) atomicAdd(&imb[c], delta); }   // a column may occur twice in a label
+        for (int k = lane; k < K; k += 64) atomicAdd(&imb[ids[jl * K + k]], delta);   // a column may occur twice in a label
         if (lane == 0) half[jl] = (unsigned char)color;
         ++placed[color];
     }
@@ -243,15 +244,15 @@ __global__ __launch_bounds__(256) void tile_color_kernel(const int32_t* __restri
     for (int jl = 0; jl < nl; ++jl) {
         const int old = half[jl];                         // (written by lane 0 above; LDS accesses of a wavefront are in order)
         const int back = old ? 1 : -1;
-        for (int k = lane; k < K; k += 64) { const int c = ids[jl * K + k]; if (c < ncols) atomicAdd(&imb[c], back); }
+        for (int k = lane; k < K; k += 64) atomicAdd(&imb[ids[jl * K + k]], back);
         int sum = 0;
-        for (int k = lane; k < K; k += 64) { const int c = ids[jl * K + k]; if (c < ncols) sum += wt[c] * imb[c]; }
+        for (int k = lane; k < K; k += 64) { const int c = ids[jl * K + k]; sum += wt[c] * imb[c]; }
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
         int color = sum > 0 ? 1 : (sum < 0 ? 0 : old);
         if (color != old && placed[color] >= cap) color = old;
         const int delta = color ? -1 : 1;
-        for (int k = lane; k < K; k += 64) { const int c = ids[jl * K + k]; if (c < ncols) atomicAdd(&imb[c], delta); }
+        for (int k = lane; k < K; k += 64) atomicAdd(&imb[ids[jl * K + k]], delta);
         if (color != old) { --placed[old]; ++placed[color]; if (lane == 0) half[jl] = (unsigned char)color; }
     }
     // rows of a half are handed out in ascending label order
@@ -691,7 +692,7 @@ int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     const int cap = tiled_rows_per_half(TL);
     if (!dev_alloc(p, &p->rowpos, (size_t)p->L)) return FFI_ERR_OUT_OF_MEMORY;
     {
-        const size_t lds = 2 * (size_t)threads * sizeof(int) + (size_t)TL * p->K * sizeof(unsigned short) + (size_t)TL;
+        const size_t lds = 2 * ((size_t)threads + 1) * sizeof(int) + (size_t)TL * p->K * sizeof(unsigned short) + (size_t)TL;
         hipError_t ea = hipFuncSetAttribute((const void*)tile_color_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (ea != hipSuccess) return hip_fail(ea);
         hipLaunchKernelGGL(tile_color_kernel, dim3(tiles), dim3(256), lds, s, lookup, p->L, p->K, TL, cap, threads, p->rowpos, p->col_lo);

@@ -110,8 +110,8 @@ int ffi_forward_noalloc_f32(const float* features, const int32_t* lookup, const 
  *   - edits by foreign code are caught by a content fingerprint that a kernel re-checks on every call, on the
  *     device, without a host wait: every call enqueued before the host has seen the verdict -- the first call after
  *     the edit and as many more as the host runs ahead of the GPU -- computes correct results by kernels that read
- *     the lookup directly (one thread per connection, float atomics for the input gradient: much slower, about
- *     20 ms at that size, and with the atomics' summation order); the first call made after the verdict has reached
+ *     the lookup directly (the input gradient sorts each label tile's connections by column on the fly: about
+ *     2 ms at that size instead of 0.5, and its sums are not reproducible bit for bit); the first call made after the verdict has reached
  *     the host rebuilds the view.  Callers that edit the lookup themselves and care should hold an explicit plan
  *     (ffi_plan_create / ffi_plan_refresh) or call ffi_arrange_connections_f32 afterwards.
  */

@@ -424,10 +424,16 @@ def test_input_grad_is_deterministic_and_zero_on_untouched_columns(ffi):
     assert rel_err(gx1, oracle.input_grad(x, lookup, w, g)) <= GRAD_RTOL
 
 
-def test_in_place_rewiring_is_picked_up(ffi):
+@pytest.mark.parametrize("shape", [(32, 128, 3000, 16),
+                                   (100, 768, 9000, 32),      # several label streams, a partly filled batch tile
+                                   (20, 300, 900, 300),       # the recomputing kernel's tiles hold 64 labels
+                                   (8, 64, 40, 5000),         # ... 4 labels
+                                   (4, 64, 6, 25000),         # a label's connections alone exceed the LDS: one thread per connection
+                                   (40, 2000, 700, 12)])      # wide input
+def test_in_place_rewiring_is_picked_up(ffi, shape):
     # the layer rewires by overwriting entries of the same index variable
     # (sparse/custom_layer.py:32-43): same pointer, new contents
-    B, N, L, K = 32, 128, 3000, 16
+    B, N, L, K = shape
     x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=31)
     dx, dl, dw, dg = dev(x), dev(lookup), dev(w), dev(g)
     gx = torch.empty_like(dx)
