@@ -616,6 +616,7 @@ int ffi_set_option(const char* name, int value) {
         {"fwd_lane64", &ffi::Options::fwd_lane64, -1, 0},
         {"plan_weights_in_lds", &ffi::Options::plan_weights_in_lds, -1, 1},
         {"workgroups_per_cu", &ffi::Options::workgroups_per_cu, 0, 16},
+        {"plan_sorted_columns", &ffi::Options::plan_sorted_columns, -1, 1},
     };
     for (const auto& t : table) {
         if (std::strcmp(name, t.name) != 0) continue;
@@ -665,9 +666,12 @@ size_t ffi_workspace_bytes(int64_t batch, int64_t num_features, int64_t num_unit
                 const size_t TL = (size_t)plan_tile_labels((int)cols, d.K, d.L, d.B, &w_in_lds);
                 const size_t tiles = (L + TL - 1) / TL, slices = threads / 64;
                 const double mu = (double)TL * (double)K / (double)N;
-                const size_t rows = (size_t)(mu + 2.6 * std::sqrt(mu) + 3.0);
+                // (plans that sort a tile's columns by length: a slice's rows are those of columns about equally long)
+                const bool sorted = plan_sorts_columns((int)threads, (int)TL, d.K, w_in_lds, (int)tiles, d.B);
+                const size_t rows = sorted ? (size_t)(mu + 0.75 * std::sqrt(mu) + 1.0) : (size_t)(mu + 2.6 * std::sqrt(mu) + 3.0);
                 const size_t slots = tiles * slices * rows * 64;
                 total += slots * 2 * 2 + (tiles * slices + 1) * 4 + L * 2;              // 4 bytes per slot (lab16 + pos16, or slot32), slice_off, rowpos
+                if (sorted) total += tiles * threads * 2;                               // the column of each thread in each tile
                 if (!w_in_lds) features_slot = std::max(features_slot, slots * 4);     // weights in slot order
                 const size_t nbt = (B + 31) / 32;
                 const size_t per_cu = (size_t)tiled_workgroups_per_cu((int)threads, (int)TL, d.K, w_in_lds, (int)((B + 31) / 32));

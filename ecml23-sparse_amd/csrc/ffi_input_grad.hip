@@ -127,13 +127,19 @@ __device__ __forceinline__ void igrad_fmas(const float4 (&v)[8], float wv, float
 // block of the weights << 17) | (LDS row << 7), in place of lab16:
 // the tile's weights are staged in LDS behind the rows of out_grad (with a zero word at tile_labels * K that
 // padding slots read) and every slot fetches its weight from there, so no slot-ordered copy of the weights exists.
-template <int MAXT, int LPT, bool WLDS>
+// PERM (with WLDS and LPT == 1): `colperm` names, per tile, the column each thread walks -- the plan sorts a tile's columns by
+// length so that the 64 columns of a wavefront are about equally long.  The thread's sums over one tile then belong to
+// another thread's column: after every tile they pass through LDS (the tile's rows and weights are dead by then; row n of
+// the exchange = column n, chunks skewed like every other row) to the column's own thread, which adds them to the
+// sums it keeps over the whole label stream.
+template <int MAXT, int LPT, bool WLDS, bool PERM = false>
 __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* __restrict__ lab16, const float* __restrict__ wp,
                                   const unsigned* __restrict__ slice_off,
                                   const float* __restrict__ g, float* __restrict__ partial, int B, int L,
                                   int tile_labels, int tiles, int tiles_per_stream, int nbt, unsigned total_rows,
                                   const unsigned short* __restrict__ rowpos, int zero_row,
-                                  const unsigned* __restrict__ slot32, int K) {
+                                  const unsigned* __restrict__ slot32, int K, const unsigned short* __restrict__ colperm = nullptr) {
+    static_assert(!PERM || (WLDS && LPT == 1), "the exchange of sums is built for the weights-in-LDS form");
     extern __shared__ __align__(16) float gs[];
     char* gs_bytes = reinterpret_cast<char*>(gs);
     const int nthreads = blockDim.x;
@@ -153,11 +159,37 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
     float* ws = gs + (size_t)(zero_row + 2) * kTileBatch;
     const unsigned wsbase = (unsigned)(size_t)(__attribute__((address_space(3))) float*)ws;
     const unsigned tile_w = (unsigned)tile_labels * (unsigned)K;       // floats of a full tile; index of the zero word
-    constexpr int kWRegs = 8;                                           // 16-byte pieces of the tile's weights a thread carries
+    constexpr int kWRegs = PERM ? 1 : 8;                                           // 16-byte pieces of the tile's weights a thread carries
 
     float acc[32];
 #pragma unroll
     for (int i = 0; i < 32; ++i) acc[i] = 0.f;
+    // (PERM) the sums of the thread's own column over the tiles so far; `acc` holds one tile's sums of whatever column
+    // the thread walks in it
+    float home[PERM ? 32 : 1];
+#pragma unroll
+    for (int i = 0; i < (PERM ? 32 : 1); ++i) home[i] = 0.f;
+    unsigned walked = 0;                                   // (PERM) the column of the tile just walked
+    // acc -> row `walked` of the exchange; a barrier; row threadIdx.x -> home.  Called between two barriers that keep
+    // the tile's rows from being read or written meanwhile.
+    auto hand_over = [&]() __attribute__((always_inline)) {
+        char* rowp = gs_bytes + ((size_t)walked << 7);
+        const int r = lane & 7;
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+            *reinterpret_cast<float4*>(rowp + ((c ^ r) << 4)) = make_float4(acc[4 * c], acc[4 * c + 1], acc[4 * c + 2], acc[4 * c + 3]);
+        __syncthreads();
+        const char* mine = gs_bytes + ((size_t)threadIdx.x << 7);
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const float4 v = *reinterpret_cast<const float4*>(mine + ((c ^ r) << 4));
+            // (group c of `home`, like group c of `acc`, holds batch entries 4 (c ^ r) ...: undone once, at the end)
+            home[PERM ? 4 * c : 0] += v.x; home[PERM ? 4 * c + 1 : 0] += v.y;
+            home[PERM ? 4 * c + 2 : 0] += v.z; home[PERM ? 4 * c + 3 : 0] += v.w;
+        }
+#pragma unroll
+        for (int i = 0; i < 32; ++i) acc[i] = 0.f;
+    };
 
     for (int t = t_begin; t < t_end; ++t) {
         const int j0 = t * tile_labels;
@@ -210,14 +242,41 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
         for (int r = 0; r < kWRegs; ++r) {
             const unsigned q = threadIdx.x + r * nthreads;
             wreg[r] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (WLDS && q < nw4) wreg[r] = reinterpret_cast<const float4*>(wt)[q];
+            if (WLDS && !PERM && q < nw4) wreg[r] = reinterpret_cast<const float4*>(wt)[q];
         }
+        unsigned next_walked = 0;
+        if (PERM) next_walked = colperm[(size_t)t * nthreads + threadIdx.x];
         __syncthreads();                       // the previous tile is no longer being read
+        // (PERM, 16-byte aligned weights) the tile's weights go from memory straight into LDS, a wavefront 1 KB per instruction
+        // -- the registers hold two sets of sums here, not a third of weights; pieces [from, to), waited for in front of the
+        // barrier that ends the staging
+        auto weights_to_lds = [&](unsigned from, unsigned to) __attribute__((always_inline)) {
+            const buffer_rsrc wr = make_rsrc(wt, (size_t)nw * sizeof(float));
+            for (unsigned i = from + (unsigned)__builtin_amdgcn_readfirstlane(wave); i < to; i += (unsigned)nthreads >> 6) {
+                if (i * 256u + (unsigned)lane * 4u < nw)
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(wr, (__attribute__((address_space(3))) float*)ws + (size_t)i * 256, 16,
+                                                             (unsigned)lane * 16u, i * 1024u, 0, 0);
+            }
+        };
+        const unsigned wpieces = (nw + 255u) / 256u;
+        if (PERM) {
+            if (t > t_begin) {
+                hand_over();
+                __syncthreads();               // the exchange has been read: the tile may be staged over it
+            }
+            // (requested only now that the exchange is over: asked for in front of it, the pieces that land behind the
+            // exchange's rows made the kernel 4 % slower)
+            if (wvec) weights_to_lds(0u, wpieces);
+            walked = next_walked;
+        }
         // rows `zero_row` (even) and `zero_row + 1` (odd) are all zero: the targets of padding slots
-        if (t == t_begin && threadIdx.x < 64) gs[zero_row * kTileBatch + threadIdx.x] = 0.f;
+        // (PERM: the exchange overwrites them after every tile)
+        if ((PERM || t == t_begin) && threadIdx.x < 64) gs[zero_row * kTileBatch + threadIdx.x] = 0.f;
         if (WLDS) {
-            if (t == t_begin && threadIdx.x == 0) ws[tile_w] = 0.f;
-            if (wvec) {
+            if ((PERM || t == t_begin) && threadIdx.x == 0) ws[tile_w] = 0.f;
+            if (wvec && PERM) {
+                // (requested above)
+            } else if (wvec) {
 #pragma unroll
                 for (int r = 0; r < kWRegs; ++r) {
                     const unsigned q = threadIdx.x + r * nthreads;
@@ -246,6 +305,7 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
                         make_float4(gbn[p][4 * c], gbn[p][4 * c + 1], gbn[p][4 * c + 2], gbn[p][4 * c + 3]);
             }
         }
+        if (PERM) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // the weights have arrived in LDS
         __syncthreads();
         if (rows == 0) continue;               // wave-uniform: no column of this slice is used in the tile
         for (unsigned i = 0; i < rows; i += kAhead) {
@@ -284,6 +344,12 @@ __global__ __launch_bounds__(MAXT) void igrad_tile_kernel(const unsigned short* 
 #pragma unroll
             for (int q = 0; q < kAhead; ++q) { e4[q] = en[q]; w4[q] = wn[q]; }
         }
+    }
+    if (PERM) {
+        __syncthreads();                       // the last tile is no longer being read
+        if (t_begin < t_end) hand_over();
+#pragma unroll
+        for (int i = 0; i < 32; ++i) acc[i] = home[PERM ? i : 0];
     }
     // back to natural batch order, then one 128-byte row per thread
     xor_permute_groups(acc, lane & 7);
@@ -359,7 +425,15 @@ int launch_tiled(const ffi_plan* p, const float* w, const float* g, float* gx, i
     if (p->w_in_lds) {
         // (plans take that form only with workgroups of at most 768 threads that stage one label each)
         if (p->threads > 768 || p->tile_labels > p->threads) return FFI_ERR_BAD_ARGUMENT;
-        FFI_LAUNCH_TILE(768, 1, true);
+        if (p->colperm != nullptr) {
+            // (the exchange of sums between the threads takes a 128-byte row per thread, wherever the tile ends)
+            const size_t lds_x = std::max(lds, (size_t)p->threads * kTileBatch * sizeof(float));
+            FFI_HIP_TRY(hipFuncSetAttribute((const void*)igrad_tile_kernel<768, 1, true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_x));
+            hipLaunchKernelGGL((igrad_tile_kernel<768, 1, true, true>), grid, block, lds_x, s, p->lab16, w, p->slice_off, g, partial, B, p->L,
+                               p->tile_labels, p->tiles, tps, nbt, (unsigned)p->total_rows, p->rowpos, p->zero_row, p->slot32, p->K, p->colperm);
+        } else {
+            FFI_LAUNCH_TILE(768, 1, true);
+        }
     } else if (per_cu > 1) {
         FFI_LAUNCH_TILE(1024, 1, false);                 // (the instantiation of at most 128 registers)
     } else if (p->threads <= 768) {

@@ -30,6 +30,7 @@ struct Options {
     int fwd_lane64 = 0;             // -1: never the 64-sample forward kernel
     int plan_weights_in_lds = 0;    // -1: never / 1: whenever the tile fits
     int workgroups_per_cu = 0;      // upper limit for the kernel that walks a tiled plan
+    int plan_sorted_columns = 0;    // -1: never / 1: always (in the weights-in-LDS form) the plans that hand the columns to the walking kernel's threads tile by tile, by length
 };
 extern Options g_options;
 
@@ -225,6 +226,10 @@ struct ffi_plan {
                                          // padding slots hold zero_row + parity (two all-zero rows)
     unsigned short* rowpos = nullptr;    // [L] LDS row each label is staged into, inside its tile (see ffi_plan.hip)
     int zero_row = 0;                    // first of the two all-zero rows = rows of the tile in LDS before them
+    // plans whose columns are handed to the walking kernel's threads anew in every tile, longest first (so that the 64
+    // columns a wavefront walks together are about equally long): [tiles * threads] the column of each thread, a
+    // permutation of 0 ... threads - 1 per tile; null in plans whose thread t always walks column t
+    unsigned short* colperm = nullptr;
     unsigned* slot32 = nullptr;          // plans with w_in_lds, instead of lab16 and pos16: [total_rows*64] (position << 17) | (LDS row << 7)
     unsigned short* pos16 = nullptr;     // [total_rows*64] position (inside the tile's rows of lookup) of each slot;
                                          // kPadPos in padding slots
@@ -300,6 +305,16 @@ inline int tiled_workgroups_per_cu(int threads, int tile_labels, int K, bool wit
     int n = by_lds < by_waves ? by_lds : by_waves;
     if (g_options.workgroups_per_cu > 0 && n > g_options.workgroups_per_cu) n = g_options.workgroups_per_cu;
     return n < 1 ? 1 : n;
+}
+// Whether a tiled plan hands its columns to the walking kernel's threads tile by tile, sorted by length (ffi_plan.hip,
+// tile_perm_kernel): the weights-in-LDS form with six or more slices, where every workgroup walks two tiles or more.
+inline bool plan_sorts_columns(int threads, int tile_labels, int K, bool weights_in_lds, int tiles, int batch_hint) {
+    if (!weights_in_lds || g_options.plan_sorted_columns < 0) return false;
+    if (g_options.plan_sorted_columns > 0) return true;                 // (tests: whenever the form allows)
+    if (threads < 384) return false;
+    const int nbt = batch_hint > 32 ? (batch_hint + 31) / 32 : 1;
+    const int per_stream = tiled_workgroups_per_cu(threads, tile_labels, K, true, nbt) * device_cu_count() / nbt;
+    return tiles >= 2 * (per_stream > 1 ? per_stream : 1);
 }
 constexpr int kArrIdBits = 11;            // column-id field of an arranged entry (narrow inputs: ids < 1216)
 // 16-bit word at which quarter t (entries 8 t ... 8 t + 7) of unit u starts in ffi_plan::idx16: units in blocks of 64, a

@@ -190,8 +190,11 @@ __device__ __forceinline__ unsigned column_slots(unsigned thread, unsigned even,
 // Rows of a half are handed out in ascending order, at most `cap` per half.  One workgroup per tile; the tile's
 // column ids are staged in LDS, one wavefront then decides label after label (lane <-> connection).
 // (`col_lo`: the plan covers the columns [col_lo, col_lo + ncols) only; connections into other columns are left out)
+// (`all_columns_count`: plans that hand the columns to threads by length -- there every column is about as long as the
+// longest of its slice, so every column's balance weighs the same)
 __global__ __launch_bounds__(256) void tile_color_kernel(const int32_t* __restrict__ idx, int L, int K, int tile_labels, int cap,
-                                                         int ncols, unsigned short* __restrict__ rowpos, int col_lo) {
+                                                         int ncols, unsigned short* __restrict__ rowpos, int col_lo,
+                                                         int all_columns_count) {
     extern __shared__ int color_lds[];
     // (entry `ncols` of both: where connections into columns outside the window go -- weight 0, so they never count)
     int* imb = color_lds;                                                        // [ncols + 1] even minus odd labels per column
@@ -219,7 +222,7 @@ __global__ __launch_bounds__(256) void tile_color_kernel(const int32_t* __restri
         for (int off = 32; off > 0; off >>= 1) longest = max(longest, __shfl_xor(longest, off, 64));
         float r = longest > 0 ? (float)len / (float)longest : 0.f;
         r *= r; r *= r; r *= r;
-        wt[c] = (int)(256.f * r);
+        wt[c] = all_columns_count ? (len > 0 ? 256 : 0) : (int)(256.f * r);
     }
     __syncthreads();
     if (threadIdx.x >= 64) return;
@@ -264,6 +267,76 @@ __global__ __launch_bounds__(256) void tile_color_kernel(const int32_t* __restri
             ++next[color];
         }
     }
+}
+
+// Which column each thread of the walking kernel takes in each tile (plans with `colperm`).  A wavefront walks as many
+// slot rows as the longest of its 64 columns needs, so with thread t <-> column t every slice pays for its longest
+// column (about 1.5 slot rows per connection for ids drawn uniformly); here the tile's columns are sorted by the slots
+// they need (stable: equal columns stay in index order), cut into blocks of 64 about equally long columns, and the
+// blocks dealt to the wavefronts so that the wavefronts of a SIMD (wave, wave + 4, wave + 8, ...) have about the same
+// rows in total: longest block first, each to the SIMD with the least so far that still has a wavefront free.
+// One workgroup per tile, one thread per column (columns up to the workgroup size exist for this purpose: the ones
+// beyond the input's width have no connections).  Also stores the slot rows of each slice, as tile_count_kernel does
+// for plans without the permutation.  LDS: counts [2][threads], keys [threads].
+__global__ void tile_perm_kernel(const int32_t* __restrict__ idx, const unsigned short* __restrict__ rowpos, int L, int K,
+                                 int tile_labels, int col_lo, unsigned short* __restrict__ colperm, unsigned* __restrict__ slice_len) {
+    extern __shared__ __align__(16) unsigned perm_lds[];
+    unsigned* cnt = perm_lds;                  // [2][threads]: labels in even rows, labels in odd rows
+    const int t = blockIdx.x, nthreads = blockDim.x, nslices = nthreads >> 6;
+    unsigned* key = cnt + 2 * nthreads;        // [threads]
+    __shared__ unsigned short wave_of_block[16];
+    __shared__ unsigned slice_rows[16];
+    if (threadIdx.x < 16) slice_rows[threadIdx.x] = 0u;
+    cnt[threadIdx.x] = 0;
+    cnt[nthreads + threadIdx.x] = 0;
+    __syncthreads();
+    const int j0 = t * tile_labels;
+    const int nl = min(tile_labels, L - j0);
+    const int* src = idx + (size_t)j0 * K;
+    const int total = nl * K;
+    for (int e = threadIdx.x; e < total; e += nthreads) {
+        const unsigned c = (unsigned)(src[e] - col_lo);
+        if (c < (unsigned)nthreads) atomicAdd(&cnt[(rowpos[j0 + e / K] & 1u) * nthreads + c], 1u);
+    }
+    __syncthreads();
+    // (the slots a column needs depend by one on the lane it gets; the larger of the two)
+    const unsigned mine = 2u * max(cnt[threadIdx.x], cnt[nthreads + threadIdx.x]);
+    key[threadIdx.x] = mine;
+    __syncthreads();
+    // place among the columns in descending order of the key: columns with a larger key, and equal ones before this one
+    unsigned place = 0;
+    for (int c0 = 0; c0 < nthreads; c0 += 4) {
+        const uint4 k4 = *reinterpret_cast<const uint4*>(key + c0);       // (the same address in every lane: one broadcast read)
+        place += (k4.x > mine || (k4.x == mine && c0 + 0 < (int)threadIdx.x)) ? 1u : 0u;
+        place += (k4.y > mine || (k4.y == mine && c0 + 1 < (int)threadIdx.x)) ? 1u : 0u;
+        place += (k4.z > mine || (k4.z == mine && c0 + 2 < (int)threadIdx.x)) ? 1u : 0u;
+        place += (k4.w > mine || (k4.w == mine && c0 + 3 < (int)threadIdx.x)) ? 1u : 0u;
+    }
+    __syncthreads();
+    // key[] now by place: the first of each block of 64 is the block's longest column
+    key[place] = mine;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned sum[4] = {0u, 0u, 0u, 0u};
+        int used[4] = {0, 0, 0, 0};
+        for (int b = 0; b < nslices; ++b) {
+            int best = -1;
+            for (int q = 0; q < 4; ++q) {
+                if (q + 4 * used[q] >= nslices) continue;                 // no wavefront left on that SIMD
+                if (best < 0 || sum[q] < sum[best]) best = q;
+            }
+            wave_of_block[b] = (unsigned short)(best + 4 * used[best]);
+            sum[best] += (used[best] == 0 ? 3u : 1u) * key[b * 64];      // (a SIMD's longest wavefront ends up walking alone)
+            ++used[best];
+        }
+    }
+    __syncthreads();
+    const unsigned thread = wave_of_block[place >> 6] * 64u + (place & 63u);
+    colperm[(size_t)t * nthreads + thread] = (unsigned short)threadIdx.x;
+    // the slot rows of each slice: those of its longest column, now that every column knows its lane
+    atomicMax(&slice_rows[thread >> 6], column_slots(thread, cnt[threadIdx.x], cnt[nthreads + threadIdx.x]));
+    __syncthreads();
+    if ((int)threadIdx.x < nslices) slice_len[(size_t)t * nslices + threadIdx.x] = slice_rows[threadIdx.x];
 }
 
 // One workgroup per label tile, one thread per column.  Counts the tile's connections per column
@@ -326,7 +399,7 @@ constexpr int kFillChunk = 8192;
 __global__ void tile_fill_kernel(const int32_t* __restrict__ idx, const unsigned short* __restrict__ rowpos, int L, int K,
                                  int tile_labels, int zero_row, const unsigned* __restrict__ slice_off,
                                  unsigned short* __restrict__ lab16, unsigned short* __restrict__ pos16, unsigned pad_pos,
-                                 unsigned* __restrict__ slot32, int col_lo) {
+                                 unsigned* __restrict__ slot32, int col_lo, const unsigned short* __restrict__ colperm) {
     __shared__ __align__(16) int keys[kFillChunk];
     __shared__ unsigned short rows_of[kPlanTileLabels];     // LDS row of each label of the tile
     const int t = blockIdx.x, nthreads = blockDim.x;
@@ -334,7 +407,7 @@ __global__ void tile_fill_kernel(const int32_t* __restrict__ idx, const unsigned
     const int nl = min(tile_labels, L - j0);
     const int* src = idx + (size_t)j0 * K;
     const int total = nl * K;
-    const int mine = (int)threadIdx.x + col_lo;
+    const int mine = (colperm != nullptr ? (int)colperm[(size_t)blockIdx.x * blockDim.x + threadIdx.x] : (int)threadIdx.x) + col_lo;
     const size_t sl = (size_t)t * (nthreads >> 6) + (threadIdx.x >> 6);
     const size_t row0 = slice_off[sl];
     const unsigned rows = slice_off[sl + 1] - slice_off[sl];
@@ -382,7 +455,8 @@ __global__ void tile_fill_kernel(const int32_t* __restrict__ idx, const unsigned
 __global__ void tile_fill_bitmap_kernel(const int32_t* __restrict__ idx, const unsigned short* __restrict__ rowpos, int L, int K,
                                         int tile_labels, int zero_row, const unsigned* __restrict__ slice_off,
                                         unsigned short* __restrict__ lab16, unsigned short* __restrict__ pos16, unsigned pad_pos,
-                                        unsigned* __restrict__ slot32, int words, int col_lo) {
+                                        unsigned* __restrict__ slot32, int words, int col_lo,
+                                        const unsigned short* __restrict__ colperm) {
     extern __shared__ __align__(16) unsigned fill_lds[];
     const int t = blockIdx.x, nthreads = blockDim.x;
     unsigned* bm = fill_lds;                                                   // [nthreads][words] (words odd: no bank conflicts)
@@ -390,7 +464,11 @@ __global__ void tile_fill_bitmap_kernel(const int32_t* __restrict__ idx, const u
     unsigned short* pre = reinterpret_cast<unsigned short*>(pm + words);       // [nthreads][words + 1][2] labels before word w, even / odd rows
     unsigned short* rows_of = pre + (size_t)nthreads * (words + 1) * 2;        // [tile_labels]
     unsigned short* ids = rows_of + ((tile_labels + 1) & ~1);                  // [tile_labels * K]
+    unsigned short* thread_of = ids + (((size_t)tile_labels * K + 1) & ~(size_t)1);   // [nthreads] the thread that walks each column
     __shared__ unsigned duplicate;
+    // (bitmap and prefix counts are kept per column; slices, lanes and slot parities belong to threads)
+    const unsigned mycol = colperm != nullptr ? colperm[(size_t)blockIdx.x * blockDim.x + threadIdx.x] : threadIdx.x;
+    thread_of[mycol] = (unsigned short)threadIdx.x;
     const int j0 = t * tile_labels;
     const int nl = min(tile_labels, L - j0);
     const int* src = idx + (size_t)j0 * K;
@@ -426,7 +504,7 @@ __global__ void tile_fill_bitmap_kernel(const int32_t* __restrict__ idx, const u
         // (uniform) a label lists a column twice -- rewiring draws such labels all the time -- and the bitmap has one bit
         // for the two connections: here the column's thread walks its bitmap row in ascending label order and scans each
         // label found for the matching connections, which yields every connection, in ascending flat position
-        const unsigned mine = threadIdx.x;
+        const unsigned mine = mycol;
         const size_t sl = (size_t)t * nslices + (threadIdx.x >> 6);
         const size_t row0 = slice_off[sl];
         const unsigned rows = slice_off[sl + 1] - slice_off[sl];
@@ -461,7 +539,7 @@ __global__ void tile_fill_bitmap_kernel(const int32_t* __restrict__ idx, const u
     }
     // per column: labels in even / odd rows before each word; then the column's padding slots
     {
-        const unsigned mine = threadIdx.x;
+        const unsigned mine = mycol;
         const unsigned* my = bm + (size_t)mine * words;
         unsigned short* mp = pre + (size_t)mine * (words + 1) * 2;
         unsigned ev = 0, od = 0;
@@ -499,8 +577,9 @@ __global__ void tile_fill_bitmap_kernel(const int32_t* __restrict__ idx, const u
                 const unsigned o = pm[wd];
                 const unsigned same = bm[(size_t)c * words + wd] & (par ? o : ~o) & ((1u << (l & 31)) - 1u);
                 const unsigned rank = pre[((size_t)c * (words + 1) + wd) * 2 + par] + __builtin_popcount(same);
-                const unsigned slot = 2u * rank + (par ^ parity_first(c));
-                const size_t at = (size_t)slice_off[(size_t)t * nslices + (c >> 6)] * 64 + (c & 63u) + (size_t)slot * 64;
+                const unsigned thr = thread_of[c];
+                const unsigned slot = 2u * rank + (par ^ parity_first(thr));
+                const size_t at = (size_t)slice_off[(size_t)t * nslices + (thr >> 6)] * 64 + (thr & 63u) + (size_t)slot * 64;
                 if (slot32 != nullptr) slot32[at] = ((unsigned)e << 17) | (row << 7);
                 else { lab16[at] = (unsigned short)row; pos16[at] = (unsigned short)e; }
             }
@@ -517,7 +596,7 @@ inline size_t tile_fill_bitmap_lds(int threads, int tile_labels, int K, int* wor
     *words_out = words;
     return (size_t)threads * words * sizeof(unsigned) + (size_t)words * sizeof(unsigned) +
            (size_t)threads * (words + 1) * 2 * sizeof(unsigned short) + (size_t)((tile_labels + 1) & ~1) * sizeof(unsigned short) +
-           (size_t)tile_labels * K * sizeof(unsigned short);
+           (((size_t)tile_labels * K + 1) & ~(size_t)1) * sizeof(unsigned short) + (size_t)threads * sizeof(unsigned short);
 }
 
 // ---- blocked global form ------------------------------------------------------------------------
@@ -558,7 +637,7 @@ void free_arrays(ffi_plan* p, bool keep = false) {
     }
     p->owned.clear();
     p->rowpos = nullptr;
-    p->perm = nullptr; p->col_ptr = nullptr; p->slice_off = nullptr; p->lab16 = nullptr; p->pos16 = nullptr; p->slot32 = nullptr; p->idx16 = nullptr;
+    p->perm = nullptr; p->col_ptr = nullptr; p->slice_off = nullptr; p->lab16 = nullptr; p->pos16 = nullptr; p->slot32 = nullptr; p->idx16 = nullptr; p->colperm = nullptr;
     p->tiled = false; p->w_in_lds = false; p->total_rows = 0; p->bytes = 0;
 }
 
@@ -686,6 +765,15 @@ int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     const int slices = threads / 64;
     const int tiles = (p->L + TL - 1) / TL;
     const size_t nslices = (size_t)tiles * slices;
+    // (the walking kernel hands its sums from the tile's thread to the column's own thread through LDS: built for the
+    // weights-in-LDS form, whose workgroup has the registers for both sets of sums)
+    // Measured (input gradient, weights-in-LDS form, sorted against thread t <-> column t): 768 columns x fan-in 32, batch 128:
+    // 1.517 -> 1.150 slot rows per connection, 251 -> 239 us; batch 64: 151 -> 141; fan-in 16: 178 -> 170; fan-in 64 (300,000
+    // labels): 207 -> 190; 512 columns: 261 -> 251; 640 columns, batch 256: 226 -> 215; no gain at 256 columns and fewer (few
+    // slices to sort into, several workgroups per CU), and a loss where a workgroup walks a single tile (131,072 labels, batch
+    // 32: 35.4 -> 36.5 us): there the order of the columns stays.
+    const bool sorted_columns = plan_sorts_columns(threads, TL, p->K, w_in_lds, tiles, p->batch_hint);
+    p->colperm = nullptr;
     unsigned* slice_len = nullptr;
     if (!dev_alloc(p, &p->slice_off, nslices + 1) || !dev_alloc(p, &slice_len, nslices)) return FFI_ERR_OUT_OF_MEMORY;
     // rows per bank half: half the tile plus some room for the balancing, within the LDS the walking kernel can have
@@ -695,10 +783,17 @@ int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
         const size_t lds = 2 * ((size_t)threads + 1) * sizeof(int) + (size_t)TL * p->K * sizeof(unsigned short) + (size_t)TL;
         hipError_t ea = hipFuncSetAttribute((const void*)tile_color_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (ea != hipSuccess) return hip_fail(ea);
-        hipLaunchKernelGGL(tile_color_kernel, dim3(tiles), dim3(256), lds, s, lookup, p->L, p->K, TL, cap, threads, p->rowpos, p->col_lo);
+        hipLaunchKernelGGL(tile_color_kernel, dim3(tiles), dim3(256), lds, s, lookup, p->L, p->K, TL, cap, threads, p->rowpos, p->col_lo,
+                           sorted_columns ? 1 : 0);
     }
-    hipLaunchKernelGGL(tile_count_kernel, dim3(tiles), dim3(threads), 2 * threads * sizeof(unsigned), s, lookup, p->rowpos, p->L,
-                       p->K, TL, slice_len, p->col_lo);
+    if (sorted_columns) {
+        if (!dev_alloc(p, &p->colperm, (size_t)tiles * threads)) return FFI_ERR_OUT_OF_MEMORY;
+        hipLaunchKernelGGL(tile_perm_kernel, dim3(tiles), dim3(threads), 3 * threads * sizeof(unsigned), s, lookup, p->rowpos, p->L, p->K, TL,
+                           p->col_lo, p->colperm, slice_len);
+    } else {
+        hipLaunchKernelGGL(tile_count_kernel, dim3(tiles), dim3(threads), 2 * threads * sizeof(unsigned), s, lookup, p->rowpos, p->L,
+                           p->K, TL, slice_len, p->col_lo);
+    }
     hipLaunchKernelGGL(slice_scan_kernel, dim3(1), dim3(1024), 0, s, slice_len, p->slice_off, (int)nslices,
                        p->d_scratch + 2);
     hipError_t e = hipGetLastError();
@@ -725,10 +820,10 @@ int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
             hipError_t ea = hipFuncSetAttribute((const void*)tile_fill_bitmap_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)fill_lds);
             if (ea != hipSuccess) return hip_fail(ea);
             hipLaunchKernelGGL(tile_fill_bitmap_kernel, dim3(tiles), dim3(threads), fill_lds, s, lookup, p->rowpos, p->L, p->K, TL, 2 * cap,
-                               p->slice_off, p->lab16, p->pos16, pad_pos, p->slot32, words, p->col_lo);
+                               p->slice_off, p->lab16, p->pos16, pad_pos, p->slot32, words, p->col_lo, p->colperm);
         } else {
             hipLaunchKernelGGL(tile_fill_kernel, dim3(tiles), dim3(threads), 0, s, lookup, p->rowpos, p->L, p->K, TL, 2 * cap, p->slice_off,
-                               p->lab16, p->pos16, pad_pos, p->slot32, p->col_lo);
+                               p->lab16, p->pos16, pad_pos, p->slot32, p->col_lo, p->colperm);
         }
     }
     e = hipGetLastError();
@@ -738,7 +833,8 @@ int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     p->w_in_lds = w_in_lds;
     p->tile_labels = TL; p->threads = threads; p->slices = slices; p->tiles = tiles; p->zero_row = 2 * cap;
     p->total_rows = (long long)rows;
-    p->bytes += (size_t)rows * 64 * 2 * sizeof(unsigned short) + (nslices + 1) * sizeof(unsigned) + (size_t)p->L * sizeof(unsigned short);
+    p->bytes += (size_t)rows * 64 * 2 * sizeof(unsigned short) + (nslices + 1) * sizeof(unsigned) + (size_t)p->L * sizeof(unsigned short) +
+                (p->colperm ? (size_t)tiles * threads * sizeof(unsigned short) : 0);
     return FFI_OK;
 }
 
@@ -1079,9 +1175,9 @@ int plan_build_arrays(ffi_plan* p, const int32_t* lookup, hipStream_t s, unsigne
     }
     if (!p->tiled) {
         // (the tiled form's arrays, if any were made, go back to the spare list; the arranged ids stay)
-        for (void* q : {(void*)p->slice_off, (void*)p->rowpos, (void*)p->lab16, (void*)p->pos16, (void*)p->slot32})
+        for (void* q : {(void*)p->slice_off, (void*)p->rowpos, (void*)p->lab16, (void*)p->pos16, (void*)p->slot32, (void*)p->colperm})
             if (q) dev_release(p, q);
-        p->slice_off = nullptr; p->rowpos = nullptr; p->lab16 = nullptr; p->pos16 = nullptr; p->slot32 = nullptr;
+        p->slice_off = nullptr; p->rowpos = nullptr; p->lab16 = nullptr; p->pos16 = nullptr; p->slot32 = nullptr; p->colperm = nullptr;
         const size_t arranged_bytes = p->idx16 ? arranged_words((long long)p->L * ((p->K + 31) / 32)) * sizeof(unsigned short) : 0;
         p->bytes = 0;
         int st = build_global(p, lookup, s);

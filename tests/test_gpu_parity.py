@@ -207,7 +207,8 @@ def test_partly_filled_batch_tiles_write_nothing_behind_the_result(ffi, shape, t
 
 
 @pytest.mark.parametrize("option", [("wgrad_units", 3), ("wgrad_units", 4), ("wgrad_stream", -1), ("fwd_lane64", -1),
-                                    ("plan_weights_in_lds", -1), ("plan_weights_in_lds", 1), ("workgroups_per_cu", 1)])
+                                    ("plan_weights_in_lds", -1), ("plan_weights_in_lds", 1), ("workgroups_per_cu", 1),
+                                    ("plan_sorted_columns", -1), ("plan_sorted_columns", 1)])
 @pytest.mark.parametrize("shape", [(128, 512, 9000, 32), (64, 768, 5000, 16), (256, 256, 6000, 32)])
 def test_overridden_kernel_choices_keep_parity(ffi, option, shape):
     # every alternative a benchmark sweep can force computes the same layer
@@ -224,6 +225,66 @@ def test_overridden_kernel_choices_keep_parity(ffi, option, shape):
     assert rel_err(out, oracle.forward(x, lookup, w)) <= FWD_RTOL
     o_gx, o_gw = oracle.backward(x, lookup, w, g)
     assert rel_err(gw, o_gw) <= GRAD_RTOL and rel_err(gx, o_gx) <= GRAD_RTOL
+
+
+@pytest.mark.parametrize("shape", [(128, 768, 9000, 32),      # the headline's columns and fan-in: 16 tiles of twelve slices
+                                   (100, 700, 4000, 24),      # columns no multiple of 64: the last slice's spare threads take part in the sorting
+                                   (64, 512, 3000, 64),
+                                   (33, 100, 2500, 8),        # two slices, two batch tiles with one sample in the second
+                                   (96, 128, 12000, 16),      # several workgroups per CU
+                                   (32, 768, 40, 32),         # fewer labels than threads: the exchange of sums needs more LDS than the tile
+                                   (7, 64, 70000, 3),         # one slice: nothing to sort into, same results
+                                   (64, 1100, 3000, 12),      # two column windows, each with its own order per tile
+                                   (128, 768, 2000, 300)])    # tiles of a hundred labels
+@pytest.mark.parametrize("ids", ["uniform", "duplicates", "long_tail", "one_parity_per_half"])
+def test_plans_that_sort_a_tiles_columns_by_length(ffi, shape, ids):
+    # plans in the weights-in-LDS form may hand the columns to the walking kernel's threads anew in every tile, longest
+    # first; the library takes them where they pay (many labels), here they are forced on shapes the oracle finishes quickly
+    B, N, L, K = shape
+    x, lookup, w, g = reference_law_inputs(B, N, L, K, seed=N + L + K)
+    rng = np.random.default_rng(L)
+    if ids == "duplicates":                                   # every fourth label lists one of its columns twice
+        for j in range(0, L, 4):
+            a, b = rng.choice(K, 2, replace=False) if K > 1 else (0, 0)
+            lookup[j, a] = lookup[j, b]
+    elif ids == "long_tail":                                  # a few columns take most connections: not too skewed for the tiled form
+        lookup = np.where(rng.random((L, K)) < 0.3, rng.integers(0, max(1, N // 16), (L, K)), lookup).astype(np.int32)
+    elif ids == "one_parity_per_half":                        # see test_columns_fed_by_one_label_parity
+        half = max(1, N // 2)
+        lookup = (lookup % half + (np.arange(L)[:, None] % 2) * half).astype(np.int32) % N
+    lib = ffi._lib.lib()
+    print(f"case shape={shape} ids={ids}", flush=True)
+    results = {}
+    for value in (1, -1):
+        ffi._lib.check(lib.ffi_set_option(b"plan_weights_in_lds", 1))
+        ffi._lib.check(lib.ffi_set_option(b"plan_sorted_columns", value))
+        try:
+            dx, dl, dw, dg = dev(x), dev(lookup), dev(w), dev(g)
+            plan = ctypes.c_void_p()
+            ffi._lib.check(lib.ffi_plan_create(dl.data_ptr(), L, K, N, B, stream(), ctypes.byref(plan)))
+            info = (ctypes.c_int64 * 8)()
+            ffi._lib.check(lib.ffi_plan_info(plan, info))
+            runs = []
+            for _ in range(2):
+                gx = torch.full_like(dx, float("nan"))
+                ffi._lib.check(lib.ffi_input_grad_planned_f32(plan, dw.data_ptr(), dg.data_ptr(), gx.data_ptr(), B, 0, stream()))
+                torch.cuda.synchronize()
+                runs.append(gx.cpu().numpy())
+            ffi._lib.check(lib.ffi_plan_destroy(plan))
+            assert np.array_equal(runs[0], runs[1])           # reproducible bit for bit
+            results[value] = (runs[0], info[0], info[1], info[5])
+            # the stateless route, and an edit of the lookup in place behind it
+            got_gx, got_gw = hip_backward(ffi, x, lookup, w, g, False)
+            o_gx, o_gw = oracle.backward(x, lookup, w, g)
+            assert rel_err(got_gx, o_gx) <= GRAD_RTOL and rel_err(got_gw, o_gw) <= GRAD_RTOL
+        finally:
+            ffi._lib.check(lib.ffi_set_option(b"plan_sorted_columns", 0))
+            ffi._lib.check(lib.ffi_set_option(b"plan_weights_in_lds", 0))
+    o_gx = oracle.input_grad(x, lookup, w, g)
+    assert rel_err(results[1][0], o_gx) <= GRAD_RTOL and rel_err(results[-1][0], o_gx) <= GRAD_RTOL
+    if results[1][1] and results[1][2] and N > 64:
+        # tiled, weights in LDS: sorting never needs more slot rows than thread t <-> column t
+        assert results[1][3] <= results[-1][3]
 
 
 @pytest.mark.parametrize("shape", [(300, 700, 5000, 32), (33, 96, 9, 5), (128, 512, 4100, 100), (40, 1216, 2500, 36), (64, 1100, 3000, 12),
