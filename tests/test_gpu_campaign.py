@@ -36,10 +36,23 @@ def draw_lookup(rng, dist, L, K, N):
     return ids.astype(np.int32)
 
 
-@pytest.mark.parametrize("seed", [11, 12, 13, 14])
-def test_random_shapes_layouts_and_id_distributions(seed):
+@pytest.mark.parametrize("seed,options", [(11, ()), (12, ()), (13, ()), (14, ()),
+                                          # the plan forms the library takes only for large layers, forced onto small ones
+                                          (15, (("plan_weights_in_lds", 1), ("plan_sorted_columns", 1))),
+                                          (16, (("plan_weights_in_lds", -1), ("wgrad_stream", -1)))])
+def test_random_shapes_layouts_and_id_distributions(seed, options):
     ffi = load_package()
     lib = ffi._lib.lib()
+    for name, value in options:
+        ffi._lib.check(lib.ffi_set_option(name.encode(), value))
+    try:
+        _campaign(ffi, lib, seed)
+    finally:
+        for name, _ in options:
+            ffi._lib.check(lib.ffi_set_option(name.encode(), 0))
+
+
+def _campaign(ffi, lib, seed):
     rng = np.random.default_rng(seed)
     dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
     stream = lambda: torch.cuda.current_stream().cuda_stream
