@@ -467,7 +467,7 @@ SWEEP_GRIDS["layer_k64"] = dict(SWEEP_GRIDS["layer"], base=(256, 512, 501070, 64
 SWEEP_VARIANTS = {
     "forward": [("fwd_lane64", -1)],
     "weight_grad": [("wgrad_units", 3), ("wgrad_units", 4), ("wgrad_stream", -1)],
-    "input_grad": [("plan_weights_in_lds", -1), ("plan_weights_in_lds", 1), ("workgroups_per_cu", 1)],
+    "input_grad": [("plan_weights_in_lds", -1), ("plan_weights_in_lds", 1), ("workgroups_per_cu", 1), ("plan_sorted_columns", -1), ("plan_sorted_columns", 1)],
 }
 
 

@@ -200,6 +200,8 @@ int ffi_lookup_edited(const int32_t* lookup);
  *   "fwd_lane64"           -1: never the forward kernel that holds 64 samples per workgroup
  *   "plan_weights_in_lds"  -1: never / 1: whenever it fits: the input-gradient form that keeps a tile's weights in LDS
  *   "workgroups_per_cu"    n > 0: at most n workgroups per CU for the kernel that walks a tiled plan
+ *   "plan_sorted_columns"  -1: never / 1: whenever the weights-in-LDS form is taken: plans that hand a tile's columns to the
+ *                          walking kernel's threads sorted by length (fewer padded slots; the sums pass through LDS after every tile)
  * Drops the cached plans and workspaces of the current device first (as ffi_cache_clear, with its rule about calls in
  * flight).  Unknown names and values outside the ranges above return FFI_ERR_BAD_ARGUMENT and change nothing.
  */

@@ -69,8 +69,8 @@ def test_option_names_and_ranges_are_checked():
     assert lib.ffi_set_option(None, 0) == -8
     assert lib.ffi_set_option(b"no_such_option", 0) == -8
     assert lib.ffi_set_option(b"wgrad_units", 5) == -8 and lib.ffi_set_option(b"wgrad_units", 2) == -8
-    assert lib.ffi_set_option(b"fwd_lane64", 1) == -8
+    assert lib.ffi_set_option(b"fwd_lane64", 1) == -8 and lib.ffi_set_option(b"plan_sorted_columns", 2) == -8
     for name, value in ((b"wgrad_units", 3), (b"wgrad_stream", -1), (b"fwd_lane64", -1), (b"plan_weights_in_lds", 1),
-                        (b"workgroups_per_cu", 2)):
+                        (b"workgroups_per_cu", 2), (b"plan_sorted_columns", -1), (b"plan_sorted_columns", 1)):
         assert lib.ffi_set_option(name, value) == 0
         assert lib.ffi_set_option(name, 0) == 0
