@@ -696,9 +696,8 @@ int plan_tile_labels(int N, int K, int L, int batch_hint, bool* weights_in_lds) 
     // copy of the weights in memory).
     // Measured (gx pass, 0.2-0.67 M labels, fan-in 8...128, 64...1024 columns), against permutation + walk with the
     // tiles and workgroups per CU that suit each form (tiled_workgroups_per_cu): with up to four batch tiles the form is
-    // 5-60 % faster (most where the fan-in exceeds 32 or the layer has at most 256 columns); with five to eight batch
-    // tiles the tile's weights are staged that many times per tile: at fan-in 32 and below still -5...-30 % with at
-    // most 256 columns (several workgroups per CU overlap the staging) and -1...-8 % with 512 or 768; with 576 to 768
+    // 5-60 % faster (most where the fan-in exceeds 32); with five to eight batch
+    // tiles the tile's weights are staged that many times per tile: at fan-in 32 and below still -1...-8 % with 512 or 768 columns; with 576 to 768
     // columns -5...-13 % at every fan-in from 40 to 128 (one workgroup per CU either way); but +12 % at fan-in
     // 64 / 512 columns against the two-workgroup slot-ordered form, which also wins at 320-448 columns; with sixteen
     // batch tiles -7...+6 %: not taken.
@@ -707,9 +706,16 @@ int plan_tile_labels(int N, int K, int L, int batch_hint, bool* weights_in_lds) 
     // A slot's position inside the tile's weights has 15 bits (the zero word that padding slots read included).
     bool w_in_lds = false;
     const int nbt_hint = (batch_hint + 31) / 32;
-    const bool wanted = batch_hint > 0 && g_options.plan_weights_in_lds >= 0 &&
-                        (g_options.plan_weights_in_lds > 0 || nbt_hint <= 4 ||
-                         (nbt_hint <= 8 && (threads > 512 || (K <= 32 && (threads == 512 || threads <= 256)))));   // (unknown batch size: the form for large batches)
+    // Measured again once a tile's columns were sorted by length (which the form gets at 384 columns and more): 576 to 768
+    // columns at 12 and 16 batch tiles, fan-in 32 and 64: -2...-6 % against the slot-ordered form, so workgroups of more than
+    // 512 threads take the form at any batch size.  And at 256 columns and fewer, where several workgroups share a CU in
+    // either form (670,091 labels): fan-in 16 -9...-20 % up to eight batch tiles; fan-in 32 -15...-36 % at one and two
+    // batch tiles, equal at three, at four -21 % with 192 columns but +8 % with 256 (+16 % at fan-in 64), and +14...+30 %
+    // at five to eight batch tiles (128 and 256 columns): from fan-in 32 on the slot-ordered form takes over there.
+    const bool by_shape = threads > 512 ? true
+                        : threads <= 256 ? (K < 32 ? nbt_hint <= 8 : (nbt_hint <= 3 || (nbt_hint == 4 && threads < 256)))
+                                         : (nbt_hint <= 4 || (nbt_hint <= 8 && K <= 32 && threads == 512));
+    const bool wanted = batch_hint > 0 && g_options.plan_weights_in_lds >= 0 && (g_options.plan_weights_in_lds > 0 || by_shape);   // (unknown batch size: the form for large batches)
     if (wanted && threads <= 768) {
         int tw = std::min(TL, threads & ~1);
         // (workgroups of at most 256 threads share a CU when there are batch tiles to overlap: tiled_workgroups_per_cu)

@@ -152,7 +152,8 @@ PATH_SHAPES = [
     # several workgroups of the input-gradient kernel per CU (narrow layers):
     (300, 200, 9000, 16),      # ten batch tiles, weights in slot order: four workgroups of 256 threads
     (96, 128, 12000, 16),      # three batch tiles, weights in LDS: six workgroups of 128 threads, a share of the LDS each
-    (160, 256, 9000, 32),      # five batch tiles, weights in LDS: three workgroups of 256 threads
+    (160, 256, 9000, 16),      # five batch tiles, weights in LDS (fan-in below 32): three workgroups of 256 threads
+    (160, 256, 9000, 32),      # five batch tiles, weights in slot order: four workgroups of 256 threads
     (288, 64, 20000, 8),       # nine batch tiles, weights in slot order: sixteen workgroups of 64 threads
     # forward over batch tiles of 64 (N <= 608; from 192 samples, from 128 with a fan-in of 64 or more, fan-in 48 / 80 / 112):
     (256, 512, 5000, 64),      # whole tiles, vector loads
