@@ -765,7 +765,8 @@ def test_plan_layouts_serve_any_batch_size(ffi, shape):
 
 @pytest.mark.parametrize("shape", [(128, 768, 60_000, 32, True), (32, 768, 40_000, 32, True), (256, 512, 30_000, 64, True),
                                    (64, 300, 20_000, 12, False), (96, 2000, 5_000, 20, False), (40, 1100, 9_000, 16, True),
-                                   (160, 128, 40_000, 16, True), (300, 200, 40_000, 16, False)])    # (several input-gradient workgroups per CU)
+                                   (160, 128, 40_000, 16, True), (300, 200, 40_000, 16, False),     # (several input-gradient workgroups per CU)
+                                   (128, 768, 160_000, 32, True), (64, 1100, 200_000, 16, True)])   # (plans that sort a tile's columns by length; two column windows)
 def test_workspace_estimate_brackets_what_the_library_holds(ffi, shape):
     # ffi_workspace_bytes() is asked before anything is allocated; ffi_cache_bytes() says what forward + backward then
     # hold (plans + workspaces).  The estimate models the padding of the plan for uniformly drawn ids.
