@@ -129,10 +129,11 @@ def rewire_costs(pkg, cfg, x, lookup, w, g, tp, stream):
     thr = torch.empty(1, device="cuda")
     gen = torch.Generator(device="cuda").manual_seed(11)
 
-    def rewire():
+    def rewire(target=lookup2):
         check(lib.ffi_select_threshold_f32(ptr(w), L * K, (L * K) // 100, ptr(thr), sh))
-        check(lib.ffi_rewire_f32(ptr(lookup2), ptr(w), None, 0, L * K, N, ptr(thr), 12345, None, sh))
+        check(lib.ffi_rewire_f32(ptr(target), ptr(w), None, 0, L * K, N, ptr(thr), 12345, None, sh))
 
+    rewire(lookup.clone())                       # (untimed, on another copy: the selection's workspace is allocated once per process)
     rewire_ms = timed(rewire)
     first_library = timed(backward)
     after_library = timed(backward)
