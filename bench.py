@@ -187,7 +187,7 @@ def parse_args():
                     help="instead of the benchmark line: batch x width x labels x fan-in grids of the passes, one CSV line per "
                          "timing (file: --sweep-csv): 'reference' = the grid of the reference's testing/detailed-bench.cpp:26-112, "
                          "'layer' = the same axes around the headline workload, each pass also with the library's kernel choices overridden")
-    ap.add_argument("--sweep-csv", default=os.path.join("gpurun_out", "sweep.csv"), help="where --sweep writes its timings (relative to this file)")
+    ap.add_argument("--sweep-csv", default="sweep.csv", help="where --sweep writes its timings (relative to this file)")
     ap.add_argument("--copy-bytes", type=int, default=0,
                     help="also run one plain device copy kernel of this many bytes (read N, write N): the "
                          "known-size reference that rocprofv3 FETCH_SIZE/WRITE_SIZE readings are scaled by")
@@ -484,7 +484,7 @@ def sweep(args, pkg, synth):
     sh = stream.cuda_stream
     ptr = lambda a: a.data_ptr()  # noqa: E731
     path = os.path.join(ROOT, args.sweep_csv)
-    os.makedirs(os.path.dirname(path), exist_ok=True)
+    os.makedirs(os.path.dirname(path) or ".", exist_ok=True)
     rows, beaten, points = [], [], 0
     names = ("batch", "num_features", "num_units", "fan_in")
     grids = [g for g in SWEEP_GRIDS if args.sweep in ("all", g)]
