@@ -8,6 +8,7 @@
 
 #include <algorithm>
 #include <cstring>
+#include <functional>
 
 #include <rocprim/device/device_radix_sort.hpp>
 #include <rocprim/iterator/counting_iterator.hpp>
@@ -198,46 +199,68 @@ __global__ __launch_bounds__(256) void tile_color_kernel(const int32_t* __restri
     extern __shared__ int color_lds[];
     // (entry `ncols` of both: where connections into columns outside the window go -- weight 0, so they never count)
     int* imb = color_lds;                                                        // [ncols + 1] even minus odd labels per column
-    int* wt = color_lds + ncols + 1;                                             // [ncols + 1] weight of the column's balance
-    unsigned short* ids = reinterpret_cast<unsigned short*>(color_lds + 2 * (ncols + 1));  // [tile_labels * K] column ids
+    // The tile's column ids, three 10-bit ids per word, a label's ids in W = ceil(K / 3) words of its own, and the weights as
+    // 16-bit numbers: with 16-bit ids and 32-bit weights a tile of 582 labels x fan-in 32 took 44 KB of LDS, three workgroups per
+    // CU and two rounds for 1,152 tiles; now 31 KB, five workgroups per CU, all tiles at once (the work of a tile is one
+    // wavefront's sequential loop).
+    const int W = (K + 2) / 3;
+    unsigned* ids3 = reinterpret_cast<unsigned*>(color_lds + ncols + 1);         // [tile_labels * W]
+    unsigned short* wt = reinterpret_cast<unsigned short*>(ids3 + (size_t)tile_labels * W);   // [ncols + 1] weight of the column's balance (at most 256)
     const int t = blockIdx.x;
     const int j0 = t * tile_labels;
     const int nl = min(tile_labels, L - j0);
     const int* src = idx + (size_t)j0 * K;
+    const unsigned outside = (unsigned)min(ncols, 1023);                          // (windows are at most 640 columns wide; a single window has no ids outside)
     for (int i = threadIdx.x; i <= ncols; i += 256) { imb[i] = 0; wt[i] = 0; }
     __syncthreads();
-    for (int e = threadIdx.x; e < nl * K; e += 256) {
-        const unsigned c = (unsigned)(src[e] - col_lo);
-        const bool in = c < (unsigned)ncols;
-        ids[e] = in ? (unsigned short)c : (unsigned short)ncols;                // (ncols <= 1024)
-        if (in) atomicAdd(&wt[c], 1);                                            // column lengths first
+    for (int wi = threadIdx.x; wi < nl * W; wi += 256) {
+        const int jl = wi / W, k0 = 3 * (wi - jl * W);
+        unsigned word = 0;
+#pragma unroll
+        for (int i = 0; i < 3; ++i) {
+            unsigned c = outside;
+            if (k0 + i < K) {
+                const unsigned v = (unsigned)(src[jl * K + k0 + i] - col_lo);
+                if (v < (unsigned)ncols) { c = v; atomicAdd(&imb[v], 1); }       // column lengths first (in imb: the LDS adds whole words)
+            } else {
+                c = (unsigned)min(ncols, 1023);                                  // (behind the label's last id: never read)
+            }
+            word |= c << (10 * i);
+        }
+        ids3[wi] = word;
     }
     __syncthreads();
     // Only the longest columns of a slice (64 columns, one wavefront of the walking kernel) set its number of slot
     // rows, so their balance counts most: weight = 256 * (length / longest of the slice)^8.
     for (int c = threadIdx.x; c < ncols; c += 256) {
-        const int len = wt[c];
+        const int len = imb[c];
+        imb[c] = 0;
         int longest = len;
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) longest = max(longest, __shfl_xor(longest, off, 64));
         float r = longest > 0 ? (float)len / (float)longest : 0.f;
         r *= r; r *= r; r *= r;
-        wt[c] = all_columns_count ? (len > 0 ? 256 : 0) : (int)(256.f * r);
+        wt[c] = (unsigned short)(all_columns_count ? (len > 0 ? 256 : 0) : (int)(256.f * r));
     }
     __syncthreads();
     if (threadIdx.x >= 64) return;
     const int lane = threadIdx.x;
-    unsigned char* half = reinterpret_cast<unsigned char*>(ids + (size_t)tile_labels * K);   // [tile_labels] the half each label goes to
+    unsigned char* half = reinterpret_cast<unsigned char*>(wt + ncols + 2);      // [tile_labels] the half each label goes to
+    // column of connection k of label jl
+    auto id_of = [&](int jl, int k) {
+        const int q = (k * 43691) >> 17;                                         // k / 3 for k < 2^15
+        return (int)((ids3[jl * W + q] >> (10 * (k - 3 * q))) & 1023u);
+    };
     int placed[2] = {0, 0};
     for (int jl = 0; jl < nl; ++jl) {
         int sum = 0;
-        for (int k = lane; k < K; k += 64) { const int c = ids[jl * K + k]; sum += wt[c] * imb[c]; }
+        for (int k = lane; k < K; k += 64) { const int c = id_of(jl, k); sum += wt[c] * imb[c]; }
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
         int color = sum > 0 ? 1 : (sum < 0 ? 0 : (placed[1] < placed[0] ? 1 : 0));
         if (placed[color] >= cap) color ^= 1;
         const int delta = color ? -1 : 1;
-        for (int k = lane; k < K; k += 64) atomicAdd(&imb[ids[jl * K + k]], delta);   // a column may occur twice in a label
+        for (int k = lane; k < K; k += 64) atomicAdd(&imb[id_of(jl, k)], delta);   // a column may occur twice in a label
         if (lane == 0) half[jl] = (unsigned char)color;
         ++placed[color];
     }
@@ -247,15 +270,15 @@ __global__ __launch_bounds__(256) void tile_color_kernel(const int32_t* __restri
     for (int jl = 0; jl < nl; ++jl) {
         const int old = half[jl];                         // (written by lane 0 above; LDS accesses of a wavefront are in order)
         const int back = old ? 1 : -1;
-        for (int k = lane; k < K; k += 64) atomicAdd(&imb[ids[jl * K + k]], back);
+        for (int k = lane; k < K; k += 64) atomicAdd(&imb[id_of(jl, k)], back);
         int sum = 0;
-        for (int k = lane; k < K; k += 64) { const int c = ids[jl * K + k]; sum += wt[c] * imb[c]; }
+        for (int k = lane; k < K; k += 64) { const int c = id_of(jl, k); sum += wt[c] * imb[c]; }
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
         int color = sum > 0 ? 1 : (sum < 0 ? 0 : old);
         if (color != old && placed[color] >= cap) color = old;
         const int delta = color ? -1 : 1;
-        for (int k = lane; k < K; k += 64) atomicAdd(&imb[ids[jl * K + k]], delta);
+        for (int k = lane; k < K; k += 64) atomicAdd(&imb[id_of(jl, k)], delta);
         if (color != old) { --placed[old]; ++placed[color]; if (lane == 0) half[jl] = (unsigned char)color; }
     }
     // rows of a half are handed out in ascending label order
@@ -759,7 +782,10 @@ namespace {
 // Builds the tiled form.  Returns FFI_OK with p->tiled == false if the padded size would exceed
 // three times the connection count (heavily skewed column usage): the caller then builds the
 // global form instead.
-int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
+// (`after_row_assignment`, may be empty: called once the kernel that assigns the labels' LDS rows is enqueued -- it takes
+// nearly all of every CU's LDS for itself, and work for another stream enqueued behind it starts when it ends instead of
+// halving the number of its workgroups that fit)
+int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s, const std::function<int()>& after_row_assignment = {}) {
     const int cols = p->col_n ? p->col_n : p->N;           // the columns this plan's tiled form covers, from col_lo on
     const int threads = ((cols + 63) / 64) * 64;
     // every thread of the kernel that walks the plan stages at most two labels of a tile (one when
@@ -786,11 +812,15 @@ int build_tiled(ffi_plan* p, const int32_t* lookup, hipStream_t s) {
     const int cap = tiled_rows_per_half(TL);
     if (!dev_alloc(p, &p->rowpos, (size_t)p->L)) return FFI_ERR_OUT_OF_MEMORY;
     {
-        const size_t lds = 2 * ((size_t)threads + 1) * sizeof(int) + (size_t)TL * p->K * sizeof(unsigned short) + (size_t)TL;
+        const size_t lds = ((size_t)threads + 1) * sizeof(int) + (size_t)TL * ((p->K + 2) / 3) * sizeof(unsigned) + ((size_t)threads + 2) * sizeof(unsigned short) + (size_t)TL;
         hipError_t ea = hipFuncSetAttribute((const void*)tile_color_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (ea != hipSuccess) return hip_fail(ea);
         hipLaunchKernelGGL(tile_color_kernel, dim3(tiles), dim3(256), lds, s, lookup, p->L, p->K, TL, cap, threads, p->rowpos, p->col_lo,
                            sorted_columns ? 1 : 0);
+    }
+    if (after_row_assignment) {
+        const int st = after_row_assignment();
+        if (st != FFI_OK) return st;
     }
     if (sorted_columns) {
         if (!dev_alloc(p, &p->colperm, (size_t)tiles * threads)) return FFI_ERR_OUT_OF_MEMORY;
@@ -1128,18 +1158,17 @@ int plan_build_arrays(ffi_plan* p, const int32_t* lookup, hipStream_t s, unsigne
                 if (p->helper_stream) { (void)hipStreamDestroy(p->helper_stream); p->helper_stream = nullptr; }
             }
         }
-        hipStream_t hs = p->helper_stream ? p->helper_stream : s;
-        if (hs != s) {
-            // (the fingerprint above has synchronised `s`: the lookup is final, the helper needs no further ordering)
-            helper_busy = true;
-        }
-        int st = build_arranged(p, lookup, hs);
-        if (st != FFI_OK) {
-            if (helper_busy) (void)hipStreamSynchronize(hs);
-            free_arrays(p);
-            return st;
-        }
     }
+    // (enqueued from inside the tiled build, behind the row-assignment kernel, where there is a tiled build)
+    bool arranged_enqueued = !arranged;
+    auto enqueue_arranged = [&]() -> int {
+        if (arranged_enqueued) return FFI_OK;
+        arranged_enqueued = true;
+        hipStream_t hs = p->helper_stream ? p->helper_stream : s;
+        // (the fingerprint above has synchronised `s`: the lookup is final, the helper needs no further ordering)
+        if (hs != s) helper_busy = true;
+        return build_arranged(p, lookup, hs);
+    };
     auto join = [&]() -> int {
         if (helper_busy) { helper_busy = false; FFI_HIP_TRY(hipStreamSynchronize(p->helper_stream)); }
         return FFI_OK;
@@ -1147,7 +1176,7 @@ int plan_build_arrays(ffi_plan* p, const int32_t* lookup, hipStream_t s, unsigne
     // tiled form: one thread per column (N <= 1024), tiles of at least 62 labels with positions in 16 bits
     // (and 32 rows of out_grad within 32-bit byte offsets, as the kernels' buffer loads need)
     if (p->N <= 1024 && p->K <= 1024 && p->L < (1 << 25)) {
-        int st = build_tiled(p, lookup, s);
+        int st = build_tiled(p, lookup, s, enqueue_arranged);
         if (st != FFI_OK) { (void)join(); free_arrays(p); return st; }
     } else if (tile_path_fits(p->N) && p->N <= 2048 && p->K <= 1024 && p->L < (1 << 25)) {
         // 1,025 to 1,216 columns: the LDS tile of the other two passes holds them, a workgroup of one thread per column
@@ -1155,7 +1184,7 @@ int plan_build_arrays(ffi_plan* p, const int32_t* lookup, hipStream_t s, unsigne
         // far less than the cache-bound global form (measured at 1,216 columns, c2's other dimensions: 1.58 ms).
         const int lower = ((p->N + 1) / 2 + 63) / 64 * 64;
         p->col_lo = 0; p->col_n = lower;
-        int st = build_tiled(p, lookup, s);
+        int st = build_tiled(p, lookup, s, enqueue_arranged);
         if (st == FFI_OK && p->tiled) {
             ffi_plan* u = new (std::nothrow) ffi_plan();
             if (u == nullptr) st = FFI_ERR_OUT_OF_MEMORY;
@@ -1178,6 +1207,10 @@ int plan_build_arrays(ffi_plan* p, const int32_t* lookup, hipStream_t s, unsigne
             p->tiled = false;
             p->col_lo = 0; p->col_n = 0;
         }
+    }
+    {
+        const int st = enqueue_arranged();         // (no tiled build took place, or it ended before its row assignment)
+        if (st != FFI_OK) { (void)join(); free_arrays(p); return st; }
     }
     if (!p->tiled) {
         // (the tiled form's arrays, if any were made, go back to the spare list; the arranged ids stay)
