@@ -105,7 +105,7 @@ int ffi_forward_noalloc_f32(const float* features, const int32_t* lookup, const 
  * pointer and shape, so in-place edits of lookup (rewiring, sparse/custom_layer.py:32-43) must be picked up:
  *   - edits made through this library (ffi_rewire_f32, ffi_arrange_connections_f32) mark the cached view outdated
  *     on the host, and the next backward call rebuilds it before it enqueues anything (that call synchronises
- *     `stream` and takes the time of a plan build, about 3 ms at 670,091 x 32 connections; results stay
+ *     `stream` and takes the time of a plan build, about 2 ms at 670,091 x 32 connections; results stay
  *     bit-reproducible);
  *   - edits by foreign code are caught by a content fingerprint that a kernel re-checks on every call, on the
  *     device, without a host wait: every call enqueued before the host has seen the verdict -- the first call after
