@@ -550,11 +550,30 @@ __global__ void tile_fill_bitmap_kernel(const int32_t* __restrict__ idx, const u
                 const unsigned row = rows_of[l];
                 const unsigned par = row & 1u;
                 const unsigned short* lrow = ids + (size_t)l * K;
-                for (int k = 0; k < K; ++k) {
-                    if (lrow[k] == mine) {
-                        const unsigned t2 = par ? seen[1]++ : seen[0]++;
-                        put(2u * t2 + (par ^ first), row, l * (unsigned)K + (unsigned)k);
+                auto found = [&](int k) {
+                    const unsigned t2 = par ? seen[1]++ : seen[0]++;
+                    put(2u * t2 + (par ^ first), row, l * (unsigned)K + (unsigned)k);
+                };
+                if ((K & 7) == 0 && ((size_t)lrow & 3) == 0) {
+                    // eight ids per step, as four words whose halves are compared with the column at once: a half is
+                    // equal where (x ^ pattern) has a zero half (the classic "has a zero byte" test, for 16-bit lanes)
+                    const unsigned* lrow2 = reinterpret_cast<const unsigned*>(lrow);
+                    const unsigned pattern = mine * 0x00010001u;
+                    for (int k = 0; k < K; k += 8) {
+                        unsigned x[4];
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) x[i] = lrow2[(k >> 1) + i] ^ pattern;
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            if (((x[i] - 0x00010001u) & ~x[i] & 0x80008000u) != 0u) {
+                                if ((x[i] & 0xffffu) == 0u) found(k + 2 * i);
+                                if ((x[i] >> 16) == 0u) found(k + 2 * i + 1);
+                            }
+                        }
                     }
+                } else {
+                    for (int k = 0; k < K; ++k)
+                        if (lrow[k] == mine) found(k);
                 }
             }
         }
